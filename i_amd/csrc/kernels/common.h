@@ -1,0 +1,48 @@
+// Shared device-side definitions for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// log2 of the f32 literal 2.71828175f, the base the reference C backend uses
+// for unary pow (compiler/src/lower/exec_plan_to_module.rs:630-633):
+// powf(2.71828175f, x) == exp2(x * I_LOG2_E32).
+#define I_LOG2_E32 1.44269499718f
+
+#define WAVE 64
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Exchange a value between lane l and lane l^32.
+__device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+  return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+
+__device__ __forceinline__ u32x4 ldg128(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.
+// Map the linear workgroup id so that ids sharing an XCD walk consecutive
+// tiles of one `group` (e.g. one attention head, whose K/V then stay in that
+// XCD's L2).  `per_group` tiles per group; groups are padded to a multiple of 8.
+__device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_t& group, uint32_t& tile) {
+  uint32_t xcd = id & 7u;
+  uint32_t slot = id >> 3;
+  group = (slot / per_group) * 8u + xcd;
+  tile = slot % per_group;
+}

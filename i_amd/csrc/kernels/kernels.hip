@@ -1,0 +1,55 @@
+// Single translation unit for the gfx950 code object (i_kernels_gfx950.hsaco).
+// Every entry point is extern "C" so the host side can look it up by name with
+// hipModuleGetFunction; each takes one parameter block by value (params.h).
+#include "attention_bf16.h"
+#include "attention_f32.h"
+#include "gemm_nt_bf16.h"
+#include "row_softmax.h"
+
+#define ATTN_BF16(DPAD, BN, NW, OCC)                                                          \
+  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN(AttnParams p) { \
+    attn_fwd_bf16_body<DPAD, BN, NW>(p);                                                      \
+  }
+ATTN_BF16(64, 64, 4, 2)
+ATTN_BF16(128, 64, 4, 2)
+
+#define ATTN_F32(DPAD, BN, NW)                                                             \
+  extern "C" __global__ void __launch_bounds__(NW * 64) attn_fwd_f32_d##DPAD##_bn##BN(AttnParams p) { \
+    attn_fwd_f32_body<DPAD, BN, NW>(p);                                                    \
+  }
+ATTN_F32(32, 32, 4)
+ATTN_F32(64, 32, 4)
+ATTN_F32(128, 32, 4)
+
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64(GemmParams p) {
+  gemm_nt_bf16_body<128, 128, 64, 2, 2>(p);
+}
+
+#define SOFTMAX_WAVE(NV)                                                                          \
+  extern "C" __global__ void __launch_bounds__(256) row_softmax_wave_v##NV(SoftmaxParams p) {     \
+    row_softmax_wave_body<NV, true>(p);                                                           \
+  }                                                                                               \
+  extern "C" __global__ void __launch_bounds__(256) row_softmax_wave_s##NV(SoftmaxParams p) {     \
+    row_softmax_wave_body<NV, false>(p);                                                          \
+  }
+SOFTMAX_WAVE(1)
+SOFTMAX_WAVE(2)
+SOFTMAX_WAVE(4)
+SOFTMAX_WAVE(8)
+SOFTMAX_WAVE(16)
+SOFTMAX_WAVE(32)
+
+extern "C" __global__ void __launch_bounds__(1024) row_softmax_block(SoftmaxParams p) { row_softmax_block_body(p); }
+
+extern "C" __global__ void __launch_bounds__(256) convert_f32_to_bf16(ConvertParams p) {
+  const float* s = reinterpret_cast<const float*>(p.src);
+  bf16_t* d = reinterpret_cast<bf16_t*>(p.dst);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < p.n; i += (uint64_t)gridDim.x * blockDim.x)
+    d[i] = (bf16_t)s[i];
+}
+extern "C" __global__ void __launch_bounds__(256) convert_bf16_to_f32(ConvertParams p) {
+  const bf16_t* s = reinterpret_cast<const bf16_t*>(p.src);
+  float* d = reinterpret_cast<float*>(p.dst);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < p.n; i += (uint64_t)gridDim.x * blockDim.x)
+    d[i] = (float)s[i];
+}

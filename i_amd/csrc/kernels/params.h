@@ -1,0 +1,37 @@
+// Kernel argument blocks shared by the device code and the host launcher.
+// Each kernel takes exactly one of these by value.
+#pragma once
+#include <stdint.h>
+
+enum { I_DT_F32 = 0, I_DT_BF16 = 1 };
+
+struct AttnParams {
+  const void* q;   // [bh, nq, d]
+  const void* k;   // [bh, nk, d]
+  const void* v;   // [bh, nk, dv]
+  void* o;         // [bh, nq, dv]
+  uint32_t bh, nq, nk, d, dv;
+  uint32_t nqt;        // query tiles per head
+  uint32_t out_bf16;   // 0: f32 output, 1: bf16 output
+  float scale_log2;    // score scale * log2(2.71828175f); scale > 0
+};
+
+struct GemmParams {
+  const void* a;   // [bh, m, k]
+  const void* b;   // [bh, n, k]
+  void* c;         // [bh, m, n]  f32
+  uint32_t bh, m, n, k;
+  uint32_t tiles_m, tiles_n;
+};
+
+struct SoftmaxParams {
+  const float* x;
+  float* y;
+  uint32_t rows, cols;
+};
+
+struct ConvertParams {
+  const void* src;
+  void* dst;
+  uint64_t n;
+};

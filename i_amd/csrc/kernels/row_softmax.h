@@ -1,0 +1,87 @@
+// Row softmax  y[i,:] = exp(x[i,:] - max_i) / sum_j exp(x[i,j] - max_i)  in f32.
+//
+// Device form of  row_max_shift >> exp >> row_normalize  (README.md:19-25).
+// The reference's valid schedules materialise the shifted / exponentiated row
+// (three kernels, ilang-python/flash-attn.py:60-62); here the row lives in
+// registers, so HBM sees exactly one read and one write per element.
+// One wavefront owns one row; reductions use cross-lane shuffles only.
+#pragma once
+#include "common.h"
+#include "params.h"
+
+// NV = float4 chunks per lane; covers cols <= 256 * NV.  VEC: cols % 4 == 0.
+template <int NV, bool VEC>
+__device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
+  const int lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= p.rows) return;
+  const float* __restrict__ x = p.x + (size_t)row * p.cols;
+  float* __restrict__ y = p.y + (size_t)row * p.cols;
+
+  f32x4 r[NV];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < NV; ++t) {
+    const uint32_t col = 4u * (lane + 64 * t);
+    if (VEC) {
+      if (col < p.cols) r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
+      else r[t] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : -INFINITY;
+    }
+    mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
+  }
+  mx = wave_max(mx);
+  const float mb = mx * I_LOG2_E32;
+  float sum = 0.0f;
+#pragma unroll
+  for (int t = 0; t < NV; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v = fast_exp2(__builtin_fmaf(r[t][e], I_LOG2_E32, -mb));
+      r[t][e] = v;
+      sum += v;
+    }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int t = 0; t < NV; ++t) {
+    const uint32_t col = 4u * (lane + 64 * t);
+    if (VEC) {
+      if (col < p.cols) __builtin_nontemporal_store(r[t] * inv, reinterpret_cast<f32x4*>(y + col));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (col + e < p.cols) y[col + e] = r[t][e] * inv;
+    }
+  }
+}
+
+// Any width: one workgroup per row, three passes over the row (max, sum, write).
+__device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
+  __shared__ float red[16];
+  const uint32_t row = blockIdx.x;
+  const float* __restrict__ x = p.x + (size_t)row * p.cols;
+  float* __restrict__ y = p.y + (size_t)row * p.cols;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  float mx = -INFINITY;
+  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) mx = fmaxf(mx, x[j]);
+  mx = wave_max(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = red[0];
+  for (int w = 1; w < nw; ++w) mx = fmaxf(mx, red[w]);
+  __syncthreads();
+  const float mb = mx * I_LOG2_E32;
+  float sum = 0.0f;
+  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) sum += fast_exp2(__builtin_fmaf(x[j], I_LOG2_E32, -mb));
+  sum = wave_sum(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  sum = 0.0f;
+  for (int w = 0; w < nw; ++w) sum += red[w];
+  const float inv = 1.0f / sum;
+  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x)
+    y[j] = fast_exp2(__builtin_fmaf(x[j], I_LOG2_E32, -mb)) * inv;
+}

@@ -1,0 +1,119 @@
+#include "hip_rt.h"
+
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <map>
+#include <mutex>
+#include <sstream>
+#include <vector>
+
+namespace ihip {
+
+Err check(hipError_t e, const char* what) {
+  if (e == hipSuccess) return {};
+  std::ostringstream os;
+  os << what << " failed: " << hipGetErrorString(e) << " (hip error " << (int)e << ")";
+  return os.str();
+}
+
+namespace {
+
+struct DeviceModule {
+  hipModule_t mod = nullptr;
+  std::map<std::string, hipFunction_t> fns;
+};
+
+std::mutex g_mu;
+std::map<int, DeviceModule> g_builtin;  // keyed by device ordinal
+std::vector<char> g_image;
+
+std::string code_object_path() {
+  if (const char* env = std::getenv("ILANG_HIP_KERNELS")) return env;
+  Dl_info info;
+  if (dladdr(reinterpret_cast<void*>(&code_object_path), &info) && info.dli_fname) {
+    std::string so = info.dli_fname;
+    auto slash = so.find_last_of('/');
+    std::string dir = slash == std::string::npos ? "." : so.substr(0, slash);
+    return dir + "/i_kernels_gfx950.hsaco";
+  }
+  return "i_kernels_gfx950.hsaco";
+}
+
+Err read_image() {
+  if (!g_image.empty()) return {};
+  const std::string path = code_object_path();
+  std::ifstream f(path, std::ios::binary);
+  if (!f) return "cannot open gfx950 code object '" + path + "' (build it with hipcc --genco, or set ILANG_HIP_KERNELS)";
+  g_image.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+  if (g_image.empty()) return "gfx950 code object '" + path + "' is empty";
+  return {};
+}
+
+}  // namespace
+
+Err builtin_function(const char* name, hipFunction_t* fn) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  int dev = 0;
+  if (Err e = check(hipGetDevice(&dev), "hipGetDevice"); !e.empty()) return e;
+  DeviceModule& dm = g_builtin[dev];
+  if (!dm.mod) {
+    if (Err e = read_image(); !e.empty()) return e;
+    if (Err e = check(hipModuleLoadData(&dm.mod, g_image.data()), "hipModuleLoadData"); !e.empty()) {
+      dm.mod = nullptr;
+      return e;
+    }
+  }
+  auto it = dm.fns.find(name);
+  if (it == dm.fns.end()) {
+    hipFunction_t f = nullptr;
+    if (Err e = check(hipModuleGetFunction(&f, dm.mod, name), "hipModuleGetFunction"); !e.empty())
+      return e + " [" + name + "]";
+    it = dm.fns.emplace(name, f).first;
+  }
+  *fn = it->second;
+  return {};
+}
+
+Err load_module(const void* image, hipModule_t* mod) { return check(hipModuleLoadData(mod, image), "hipModuleLoadData"); }
+
+Err module_function(hipModule_t mod, const char* name, hipFunction_t* fn) {
+  Err e = check(hipModuleGetFunction(fn, mod, name), "hipModuleGetFunction");
+  if (!e.empty()) e += std::string(" [") + name + "]";
+  return e;
+}
+
+void unload_module(hipModule_t mod) {
+  if (mod) (void)hipModuleUnload(mod);
+}
+
+Err launch(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, const void* params,
+           size_t params_size, hipStream_t stream) {
+  if (gx == 0 || gy == 0 || gz == 0) return {};
+  size_t size = params_size;
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(params), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                    HIP_LAUNCH_PARAM_END};
+  return check(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, 0, stream, nullptr, config), "hipModuleLaunchKernel");
+}
+
+Err dev_alloc(void** p, size_t bytes) {
+  *p = nullptr;
+  if (bytes == 0) bytes = 4;
+  return check(hipMalloc(p, bytes), "hipMalloc");
+}
+void dev_free(void* p) {
+  if (p) (void)hipFree(p);
+}
+Err h2d(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return {};
+  return check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream), "hipMemcpy H2D");
+}
+Err d2h(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return {};
+  return check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream), "hipMemcpy D2H");
+}
+Err sync(hipStream_t stream) { return check(hipStreamSynchronize(stream), "hipStreamSynchronize"); }
+
+}  // namespace ihip

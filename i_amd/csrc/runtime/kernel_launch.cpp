@@ -1,0 +1,108 @@
+#include "kernel_launch.h"
+
+#include <cmath>
+#include <cstdint>
+#include <string>
+
+#include "../kernels/params.h"
+
+namespace ihip {
+namespace {
+constexpr float kLog2E32 = 1.44269499718f;  // log2(2.71828175f)
+constexpr size_t kMaxGrid = 0x7fffffffu;
+
+bool fits_u32(size_t v) { return v <= 0xffffffffull; }
+}  // namespace
+
+bool attention_supported(DType in_dtype, size_t d, size_t dv, float scale) {
+  if (!(scale > 0.0f) || !std::isfinite(scale)) return false;
+  if (d == 0 || dv == 0 || d > 128 || dv > 128) return false;
+  if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
+  return true;
+}
+
+Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
+                     size_t nq, size_t nk, size_t d, size_t dv, float scale, hipStream_t stream) {
+  if (!attention_supported(in_dtype, d, dv, scale))
+    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, scale > 0; bf16 needs d, dv % 8 == 0)";
+  if (in_dtype == F32 && out_dtype != F32) return "attention kernel: f32 inputs produce f32 output";
+  if (bh == 0 || nq == 0) return {};
+  if (nk == 0) return "attention kernel: no keys";
+  if (!fits_u32(bh) || !fits_u32(nq) || !fits_u32(nk)) return "attention kernel: extent exceeds 32 bits";
+  if (!q || !k || !v || !o) return "attention kernel: null device pointer";
+
+  const size_t dmax = d > dv ? d : dv;
+  const unsigned bm = 128;
+  AttnParams p{};
+  p.q = q; p.k = k; p.v = v; p.o = o;
+  p.bh = (uint32_t)bh; p.nq = (uint32_t)nq; p.nk = (uint32_t)nk; p.d = (uint32_t)d; p.dv = (uint32_t)dv;
+  p.nqt = (uint32_t)((nq + bm - 1) / bm);
+  p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
+  p.scale_log2 = scale * kLog2E32;
+
+  const char* name;
+  if (in_dtype == BF16) name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
+  else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
+
+  const size_t groups = (bh + 7) / 8 * 8;  // heads padded to the XCD count
+  const size_t grid = groups * p.nqt;
+  if (grid > kMaxGrid) return "attention kernel: grid too large";
+  hipFunction_t fn;
+  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+}
+
+bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }
+
+Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream) {
+  if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
+  if (bh == 0 || m == 0 || n == 0) return {};
+  if (!fits_u32(m) || !fits_u32(n) || !fits_u32(k) || !fits_u32(bh)) return "gemm_nt kernel: extent exceeds 32 bits";
+  if (!a || !b || !c) return "gemm_nt kernel: null device pointer";
+  GemmParams p{};
+  p.a = a; p.b = b; p.c = c;
+  p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.tiles_m = (uint32_t)((m + 127) / 128);
+  p.tiles_n = (uint32_t)((n + 127) / 128);
+  const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
+  const size_t grid = ((tiles + 7) / 8 * 8) * bh;
+  if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
+  hipFunction_t fn;
+  if (Err e = builtin_function("gemm_nt_bf16_128x128x64", &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+}
+
+Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream) {
+  if (rows == 0 || cols == 0) return {};
+  if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
+  if (!x || !y) return "row_softmax kernel: null device pointer";
+  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols};
+  hipFunction_t fn;
+  if (cols <= 8192) {
+    int nv = 1;
+    while ((size_t)256 * nv < cols) nv *= 2;
+    const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+    const std::string name = std::string("row_softmax_wave_") + (vec ? "v" : "s") + std::to_string(nv);
+    if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
+    const size_t grid = (rows + 3) / 4;  // four wavefronts (rows) per workgroup
+    if (grid > kMaxGrid) return "row_softmax kernel: grid too large";
+    return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+  }
+  if (rows > kMaxGrid) return "row_softmax kernel: grid too large";
+  if (Err e = builtin_function("row_softmax_block", &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
+}
+
+Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, hipStream_t stream) {
+  if (n == 0) return {};
+  if (from == to) return "convert kernel: identical dtypes";
+  ConvertParams p{src, dst, (uint64_t)n};
+  hipFunction_t fn;
+  if (Err e = builtin_function(from == F32 ? "convert_f32_to_bf16" : "convert_bf16_to_f32", &fn); !e.empty()) return e;
+  size_t grid = (n + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+}
+
+}  // namespace ihip

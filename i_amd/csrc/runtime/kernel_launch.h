@@ -1,0 +1,29 @@
+// Host-side launchers for the hand-written gfx950 kernels.  They validate the
+// operand shapes against what each kernel and its grid assume, pick the
+// kernel variant, and enqueue it on `stream`.  All pointers are device memory.
+#pragma once
+#include <cstddef>
+
+#include "hip_rt.h"
+
+namespace ihip {
+
+enum DType { F32 = 0, BF16 = 1 };
+
+// o[bh,nq,dv] = softmax(scale * q[bh,nq,d] k[bh,nk,d]^T) v[bh,nk,dv]
+// in_dtype applies to q, k, v; out_dtype to o (F32 or BF16; BF16 only with bf16 inputs).
+Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
+                     size_t nq, size_t nk, size_t d, size_t dv, float scale, hipStream_t stream);
+bool attention_supported(DType in_dtype, size_t d, size_t dv, float scale);
+
+// c[bh,m,n] (f32) = a[bh,m,k] b[bh,n,k]^T, a and b bf16
+Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream);
+bool gemm_nt_bf16_supported(size_t k);
+
+// y[rows,cols] = row softmax of x, f32
+Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream);
+
+Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, hipStream_t stream);
+
+}  // namespace ihip

@@ -1,0 +1,60 @@
+/*
+ * Device-side additions of the gfx950 backend to the 𝚒 runtime ABI (i.h).
+ *
+ * The reference runtime only knows host f32 buffers (core/i.h:8-30) and its
+ * generated libraries export their kernels as plain functions
+ * `void fK(const View* readonlys, ViewMut* writeables)`
+ * (compiler/src/backends/c/stmt.rs:36-41).  The entry points below are the
+ * GPU counterparts of those two things and do not change any i.h signature:
+ *
+ *   i_hip_*  kernel launchers: the hand-written kernels a compiled program
+ *            dispatches to, callable directly on device memory (the `fK`
+ *            level of the generated-library ABI, ABI.md:4-9).
+ *
+ * All pointers are device pointers unless stated; `stream` is a hipStream_t
+ * (NULL = the default stream).  Launches are asynchronous on that stream.
+ * Return value 0 = enqueued, -1 = failure with the text in i_error().
+ */
+#pragma once
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { I_DTYPE_F32 = 0, I_DTYPE_BF16 = 1 };
+
+/*
+ * FlashAttention forward,  o = softmax(scale * q k^T) v  per (batch*head):
+ * the fused kernel for  mm_t >> [scale] >> row_max_shift >> exp >> row_normalize >> mm
+ * (reference emission of the same component: ilang-python/annotated-flashattn.c:52-310,
+ * `f0`).  q [bh,nq,d], k [bh,nk,d], v [bh,nk,dv], o [bh,nq,dv], row-major.
+ * in_dtype applies to q/k/v, out_dtype to o.  Requires 0 < d,dv <= 128, scale > 0,
+ * and d,dv multiples of 8 for bf16.
+ */
+int i_hip_attention(const void* q, const void* k, const void* v, void* o,
+                    int in_dtype, int out_dtype,
+                    size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
+                    float scale, void* stream);
+
+/*
+ * mm_t,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,n,k]  with bf16 a, b and f32 c:
+ * the fused kernel for  i("ik*jk~ijk") >> i("+ijk~ij ... k0")  (README.md:16;
+ * same nest as annotated-flashattn.c:57-89).  Requires k % 8 == 0.
+ */
+int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c,
+                       size_t bh, size_t m, size_t n, size_t k, void* stream);
+
+/*
+ * Row softmax over the last axis of an f32 [rows, cols] matrix: the fused
+ * kernel for  row_max_shift >> exp >> row_normalize  (README.md:19-25).
+ */
+int i_hip_row_softmax(const float* x, float* y, size_t rows, size_t cols, void* stream);
+
+/* Element-wise dtype conversion between f32 and bf16 device buffers (n elements). */
+int i_hip_convert(const void* src, void* dst, int from_dtype, int to_dtype, size_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
