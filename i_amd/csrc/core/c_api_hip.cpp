@@ -34,6 +34,5 @@ int i_hip_convert(const void* src, void* dst, int from_dtype, int to_dtype, size
   return finish(ihip::launch_convert(src, dst, (ihip::DType)from_dtype, (ihip::DType)to_dtype, n, (hipStream_t)stream));
 }
 
-const char* i_error(void) { return icore::last_error(); }
 
 }  // extern "C"

@@ -1,0 +1,224 @@
+"""Parity of the hand-written gfx950 kernels (called through the C ABI of
+include/i_hip.h) against the CPU oracle on identical seeded inputs.
+
+Tolerances (relative to max|oracle|): 1e-4 for f32 paths, 2e-2 for bf16 inputs
+with f32 accumulation.
+"""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+RTOL_F32 = 1e-4
+RTOL_BF16 = 2e-2
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+
+    assert torch.cuda.is_available(), "GPU tests need a visible MI355X"
+    from i_amd import _native as nat
+
+    class Env:
+        pass
+
+    e = Env()
+    e.torch, e.nat = torch, nat
+    e.stream = lambda: torch.cuda.current_stream().cuda_stream
+    return e
+
+
+def rnd(shape, seed, kind="normal"):
+    rng = np.random.default_rng(seed)
+    if kind == "uniform":
+        return rng.uniform(-1, 1, shape).astype(np.float32)
+    return rng.standard_normal(shape, dtype=np.float32)
+
+
+def relerr(got, ref):
+    return float(np.abs(got - ref).max() / np.abs(ref).max())
+
+
+def assert_close(got, ref, rtol):
+    assert got.shape == ref.shape
+    assert np.isfinite(got).all()
+    err = relerr(got, ref)
+    assert err <= rtol, f"relative error {err} > {rtol}"
+    assert np.allclose(got, ref, rtol=rtol, atol=rtol * np.abs(ref).max())
+
+
+def gpu_attention(env, q, k, v, scale, bf16, out_bf16=False):
+    t = env.torch
+    lead = q.shape[:-2]
+    bh = int(np.prod(lead)) if lead else 1
+    nq, d = q.shape[-2:]
+    nk, dv = v.shape[-2:]
+    dt = t.bfloat16 if bf16 else t.float32
+    qd, kd, vd = (t.from_numpy(a).cuda().to(dt).contiguous() for a in (q, k, v))
+    od = t.full(lead + (nq, dv), float("nan"), device="cuda", dtype=t.bfloat16 if out_bf16 else t.float32)
+    env.nat.check(env.nat.core.i_hip_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), od.data_ptr(),
+                                               env.nat.BF16 if bf16 else env.nat.F32,
+                                               env.nat.BF16 if out_bf16 else env.nat.F32,
+                                               bh, nq, nk, d, dv, 1.0 if scale is None else scale, env.stream()))
+    t.cuda.synchronize()
+    return od.float().cpu().numpy()
+
+
+# ------------------------------------------------------------------ attention, f32
+@pytest.mark.parametrize("case", ["u_48x24", "u_64x64", "u_100x40", "n_48x24", "n_33x17"])
+def test_attention_f32_vs_reference_golden(env, golden, case):
+    q, k, v, o = (golden[f"{case}.{x}"] for x in "qkvo")
+    assert_close(gpu_attention(env, q, k, v, None, bf16=False), o, RTOL_F32)
+
+
+@pytest.mark.parametrize("shape,kind", [((512, 64), "uniform"), ((500, 60), "uniform"), ((1, 1), "normal"),
+                                        ((2, 3, 4, 8), "normal"), ((6, 100, 40), "normal"), ((2, 130, 128), "normal")])
+def test_attention_f32_vs_oracle(env, shape, kind):
+    q, k, v = (rnd(shape, s, kind) for s in (1, 2, 3))
+    assert_close(gpu_attention(env, q, k, v, None, bf16=False), oracle.attention_tiled(q, k, v), RTOL_F32)
+
+
+def test_attention_f32_ragged_nq_nk_dv_and_scale(env):
+    q, k, v = rnd((3, 77, 24), 1), rnd((3, 130, 24), 2), rnd((3, 130, 40), 3)
+    assert_close(gpu_attention(env, q, k, v, 0.2, bf16=False), oracle.attention_tiled(q, k, v, 0.2), RTOL_F32)
+
+
+def test_attention_f32_online_rescale_stress(env):
+    nq, nk, d = 40, 300, 8
+    q = np.ones((nq, d), np.float32)
+    k = (np.arange(nk, dtype=np.float32)[:, None] * np.ones((1, d), np.float32)) * 0.25
+    v = rnd((nk, d), 3)
+    assert_close(gpu_attention(env, q, k, v, None, bf16=False), oracle.attention_tiled(q, k, v), RTOL_F32)
+
+
+# ------------------------------------------------------------------ attention, bf16 in / f32 accumulate
+@pytest.mark.parametrize("bh,nq,nk,d", [(1, 64, 64, 64), (2, 128, 128, 128), (3, 200, 333, 128), (2, 77, 130, 64),
+                                        (1, 512, 512, 64), (2, 100, 100, 40), (1, 1, 1, 8)])
+def test_attention_bf16_vs_oracle(env, bh, nq, nk, d):
+    q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    ref = oracle.attention_tiled(q, k, v, scale)
+    assert_close(gpu_attention(env, q, k, v, scale, bf16=True), ref, RTOL_BF16)
+    assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
+
+
+def test_attention_bf16_config4_slice_vs_oracle(env):
+    """One (b, h) slice of B8 H32 N4096 d128 at full sequence length, against the oracle on 256 query rows."""
+    n, d = 4096, 128
+    q, k, v = (oracle.to_bf16_f32(rnd((1, n, d), s)) for s in (1, 2, 3))
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    got = gpu_attention(env, q, k, v, scale, bf16=True)
+    rows = np.r_[0:128, n - 128:n]
+    ref = oracle.attention_tiled(q[:, rows], k, v, scale)
+    assert_close(got[:, rows], ref, RTOL_BF16)
+
+
+def test_attention_bf16_long_sequence_rescale_stress(env):
+    """Config 5 recipe (inputs x2.0, d=64) at N=8192: heavy running-max movement."""
+    n, d = 8192, 64
+    q, k, v = (oracle.to_bf16_f32(rnd((1, n, d), s) * 2.0) for s in (1, 2, 3))
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    got = gpu_attention(env, q, k, v, scale, bf16=True)
+    rows = np.r_[0:64, n - 64:n]
+    ref = oracle.attention_tiled(q[:, rows], k, v, scale)
+    assert_close(got[:, rows], ref, RTOL_BF16)
+
+
+def test_attention_full_size_properties(env):
+    """Size-independent properties at B8 H32 N4096 d128: rows are convex combinations of V
+    (constant V column -> constant output), and identical heads give identical outputs."""
+    t = env.torch
+    bh, n, d = 256, 4096, 128
+    g = t.Generator(device="cuda").manual_seed(1)
+    q = t.randn(bh, n, d, device="cuda", generator=g).bfloat16()
+    k = t.randn(bh, n, d, device="cuda", generator=g).bfloat16()
+    v = t.randn(bh, n, d, device="cuda", generator=g).bfloat16()
+    v[:, :, 0] = 1.5
+    q[7], k[7], v[7] = q[200], k[200], v[200]
+    o = t.empty(bh, n, d, device="cuda", dtype=t.float32)
+    env.nat.check(env.nat.core.i_hip_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), 1, 0,
+                                               bh, n, n, d, d, d ** -0.5, env.stream()))
+    t.cuda.synchronize()
+    assert t.isfinite(o).all()
+    assert (o[:, :, 0] - 1.5).abs().max().item() < 2e-2
+    assert t.equal(o[7], o[200])
+    vmax = v.float().amax(dim=1, keepdim=True)
+    vmin = v.float().amin(dim=1, keepdim=True)
+    assert (o <= vmax + 1e-3).all() and (o >= vmin - 1e-3).all()
+
+
+def test_attention_rejects_unsupported(env):
+    t = env.torch
+    x = t.zeros(1, 8, 256, device="cuda")
+    rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 0, 0, 1, 8, 8, 256, 256,
+                                      1.0, env.stream())
+    assert rc == -1 and "unsupported" in env.nat.last_error()
+    rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 0, 0, 1, 8, 8, 64, 64,
+                                      -1.0, env.stream())
+    assert rc == -1
+
+
+# ------------------------------------------------------------------ mm_t
+@pytest.mark.parametrize("bh,m,n,k", [(1, 128, 128, 64), (1, 100, 70, 40), (2, 300, 260, 136), (1, 1, 1, 8),
+                                      (1, 512, 384, 1024)])
+def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
+    t = env.torch
+    a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
+    ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+    cd = t.full((bh, m, n), float("nan"), device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nt_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+    t.cuda.synchronize()
+    assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
+
+
+def test_gemm_nt_bf16_full_size_linearity(env):
+    """M=N=K=4096: C(A1+A2, B) == C(A1,B) + C(A2,B) for bf16-exact sums, and row block vs oracle."""
+    t = env.torch
+    n = 4096
+    a = oracle.to_bf16_f32(rnd((n, n), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((n, n), 2, "uniform"))
+    ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+    cd = t.empty(n, n, device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nt_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), 1, n, n, n, env.stream()))
+    t.cuda.synchronize()
+    rows = np.r_[0:8, n - 8:n]
+    assert_close(cd[rows].cpu().numpy(), oracle.mm_t(a[rows], b), RTOL_BF16)
+    a2 = (ad.float() * 2).bfloat16()  # exact in bf16
+    c2 = t.empty(n, n, device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nt_bf16(a2.data_ptr(), bd.data_ptr(), c2.data_ptr(), 1, n, n, n, env.stream()))
+    t.cuda.synchronize()
+    assert t.equal(c2, cd * 2)
+
+
+# ------------------------------------------------------------------ row softmax
+@pytest.mark.parametrize("rows,cols", [(16, 8), (1, 1), (33, 1000), (64, 4096), (7, 4099), (5, 8192), (3, 20000)])
+def test_row_softmax_vs_oracle(env, rows, cols):
+    t = env.torch
+    x = rnd((rows, cols), 1) * 2
+    xd = t.from_numpy(x).cuda()
+    yd = t.full_like(xd, float("nan"))
+    env.nat.check(env.nat.core.i_hip_row_softmax(xd.data_ptr(), yd.data_ptr(), rows, cols, env.stream()))
+    t.cuda.synchronize()
+    assert_close(yd.cpu().numpy(), oracle.row_softmax(x), RTOL_F32)
+
+
+def test_row_softmax_full_size_properties(env):
+    """[16384, 4096] normal(0,1) seed 1: rows sum to 1, shift invariance, sampled rows vs oracle."""
+    t = env.torch
+    x = rnd((16384, 4096), 1)
+    xd = t.from_numpy(x).cuda()
+    yd = t.empty_like(xd)
+    env.nat.check(env.nat.core.i_hip_row_softmax(xd.data_ptr(), yd.data_ptr(), 16384, 4096, env.stream()))
+    t.cuda.synchronize()
+    assert (yd.sum(dim=-1) - 1).abs().max().item() < 1e-4
+    rows = np.r_[0:16, 16384 - 16:16384]
+    assert_close(yd[rows].cpu().numpy(), oracle.row_softmax(x[rows]), RTOL_F32)
+    y2 = t.empty_like(xd)
+    x2 = xd + 3.0
+    env.nat.check(env.nat.core.i_hip_row_softmax(x2.data_ptr(), y2.data_ptr(), 16384, 4096, env.stream()))
+    t.cuda.synchronize()
+    assert (y2 - yd).abs().max().item() <= 1e-4 * yd.abs().max().item()
