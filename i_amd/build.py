@@ -35,7 +35,7 @@ def build_kernels():
 
 
 def build_host():
-    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-fvisibility=hidden", "-Wno-unused-function",
           "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{PKG.parent / 'include'}",
           *host_sources(), "-o", LIB,
           f"-L{ROCM / 'lib'}", "-lamdhip64", f"-Wl,-rpath,{ROCM / 'lib'}", "-ldl", "-lpthread"])

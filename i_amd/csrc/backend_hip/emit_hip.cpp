@@ -1,0 +1,324 @@
+#include "emit_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <map>
+#include <set>
+#include <sstream>
+
+namespace ihipc {
+using namespace ic;
+namespace {
+
+// ------------------------------------------------------------------ expression printer
+std::string scalar_text(float v) {
+  if (std::isnan(v)) return "NAN";
+  if (std::isinf(v)) return v > 0 ? "INFINITY" : "(-INFINITY)";
+  char buf[64];
+  snprintf(buf, sizeof buf, "%.9g", (double)v);
+  std::string s = buf;
+  if (s.find('.') == std::string::npos && s.find('e') == std::string::npos && s.find("inf") == std::string::npos) s += ".0";
+  return s + "f";
+}
+
+std::string expr_text(const MExpr& e);
+
+std::string fold_call(const char* fn, const std::vector<MExprPtr>& args) {
+  std::string acc = expr_text(*args[0]);
+  for (size_t i = 1; i < args.size(); ++i) acc = std::string(fn) + "(" + acc + ", " + expr_text(*args[i]) + ")";
+  return acc;
+}
+std::string fold_infix(const char* sym, const std::vector<MExprPtr>& args, bool as_float) {
+  std::string acc = "(" + expr_text(*args[0]) + ")";
+  for (size_t i = 1; i < args.size(); ++i) acc = "(" + acc + " " + sym + " (" + expr_text(*args[i]) + "))";
+  return as_float ? "((float)" + acc + ")" : acc;
+}
+
+// scalar semantics of the C backend (compiler/src/backends/c/expr.rs:127-148)
+std::string op_text(Op op, const std::vector<MExprPtr>& args) {
+  switch (op) {
+    case Op::Add: return fold_infix("+", args, false);
+    case Op::Mul: return fold_infix("*", args, false);
+    case Op::Div: return fold_infix("/", args, false);
+    case Op::Sub: return fold_infix("-", args, false);
+    case Op::Max: return fold_call("fmaxf", args);
+    case Op::Min: return fold_call("fminf", args);
+    case Op::Pow: return fold_call("powf", args);
+    case Op::Log: return "logf(" + expr_text(*args[0]) + ")";
+    case Op::Gt: return fold_infix(">", args, true);
+    case Op::Ge: return fold_infix(">=", args, true);
+    case Op::Lt: return fold_infix("<", args, true);
+    case Op::Le: return fold_infix("<=", args, true);
+    case Op::Eq: return fold_infix("==", args, true);
+    case Op::Ne: return fold_infix("!=", args, true);
+    case Op::And: return fold_infix("&&", args, true);
+    case Op::Or: return fold_infix("||", args, true);
+    case Op::Xor: {
+      std::string acc = expr_text(*args[0]);
+      for (size_t i = 1; i < args.size(); ++i)
+        acc = "((float)(((" + acc + ") != 0.0f) != ((" + expr_text(*args[i]) + ") != 0.0f)))";
+      return acc;
+    }
+    case Op::Not: return "((float)!(" + expr_text(*args[0]) + "))";
+  }
+  return "0.0f";
+}
+
+std::string expr_text(const MExpr& e) {
+  auto b = [&](const char* sym) { return "(" + expr_text(*e.args[0]) + " " + sym + " " + expr_text(*e.args[1]) + ")"; };
+  switch (e.kind) {
+    case MExpr::Usize: return "(size_t)" + std::to_string(e.usize);
+    case MExpr::Scalar: return scalar_text(e.scalar);
+    case MExpr::Ident: return e.ident;
+    case MExpr::Index: return expr_text(*e.args[0]) + "[" + expr_text(*e.args[1]) + "]";
+    case MExpr::Field: {
+      const char* f = e.field == MField::Data ? "data" : e.field == MField::Shape ? "shape" : e.field == MField::Layout ? "layout" : "rank";
+      return expr_text(*e.args[0]) + "." + f;
+    }
+    case MExpr::Cast: return expr_text(*e.args[0]);
+    case MExpr::OpCall: return op_text(e.op, e.args);
+    case MExpr::Add: return b("+");
+    case MExpr::Sub: return b("-");
+    case MExpr::Mul: return b("*");
+    case MExpr::Div: return b("/");
+    case MExpr::Rem: return b("%");
+    case MExpr::Lt: return b("<");
+    case MExpr::Eq: return b("==");
+    case MExpr::And: return b("&&");
+  }
+  return "0";
+}
+
+// ------------------------------------------------------------------ parallelism analysis
+using PAct = Action<Param>;
+
+bool iter_uses(const Iter& it, size_t loop) {
+  if (it.raw) return it.loop == loop;
+  return std::find(it.loops.begin(), it.loops.end(), loop) != it.loops.end();
+}
+bool access_uses(const Access<Param>& a, size_t loop) {
+  for (const Iter& it : a.index)
+    if (iter_uses(it, loop)) return true;
+  return false;
+}
+
+struct Uses {
+  std::vector<const Access<Param>*> all;     // every access
+  std::set<Param> written;
+};
+void collect_scalar(const ScalarExpr<Param>& e, Uses& u) {
+  if (e.kind == ScalarExpr<Param>::Acc) u.all.push_back(&e.access);
+  for (const auto& a : e.args) collect_scalar(a, u);
+}
+void collect(const Block<Param>& block, Uses& u) {
+  for (const PAct& a : block) {
+    switch (a.kind) {
+      case PAct::Loop: collect(a.body, u); break;
+      case PAct::Init:
+        u.all.push_back(&a.write);
+        u.written.insert(a.write.buffer);
+        break;
+      case PAct::Compute:
+      case PAct::Snapshot:
+        u.all.push_back(&a.write);
+        u.written.insert(a.write.buffer);
+        for (const auto& r : a.reads) u.all.push_back(&r);
+        break;
+      case PAct::Scale:
+        u.all.push_back(&a.write);
+        u.written.insert(a.write.buffer);
+        collect_scalar(a.factor, u);
+        break;
+    }
+  }
+}
+
+// Buffers that only this kernel touches (fused temporaries) may be privatised.
+std::set<size_t> exclusive_intermediates(const ExecPlan& plan, size_t kernel) {
+  std::map<size_t, std::set<size_t>> users;
+  for (const Step& s : plan.exec)
+    if (s.kind == Step::Dispatch) {
+      for (BufferRef r : s.reads)
+        if (r.kind == BufferRef::Intermediate) users[r.id].insert(s.id);
+      for (BufferRef r : s.writes)
+        if (r.kind == BufferRef::Intermediate) users[r.id].insert(s.id);
+    }
+  std::set<size_t> out;
+  for (const auto& [id, ks] : users)
+    if (ks.size() == 1 && *ks.begin() == kernel) out.insert(id);
+  return out;
+}
+
+void analyze(const ExecPlan& plan, size_t k, GenericKernel& info) {
+  const Kernel<Param>& kernel = plan.kernels[k];
+  const Step* dispatch = nullptr;
+  for (const Step& s : plan.exec)
+    if (s.kind == Step::Dispatch && s.id == k) dispatch = &s;
+  const std::set<size_t> exclusive = exclusive_intermediates(plan, k);
+
+  const Block<Param>* block = &kernel.body;
+  std::set<Param> privatized;
+  while (block->size() == 1 && (*block)[0].kind == PAct::Loop) {
+    const PAct& loop = (*block)[0];
+    Uses u;
+    collect(loop.body, u);
+    bool ok = true;
+    std::set<Param> want_private;
+    for (const Param& w : u.written) {
+      bool all_use = true, none_use = true;
+      for (const auto* a : u.all)
+        if (a->buffer == w) {
+          const bool uses = access_uses(*a, loop.id);
+          all_use &= uses;
+          none_use &= !uses;
+        }
+      if (all_use) continue;  // distinct iterations touch distinct elements
+      const bool can_privatize = none_use && w.writeable && dispatch && w.ind < dispatch->writes.size() &&
+                                 dispatch->writes[w.ind].kind == BufferRef::Intermediate &&
+                                 exclusive.count(dispatch->writes[w.ind].id);
+      if (can_privatize) want_private.insert(w);
+      else ok = false;
+    }
+    if (ok) {
+      info.parallel_loops.push_back(loop.id);
+      info.parallel_extents.push_back(loop.extent);
+      privatized.insert(want_private.begin(), want_private.end());
+    }
+    block = &loop.body;
+  }
+  if (info.parallel_loops.empty()) return;
+  for (const Param& w : privatized) {
+    PrivateBuffer pb;
+    pb.writeable = w.ind;
+    const PlanBuffer& buf = plan.intermediates[dispatch->writes[w.ind].id];
+    pb.is_static = true;
+    pb.static_size = 1;
+    for (const auto& e : buf.layout) {
+      if (e.kind.kind == ExtentKind::Split) pb.static_size *= e.kind.factor;
+      else pb.is_static = false;
+    }
+    if (pb.is_static && pb.static_size > 4096) pb.is_static = false;
+    info.privates.push_back(pb);
+  }
+}
+
+// ------------------------------------------------------------------ statement printer
+struct Printer {
+  std::ostringstream os;
+  std::set<std::string> parallel;  // iterator names handled by the work-item decomposition
+  void line(int depth, const std::string& s) { os << std::string(2 * depth, ' ') << s << "\n"; }
+  void block(const std::vector<MStmt>& stmts, int depth) {
+    for (const MStmt& s : stmts) stmt(s, depth);
+  }
+  void stmt(const MStmt& s, int depth) {
+    switch (s.kind) {
+      case MStmt::Set: line(depth, expr_text(*s.dst) + " = " + expr_text(*s.value) + ";"); break;
+      case MStmt::Loop:
+        if (parallel.count(s.ident)) {
+          block(s.body, depth);
+        } else {
+          line(depth, "for (size_t " + s.ident + " = 0; " + s.ident + " < " + expr_text(*s.value) + "; ++" + s.ident + ") {");
+          block(s.body, depth + 1);
+          line(depth, "}");
+        }
+        break;
+      case MStmt::If:
+        line(depth, "if (" + expr_text(*s.value) + ") {");
+        block(s.body, depth + 1);
+        line(depth, "}");
+        break;
+      case MStmt::Return: break;
+      default: lower_error("statement kind is not valid inside a kernel");
+    }
+  }
+};
+
+const MStmt* find_loop(const std::vector<MStmt>& stmts, const std::string& iter) {
+  for (const MStmt& s : stmts) {
+    if (s.kind == MStmt::Loop && s.ident == iter) return &s;
+    if (s.kind == MStmt::Loop || s.kind == MStmt::If)
+      if (const MStmt* r = find_loop(s.body, iter)) return r;
+  }
+  return nullptr;
+}
+
+}  // namespace
+
+GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const std::vector<bool>& emit) {
+  GenericModule out;
+  out.kernels.resize(plan.kernels.size());
+  size_t rank = 1;
+  for (const auto& b : plan.inputs) rank = std::max({rank, b.shape.size(), b.layout.size()});
+  for (const auto& b : plan.intermediates) rank = std::max({rank, b.shape.size(), b.layout.size()});
+  for (const auto& b : plan.outputs) rank = std::max({rank, b.shape.size(), b.layout.size()});
+  out.rank = rank;
+
+  std::ostringstream src;
+  bool any = false;
+  src << "// generated by the i gfx950 backend\n#include <hip/hip_runtime.h>\n#include <math.h>\n#include <stddef.h>\n\n";
+  src << "struct View { float* data; size_t shape[" << rank << "]; size_t layout[" << rank << "]; };\n\n";
+  for (size_t k = 0; k < plan.kernels.size(); ++k) {
+    if (!emit[k]) continue;
+    any = true;
+    GenericKernel& info = out.kernels[k];
+    info.name = "f" + std::to_string(k);
+    info.n_reads = plan.kernels[k].reads.size();
+    info.n_writes = plan.kernels[k].writes.size();
+    analyze(plan, k, info);
+    const MFn& fn = module.kernels[k];
+
+    const size_t nr = std::max<size_t>(info.n_reads, 1), nw = std::max<size_t>(info.n_writes, 1);
+    src << "struct Args_" << info.name << " { View readonlys[" << nr << "]; View writeables[" << nw << "]; };\n";
+    src << "extern \"C\" __global__ void __launch_bounds__(64) " << info.name << "(Args_" << info.name << " args) {\n";
+    src << "  const View* readonlys = args.readonlys;\n";
+    src << "  View writeables[" << nw << "];\n";
+    src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
+    src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
+    src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
+    for (const PrivateBuffer& pb : info.privates) {
+      if (pb.is_static) {
+        src << "  float priv" << pb.writeable << "[" << pb.static_size << "];\n";
+        src << "  writeables[" << pb.writeable << "].data = priv" << pb.writeable << ";\n";
+      } else {
+        const Step* dispatch = nullptr;
+        for (const Step& st : plan.exec)
+          if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
+        const size_t prank = plan.intermediates[dispatch->writes[pb.writeable].id].layout.size();
+        src << "  { size_t n = 1; for (int d = 0; d < " << prank << "; ++d) n *= writeables[" << pb.writeable
+            << "].layout[d]; writeables[" << pb.writeable << "].data += wi_first * n; }\n";
+      }
+    }
+    Printer pr;
+    if (info.parallel_loops.empty()) {
+      src << "  if (wi_first != 0) return;\n";
+      pr.block(fn.body, 1);
+      src << pr.os.str();
+    } else {
+      std::vector<std::string> iters;
+      for (size_t id : info.parallel_loops) iters.push_back("i" + std::to_string(id));
+      for (const std::string& it : iters) {
+        const MStmt* loop = find_loop(fn.body, it);
+        if (!loop) lower_error("parallel loop " + it + " not found in kernel body");
+        src << "  const size_t n_" << it << " = " << expr_text(*loop->value) << ";\n";
+        pr.parallel.insert(it);
+      }
+      src << "  size_t wi_total = 1;\n";
+      for (const std::string& it : iters) src << "  wi_total *= n_" << it << ";\n";
+      src << "  for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
+      src << "    size_t wi_rest = wi;\n";
+      for (size_t t = iters.size(); t-- > 0;) {
+        src << "    const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
+        src << " wi_rest /= n_" << iters[t] << ";\n";
+      }
+      pr.block(fn.body, 2);
+      src << pr.os.str();
+      src << "  }\n";
+    }
+    src << "}\n\n";
+  }
+  if (any) out.source = src.str();
+  return out;
+}
+
+}  // namespace ihipc

@@ -1,0 +1,43 @@
+// Generic HIP lowering: any kernel of an exec plan that has no hand-written
+// counterpart is printed as a gfx950 `extern "C" __global__` function.
+//
+// The loop nest and scalar semantics come from the statement IR (ic::Module),
+// exactly what the C backend prints; what is added here is the mapping to the
+// GPU: independent loops on the kernel's outer spine become the work-item
+// index space (tile loops -> workgroups, element loops -> lanes, flattened into
+// one grid-stride index), reduction loops stay sequential inside a work-item,
+// and intermediates that fusion folded below a parallel loop become
+// work-item-private storage (registers / scratch when their size is static,
+// a per-work-item slice of a device buffer otherwise).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "../compiler/ir.h"
+
+namespace ihipc {
+
+struct PrivateBuffer {
+  size_t writeable = 0;   // index into the kernel's writeables
+  bool is_static = false;
+  size_t static_size = 0; // elements, when static
+};
+
+struct GenericKernel {
+  std::string name;                       // f<k>
+  size_t n_reads = 0, n_writes = 0;
+  std::vector<size_t> parallel_loops;     // loop ids, outermost first (empty: one work-item)
+  std::vector<ic::Extent<ic::Param>> parallel_extents;
+  std::vector<PrivateBuffer> privates;
+};
+
+struct GenericModule {
+  std::string source;                // full HIP translation unit ("" when no kernel needs it)
+  size_t rank = 1;                   // R of the View structs in the kernel argument block
+  std::vector<GenericKernel> kernels;  // one entry per plan kernel; name empty when not emitted
+};
+
+// `emit[k]` selects the kernels to print.
+GenericModule emit_generic_hip(const ic::ExecPlan& plan, const ic::Module& module, const std::vector<bool>& emit);
+
+}  // namespace ihipc

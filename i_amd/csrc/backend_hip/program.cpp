@@ -1,0 +1,452 @@
+#include "program.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <set>
+#include <sstream>
+
+#include "../runtime/hip_rt.h"
+#include "../runtime/kernel_launch.h"
+#include "hipcc.h"
+
+namespace ihipc {
+using namespace ic;
+namespace {
+
+size_t product(const std::vector<size_t>& v) {
+  size_t n = 1;
+  for (size_t x : v) n *= x;
+  return n;
+}
+
+const PlanBuffer& plan_buffer(const ExecPlan& plan, BufferRef r) {
+  return r.kind == BufferRef::Input ? plan.inputs.at(r.id) : r.kind == BufferRef::Intermediate ? plan.intermediates.at(r.id) : plan.outputs.at(r.id);
+}
+
+std::string ref_name(BufferRef r) {
+  return (r.kind == BufferRef::Input ? "in" : r.kind == BufferRef::Intermediate ? "s" : "out") + std::to_string(r.id);
+}
+
+// Everything the executor needs to know about one invocation.
+struct Run {
+  Program& p;
+  const ExecPlan& plan;
+  const std::vector<DeviceTensor>& inputs;
+  const std::vector<DeviceTensor>& outputs;
+  hipStream_t stream;
+  std::vector<void*> temps;                  // stream-ordered allocations to release
+  std::vector<void*> intermediates;          // device pointers (f32), null when not needed
+  std::map<size_t, void*> input_f32;         // bf16 inputs widened for f32 kernels
+  std::map<size_t, void*> output_f32;        // f32 staging for bf16 outputs
+
+  size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
+  size_t extent(const Extent<size_t>& e) const {
+    const size_t n = dim(e.source);
+    switch (e.kind.kind) {
+      case ExtentKind::Semantic: return n;
+      case ExtentKind::Base: {
+        const size_t f = product(e.kind.factors);
+        return f <= 1 ? n : (n + f - 1) / f;
+      }
+      case ExtentKind::Split: return e.kind.factor;
+    }
+    return n;
+  }
+  std::vector<size_t> shape_of(BufferRef r) const {
+    std::vector<size_t> out;
+    for (const auto& d : plan_buffer(plan, r).shape) out.push_back(dim(d));
+    return out;
+  }
+  std::vector<size_t> layout_of(BufferRef r) const {
+    std::vector<size_t> out;
+    for (const auto& e : plan_buffer(plan, r).layout) out.push_back(extent(e));
+    return out;
+  }
+  DType dtype_of(BufferRef r) const {
+    if (r.kind == BufferRef::Input) return inputs[r.id].dtype;
+    if (r.kind == BufferRef::Output) return outputs[r.id].dtype;
+    return DType::F32;
+  }
+  void* raw_ptr(BufferRef r) const {
+    if (r.kind == BufferRef::Input) return inputs[r.id].data;
+    if (r.kind == BufferRef::Output) return outputs[r.id].data;
+    return intermediates[r.id];
+  }
+
+  ihip::Err alloc(void** ptr, size_t bytes) {
+    if (bytes == 0) bytes = 4;
+    if (ihip::Err e = ihip::check(hipMallocAsync(ptr, bytes, stream), "hipMallocAsync"); !e.empty()) return e;
+    temps.push_back(*ptr);
+    return {};
+  }
+
+  // Device pointer to f32 data of a buffer some f32 kernel reads.
+  ihip::Err read_f32(BufferRef r, void** ptr) {
+    if (dtype_of(r) == DType::F32) {
+      *ptr = r.kind == BufferRef::Output && output_f32.count(r.id) ? output_f32[r.id] : raw_ptr(r);
+      return {};
+    }
+    if (r.kind == BufferRef::Output) {  // a bf16 output that a later kernel reads back: use its f32 staging
+      *ptr = output_f32.at(r.id);
+      return {};
+    }
+    auto it = input_f32.find(r.id);
+    if (it == input_f32.end()) {
+      const size_t n = product(inputs[r.id].shape);
+      void* tmp = nullptr;
+      if (ihip::Err e = alloc(&tmp, n * 4); !e.empty()) return e;
+      if (ihip::Err e = ihip::launch_convert(inputs[r.id].data, tmp, ihip::BF16, ihip::F32, n, stream); !e.empty()) return e;
+      it = input_f32.emplace(r.id, tmp).first;
+    }
+    *ptr = it->second;
+    return {};
+  }
+  // Device pointer an f32-producing kernel writes to.
+  ihip::Err write_f32(BufferRef r, void** ptr) {
+    if (r.kind != BufferRef::Output || outputs[r.id].dtype == DType::F32) {
+      *ptr = raw_ptr(r);
+      return {};
+    }
+    auto it = output_f32.find(r.id);
+    if (it == output_f32.end()) {
+      void* tmp = nullptr;
+      if (ihip::Err e = alloc(&tmp, product(shape_of(r)) * 4); !e.empty()) return e;
+      it = output_f32.emplace(r.id, tmp).first;
+    }
+    *ptr = it->second;
+    return {};
+  }
+};
+
+// ---------------------------------------------------------------- hand-written kernels
+// Returns true when kernel k can run on its hand-written form with these operands.
+bool hand_usable(const Run& run, const Recognized& r) {
+  // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
+  if (const char* v = std::getenv("ILANG_HIP_GENERATED_ONLY"))
+    if (*v && *v != '0') return false;
+  auto rows_cols = [&](const Operand& o) { return run.shape_of(o.buffer); };
+  switch (r.kind) {
+    case Recognized::None: return false;
+    case Recognized::Attention: {
+      const DType t = run.dtype_of(r.a.buffer);
+      if (run.dtype_of(r.b.buffer) != t || run.dtype_of(r.c.buffer) != t) return false;
+      const auto q = rows_cols(r.a), v = rows_cols(r.c);
+      if (q.size() < 2 || v.size() < 2) return false;
+      return ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back());
+    }
+    case Recognized::GemmNT: {
+      if (run.dtype_of(r.a.buffer) != DType::BF16 || run.dtype_of(r.b.buffer) != DType::BF16) return false;
+      const auto a = rows_cols(r.a);
+      return a.size() >= 2 && ihip::gemm_nt_bf16_supported(a.back());
+    }
+    case Recognized::RowSoftmax: return true;
+  }
+  return false;
+}
+
+std::set<size_t> hand_intermediates(const Recognized& r) {
+  std::set<size_t> out;
+  auto add = [&](BufferRef b) {
+    if (b.kind == BufferRef::Intermediate) out.insert(b.id);
+  };
+  add(r.out);
+  add(r.a.buffer);
+  if (r.kind != Recognized::RowSoftmax) add(r.b.buffer);
+  if (r.kind == Recognized::Attention) {
+    add(r.c.buffer);
+    if (r.has_scale) add(r.scale.buffer);
+  }
+  return out;
+}
+
+ihip::Err launch_hand(Run& run, const Recognized& r) {
+  switch (r.kind) {
+    case Recognized::Attention: {
+      const auto q = run.shape_of(r.a.buffer), k = run.shape_of(r.b.buffer), v = run.shape_of(r.c.buffer);
+      const size_t nb = r.batch_rank;
+      size_t bh = 1;
+      for (size_t d = 0; d < nb; ++d) bh *= q[d];
+      const size_t nq = q[nb], dq = q[nb + 1], nk = k[nb], dv = v[nb + 1];
+      // repeated indexes constrain shapes; a mismatch would send the kernel out of bounds
+      for (size_t d = 0; d < nb; ++d)
+        if (k[d] != q[d] || v[d] != q[d]) return "attention operands disagree on a batch extent";
+      if (k[nb + 1] != dq || v[nb] != nk) return "attention operands disagree on a contracted extent";
+      const bool bf16 = run.dtype_of(r.a.buffer) == DType::BF16;
+      const float* scale_ptr = nullptr;
+      if (r.has_scale) {
+        void* sp = nullptr;
+        if (ihip::Err e = run.read_f32(r.scale.buffer, &sp); !e.empty()) return e;
+        scale_ptr = static_cast<const float*>(sp);
+      }
+      void* out = nullptr;
+      ihip::DType out_dt = ihip::F32;
+      if (bf16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16) {
+        out = run.raw_ptr(r.out);
+        out_dt = ihip::BF16;
+      } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
+        return e;
+      }
+      return ihip::launch_attention(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), run.raw_ptr(r.c.buffer), out,
+                                    bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream);
+    }
+    case Recognized::GemmNT: {
+      const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
+      const size_t nb = r.batch_rank;
+      size_t bh = 1;
+      for (size_t d = 0; d < nb; ++d) {
+        if (b[d] != a[d]) return "gemm operands disagree on a batch extent";
+        bh *= a[d];
+      }
+      if (b[nb + 1] != a[nb + 1]) return "gemm operands disagree on the contracted extent";
+      void* out = nullptr;
+      if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
+                                       a[nb], b[nb], a[nb + 1], run.stream);
+    }
+    case Recognized::RowSoftmax: {
+      const auto x = run.shape_of(r.a.buffer);
+      size_t rows = 1;
+      for (size_t d = 0; d + 1 < x.size(); ++d) rows *= x[d];
+      void *in = nullptr, *out = nullptr;
+      if (ihip::Err e = run.read_f32(r.a.buffer, &in); !e.empty()) return e;
+      if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream);
+    }
+    default: return "no hand-written kernel";
+  }
+}
+
+// ---------------------------------------------------------------- generated kernels
+ihip::Err ensure_image(Program& p) {
+  std::lock_guard<std::mutex> lock(p.mu);
+  if (p.image_built) return {};
+  if (p.generic.source.empty()) return "program has no generated kernels";
+  if (std::string e = hipcc_build(p.generic.source, &p.image); !e.empty()) return e;
+  p.image_built = true;
+  return {};
+}
+
+ihip::Err generic_function(Program& p, const std::string& name, hipFunction_t* fn) {
+  if (ihip::Err e = ensure_image(p); !e.empty()) return e;
+  std::lock_guard<std::mutex> lock(p.mu);
+  int dev = 0;
+  if (ihip::Err e = ihip::check(hipGetDevice(&dev), "hipGetDevice"); !e.empty()) return e;
+  auto it = p.modules.find(dev);
+  if (it == p.modules.end()) {
+    hipModule_t mod = nullptr;
+    if (ihip::Err e = ihip::load_module(p.image.data(), &mod); !e.empty()) return e;
+    it = p.modules.emplace(dev, mod).first;
+  }
+  return ihip::module_function(it->second, name.c_str(), fn);
+}
+
+ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
+  Program& p = run.p;
+  const GenericKernel& gk = p.generic.kernels[k];
+  if (gk.name.empty()) return "kernel " + std::to_string(k) + " has no generated form";
+  const size_t R = p.generic.rank;
+  const size_t view_bytes = 8 + 16 * R;
+  const size_t nr = std::max<size_t>(gk.n_reads, 1), nw = std::max<size_t>(gk.n_writes, 1);
+  std::vector<unsigned char> args((nr + nw) * view_bytes, 0);
+  if (args.size() > 4000) return "kernel " + std::to_string(k) + " takes too many buffers for one launch";
+
+  // work-item space
+  size_t total = 1;
+  for (const auto& e : gk.parallel_extents) {
+    const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
+    Extent<size_t> resolved{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind};
+    total *= run.extent(resolved);
+  }
+  if (total == 0) return {};
+  size_t threads = gk.parallel_loops.empty() ? 1 : total;
+  // dynamic private buffers cost memory per work-item slot: cap the slots
+  size_t slot_elems = 0;
+  for (const PrivateBuffer& pb : gk.privates)
+    if (!pb.is_static) slot_elems += std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+  size_t max_threads = size_t(1) << 20;
+  if (slot_elems) max_threads = std::max<size_t>(64, std::min(max_threads, (size_t(1) << 28) / (slot_elems * 4)));
+  threads = std::min(threads, max_threads);
+  const unsigned grid = (unsigned)((threads + 63) / 64);
+  const size_t slots = (size_t)grid * 64;
+
+  auto fill = [&](size_t slot, void* data, BufferRef r) {
+    unsigned char* v = args.data() + slot * view_bytes;
+    std::memcpy(v, &data, 8);
+    const auto shape = run.shape_of(r), layout = run.layout_of(r);
+    for (size_t d = 0; d < shape.size() && d < R; ++d) std::memcpy(v + 8 + 8 * d, &shape[d], 8);
+    for (size_t d = 0; d < layout.size() && d < R; ++d) std::memcpy(v + 8 + 8 * R + 8 * d, &layout[d], 8);
+  };
+  for (size_t i = 0; i < dispatch.reads.size(); ++i) {
+    void* ptr = nullptr;
+    if (ihip::Err e = run.read_f32(dispatch.reads[i], &ptr); !e.empty()) return e;
+    fill(i, ptr, dispatch.reads[i]);
+  }
+  for (size_t i = 0; i < dispatch.writes.size(); ++i) {
+    const BufferRef r = dispatch.writes[i];
+    void* ptr = nullptr;
+    const PrivateBuffer* priv = nullptr;
+    for (const PrivateBuffer& pb : gk.privates)
+      if (pb.writeable == i) priv = &pb;
+    if (priv && !priv->is_static) {
+      const size_t n = std::max<size_t>(1, product(run.layout_of(r)));
+      if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
+    } else if (!priv) {
+      if (ihip::Err e = run.write_f32(r, &ptr); !e.empty()) return e;
+    }
+    fill(nr + i, ptr, r);
+  }
+  hipFunction_t fn;
+  if (ihip::Err e = generic_function(p, gk.name, &fn); !e.empty()) return e;
+  return ihip::launch(fn, grid, 1, 1, 64, args.data(), args.size(), run.stream);
+}
+
+const Step* find_dispatch(const ExecPlan& plan, size_t k) {
+  for (const Step& s : plan.exec)
+    if (s.kind == Step::Dispatch && s.id == k) return &s;
+  return nullptr;
+}
+
+}  // namespace
+
+Program::~Program() {
+  for (auto& kv : modules) ihip::unload_module(kv.second);
+}
+
+std::string compile_program(const Component& component, Program** out) {
+  auto p = std::make_unique<Program>();
+  p->low = lower_component(component);
+  p->module = lower_exec_plan_to_module(p->low.plan);
+  p->recognized = recognize_kernels(p->low);
+  if (p->recognized.size() != p->low.plan.kernels.size()) lower_error("kernel recognition lost track of the kernel list");
+  std::vector<bool> emit(p->low.plan.kernels.size(), true);
+  p->generic = emit_generic_hip(p->low.plan, p->module, emit);
+  bool needs_generated = false;
+  for (const Recognized& r : p->recognized) needs_generated |= r.kind == Recognized::None;
+  if (needs_generated)
+    if (ihip::Err e = ensure_image(*p); !e.empty()) return e;
+  *out = p.release();
+  return {};
+}
+
+std::string program_code(const Component& component) {
+  const Lowered low = lower_component(component);
+  const Module module = lower_exec_plan_to_module(low.plan);
+  const auto rec = recognize_kernels(low);
+  const GenericModule gen = emit_generic_hip(low.plan, module, std::vector<bool>(low.plan.kernels.size(), true));
+  std::ostringstream os;
+  os << "// 𝚒 gfx950 backend plan: " << low.plan.inputs.size() << " input(s), " << low.plan.intermediates.size()
+     << " intermediate(s), " << low.plan.outputs.size() << " output(s), " << low.plan.kernels.size() << " kernel(s)\n";
+  for (size_t k = 0; k < low.plan.kernels.size(); ++k) {
+    const Step* d = find_dispatch(low.plan, k);
+    os << "// f" << k << ": " << rec[k].describe();
+    if (rec[k].kind != Recognized::None) {
+      os << " [";
+      os << ref_name(rec[k].a.buffer);
+      if (rec[k].kind != Recognized::RowSoftmax) os << ", " << ref_name(rec[k].b.buffer);
+      if (rec[k].kind == Recognized::Attention) os << ", " << ref_name(rec[k].c.buffer);
+      if (rec[k].has_scale) os << ", scale " << ref_name(rec[k].scale.buffer);
+      os << " -> " << ref_name(rec[k].out) << "]; generated form below runs when operands are outside its limits";
+    }
+    os << "\n//     reads";
+    for (BufferRef r : d->reads) os << " " << ref_name(r);
+    os << "; writes";
+    for (BufferRef r : d->writes) os << " " << ref_name(r);
+    os << "\n//     work-items:";
+    if (gen.kernels[k].parallel_loops.empty()) os << " 1 (no independent outer loop)";
+    for (size_t id : gen.kernels[k].parallel_loops) os << " i" << id;
+    if (!gen.kernels[k].privates.empty()) {
+      os << "; work-item-private:";
+      for (const auto& pb : gen.kernels[k].privates)
+        os << " " << ref_name(d->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
+    }
+    os << "\n";
+  }
+  os << "\n" << gen.source;
+  return os.str();
+}
+
+size_t output_count(const Program& p) { return p.low.plan.count; }
+std::vector<size_t> output_ranks(const Program& p) { return p.low.plan.ranks; }
+size_t input_count(const Program& p) { return p.low.plan.inputs.size(); }
+size_t input_rank(const Program& p, size_t input) { return p.low.plan.inputs.at(input).shape.size(); }
+
+std::string output_shapes(const Program& p, const std::vector<std::vector<size_t>>& input_shapes,
+                          std::vector<std::vector<size_t>>* shapes) {
+  shapes->clear();
+  for (const auto& shape : p.low.plan.shapes) {
+    std::vector<size_t> out;
+    for (const auto& d : shape) {
+      if (d.buffer >= input_shapes.size()) return "program needs input " + std::to_string(d.buffer) + " to size its outputs";
+      if (d.dim >= input_shapes[d.buffer].size())
+        return "input " + std::to_string(d.buffer) + " has rank " + std::to_string(input_shapes[d.buffer].size()) +
+               ", program reads dimension " + std::to_string(d.dim);
+      out.push_back(input_shapes[d.buffer][d.dim]);
+    }
+    shapes->push_back(std::move(out));
+  }
+  return {};
+}
+
+std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
+                    hipStream_t stream) {
+  const ExecPlan& plan = p.low.plan;
+  if (inputs.size() < plan.inputs.size())
+    return "program takes " + std::to_string(plan.inputs.size()) + " inputs, got " + std::to_string(inputs.size());
+  for (size_t i = 0; i < plan.inputs.size(); ++i) {
+    if (inputs[i].shape.size() != plan.inputs[i].shape.size())
+      return "input " + std::to_string(i) + " has rank " + std::to_string(inputs[i].shape.size()) + ", program expects rank " +
+             std::to_string(plan.inputs[i].shape.size());
+    if (!inputs[i].data && product(inputs[i].shape) != 0) return "input " + std::to_string(i) + " has no data";
+  }
+  if (outputs.size() != plan.count) return "wrong output count";
+  Run run{p, plan, inputs, outputs, stream, {}, std::vector<void*>(plan.intermediates.size(), nullptr), {}, {}};
+  for (size_t o = 0; o < outputs.size(); ++o) {
+    const auto want = run.shape_of({BufferRef::Output, o});
+    if (!outputs[o].shape.empty() && outputs[o].shape != want) return "output " + std::to_string(o) + " has the wrong shape";
+    if (!outputs[o].data && product(want) != 0) return "output " + std::to_string(o) + " has no data";
+  }
+
+  // which kernels run hand-written, and which intermediates must exist
+  std::vector<bool> hand(plan.kernels.size(), false);
+  std::set<size_t> needed;
+  for (size_t k = 0; k < plan.kernels.size(); ++k) {
+    const Step* d = find_dispatch(plan, k);
+    if (!d) return "kernel " + std::to_string(k) + " is never dispatched";
+    hand[k] = hand_usable(run, p.recognized[k]);
+    if (hand[k]) {
+      for (size_t id : hand_intermediates(p.recognized[k])) needed.insert(id);
+    } else {
+      std::set<size_t> priv;
+      for (const PrivateBuffer& pb : p.generic.kernels[k].privates) priv.insert(pb.writeable);
+      for (BufferRef r : d->reads)
+        if (r.kind == BufferRef::Intermediate) needed.insert(r.id);
+      for (size_t i = 0; i < d->writes.size(); ++i)
+        if (d->writes[i].kind == BufferRef::Intermediate && !priv.count(i)) needed.insert(d->writes[i].id);
+    }
+  }
+
+  ihip::Err err;
+  auto finish = [&](ihip::Err e) {
+    for (auto it = run.temps.rbegin(); it != run.temps.rend(); ++it) (void)hipFreeAsync(*it, stream);
+    return e;
+  };
+  for (const Step& step : plan.exec) {
+    if (step.kind == Step::Alloc) {
+      if (!needed.count(step.id)) continue;
+      const size_t n = product(run.layout_of({BufferRef::Intermediate, step.id}));
+      if (ihip::Err e = run.alloc(&run.intermediates[step.id], n * 4); !e.empty()) return finish(e);
+    } else if (step.kind == Step::Dispatch) {
+      ihip::Err e = hand[step.id] ? launch_hand(run, p.recognized[step.id]) : launch_generic(run, step.id, step);
+      if (!e.empty()) return finish("kernel f" + std::to_string(step.id) + ": " + e);
+    }
+  }
+  // bf16 outputs that were produced through f32 staging
+  for (const auto& [o, tmp] : run.output_f32) {
+    const size_t n = product(run.shape_of({BufferRef::Output, o}));
+    if (ihip::Err e = ihip::launch_convert(tmp, outputs[o].data, ihip::F32, ihip::BF16, n, stream); !e.empty()) return finish(e);
+  }
+  return finish({});
+}
+
+}  // namespace ihipc

@@ -1,0 +1,63 @@
+// A compiled 𝚒 program for the gfx950 backend: the lowered component, the
+// per-kernel choice between a hand-written kernel and a generated one, the
+// generated code object, and the executor that walks the exec plan
+// (alloc intermediates -> dispatch kernels in order -> free), the device-side
+// counterpart of the `exec` function the reference's C backend emits
+// (ilang-python/annotated-flashattn.c:312-422).
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../compiler/ir.h"
+#include "emit_hip.h"
+#include "recognize.h"
+
+namespace ihipc {
+
+enum class DType { F32 = 0, BF16 = 1 };
+
+struct DeviceTensor {
+  void* data = nullptr;
+  std::vector<size_t> shape;
+  DType dtype = DType::F32;
+};
+
+struct Program {
+  ic::Lowered low;
+  ic::Module module;
+  std::vector<Recognized> recognized;  // per plan kernel
+  GenericModule generic;               // source for every kernel (hand-written ones keep a generated twin)
+  std::vector<char> image;             // built lazily unless some kernel can only run generated
+  bool image_built = false;
+  std::mutex mu;
+  std::map<int, hipModule_t> modules;  // per device
+
+  ~Program();
+};
+
+// Lower, recognise, emit; builds the generated code object right away when a
+// kernel has no hand-written form.  Throws ic::CompileError / returns error text.
+std::string compile_program(const ic::Component& component, Program** out);
+
+// Human-readable backend source: the kernel plan followed by the generated HIP.
+std::string program_code(const ic::Component& component);
+
+size_t output_count(const Program& p);
+std::vector<size_t> output_ranks(const Program& p);
+// "" on success
+std::string output_shapes(const Program& p, const std::vector<std::vector<size_t>>& input_shapes,
+                          std::vector<std::vector<size_t>>* shapes);
+size_t input_count(const Program& p);
+size_t input_rank(const Program& p, size_t input);
+
+// Enqueue the program on `stream`.  All tensors live in device memory.
+// Temporary buffers are stream-ordered allocations, so the call does not wait
+// for the GPU.  Returns "" on success.
+std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
+                    hipStream_t stream);
+
+}  // namespace ihipc

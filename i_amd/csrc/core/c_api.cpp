@@ -4,10 +4,20 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <string>
+#include <vector>
 
+#include "../../../include/i_hip.h"
+#include "../backend_hip/program.h"
+#include "../runtime/hip_rt.h"
 #include "error.h"
 #include "handles.h"
+
+struct i_program {
+  ihipc::Program* inner = nullptr;
+  ~i_program() { delete inner; }
+};
 
 namespace {
 
@@ -43,8 +53,84 @@ bool valid_utf8(const char* s) {
   return true;
 }
 
+int fail(const std::string& message) {
+  icore::set_error(message);
+  return -1;
+}
+
+// Shapes of the host operands, cut to the ranks the program reads.
+std::vector<std::vector<size_t>> host_shapes(const ihipc::Program& p, const i_tensor* inputs, size_t input_count) {
+  std::vector<std::vector<size_t>> out;
+  for (size_t i = 0; i < input_count; ++i)
+    out.emplace_back(inputs[i].shape ? std::vector<size_t>(inputs[i].shape, inputs[i].shape + inputs[i].rank) : std::vector<size_t>());
+  return out;
+}
+
+// Host entry: upload f32 operands, run, download, wait.  Mirrors the
+// blocking behaviour of the reference's exec (core/src/lib.rs:200-225).
+std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_count, const std::vector<float*>& out_ptrs) {
+  const auto in_shapes = host_shapes(p, inputs, input_count);
+  std::vector<std::vector<size_t>> out_shapes;
+  if (std::string e = ihipc::output_shapes(p, in_shapes, &out_shapes); !e.empty()) return e;
+  std::vector<void*> owned;
+  auto cleanup = [&] {
+    for (void* ptr : owned) ihip::dev_free(ptr);
+  };
+  std::vector<ihipc::DeviceTensor> in, out;
+  hipStream_t stream = nullptr;
+  for (size_t i = 0; i < input_count; ++i) {
+    size_t n = 1;
+    for (size_t d : in_shapes[i]) n *= d;
+    ihipc::DeviceTensor t;
+    t.shape = in_shapes[i];
+    if (n && !inputs[i].data) {
+      cleanup();
+      return "input " + std::to_string(i) + " has no data";
+    }
+    if (ihip::Err e = ihip::dev_alloc(&t.data, n * 4); !e.empty()) {
+      cleanup();
+      return e;
+    }
+    owned.push_back(t.data);
+    if (ihip::Err e = ihip::h2d(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
+      cleanup();
+      return e;
+    }
+    in.push_back(std::move(t));
+  }
+  for (size_t o = 0; o < out_shapes.size(); ++o) {
+    size_t n = 1;
+    for (size_t d : out_shapes[o]) n *= d;
+    ihipc::DeviceTensor t;
+    t.shape = out_shapes[o];
+    if (ihip::Err e = ihip::dev_alloc(&t.data, n * 4); !e.empty()) {
+      cleanup();
+      return e;
+    }
+    owned.push_back(t.data);
+    out.push_back(std::move(t));
+  }
+  std::string err;
+  try {
+    err = ihipc::execute(p, in, out, stream);
+  } catch (const std::exception& e) {
+    err = e.what();
+  }
+  for (size_t o = 0; err.empty() && o < out.size(); ++o) {
+    size_t n = 1;
+    for (size_t d : out_shapes[o]) n *= d;
+    if (n && !out_ptrs[o]) err = "output " + std::to_string(o) + " has no data";
+    else err = ihip::d2h(out_ptrs[o], out[o].data, n * 4, stream);
+  }
+  const ihip::Err sync_err = ihip::sync(stream);
+  if (err.empty()) err = sync_err;
+  cleanup();
+  return err;
+}
+
 }  // namespace
 
+#pragma GCC visibility push(default)
 extern "C" {
 
 i_component* i_parse(const char* src) {
@@ -83,10 +169,180 @@ i_component* i_swap(const i_component* component) {
   return wrap(std::move(c));
 }
 
+char* i_code(const i_component* component) {
+  if (!component) {
+    icore::set_error("null component");
+    return nullptr;
+  }
+  try {
+    const std::string text = ihipc::program_code(*component->inner);
+    if (text.find('\0') != std::string::npos) {
+      icore::set_error("source contains interior NUL");
+      return nullptr;
+    }
+    char* out = static_cast<char*>(std::malloc(text.size() + 1));
+    if (!out) {
+      icore::set_error("out of memory");
+      return nullptr;
+    }
+    std::memcpy(out, text.c_str(), text.size() + 1);
+    return out;
+  } catch (const ic::CompileError& e) {
+    icore::set_error(e.debug_string());
+  } catch (const std::exception& e) {
+    icore::set_error(e.what());
+  }
+  return nullptr;
+}
+
+i_program* i_compile(const i_component* component) {
+  if (!component) {
+    icore::set_error("null component");
+    return nullptr;
+  }
+  try {
+    ihipc::Program* inner = nullptr;
+    const std::string err = ihipc::compile_program(*component->inner, &inner);
+    if (!err.empty()) {
+      icore::set_error(err);
+      return nullptr;
+    }
+    auto* program = new i_program;
+    program->inner = inner;
+    return program;
+  } catch (const ic::CompileError& e) {
+    icore::set_error(e.debug_string());
+  } catch (const std::exception& e) {
+    icore::set_error(e.what());
+  }
+  return nullptr;
+}
+
+size_t i_output_count(const i_program* program) {
+  if (!program) {
+    icore::set_error("null program");
+    return 0;
+  }
+  return ihipc::output_count(*program->inner);
+}
+
+int i_output_ranks(const i_program* program, size_t* ranks) {
+  if (!program) return fail("null program");
+  if (!ranks) return fail("null ranks");
+  const auto r = ihipc::output_ranks(*program->inner);
+  for (size_t i = 0; i < r.size(); ++i) ranks[i] = r[i];
+  return 0;
+}
+
+int i_output_shapes(const i_program* program, const i_tensor* inputs, size_t input_count, size_t** shapes) {
+  if (!program) return fail("null program");
+  if (input_count > 0 && !inputs) return fail("null inputs");
+  if (!shapes) return fail("null shapes");
+  std::vector<std::vector<size_t>> out;
+  const std::string err = ihipc::output_shapes(*program->inner, host_shapes(*program->inner, inputs, input_count), &out);
+  if (!err.empty()) return fail(err);
+  for (size_t o = 0; o < out.size(); ++o)
+    for (size_t d = 0; d < out[o].size(); ++d) shapes[o][d] = out[o][d];
+  return 0;
+}
+
+int i_exec_into(const i_program* program, const i_tensor* inputs, size_t input_count, i_tensor_mut* outputs,
+                size_t output_count) {
+  if (!program) return fail("null program");
+  if (input_count > 0 && !inputs) return fail("null inputs");
+  if (output_count != ihipc::output_count(*program->inner)) return fail("wrong output count");
+  if (output_count > 0 && !outputs) return fail("null outputs");
+  std::vector<float*> out_ptrs;
+  for (size_t o = 0; o < output_count; ++o) out_ptrs.push_back(outputs[o].data);
+  const std::string err = run_host(*program->inner, inputs, input_count, out_ptrs);
+  return err.empty() ? 0 : fail(err);
+}
+
+i_outputs i_exec(const i_program* program, const i_tensor* inputs, size_t input_count) {
+  i_outputs none{nullptr, 0};
+  if (!program) {
+    icore::set_error("null program");
+    return none;
+  }
+  if (input_count > 0 && !inputs) {
+    icore::set_error("null inputs");
+    return none;
+  }
+  ihipc::Program& p = *program->inner;
+  std::vector<std::vector<size_t>> shapes;
+  if (std::string err = ihipc::output_shapes(p, host_shapes(p, inputs, input_count), &shapes); !err.empty()) {
+    icore::set_error(err);
+    return none;
+  }
+  const size_t count = shapes.size();
+  auto* tensors = static_cast<i_owned_tensor*>(std::calloc(count ? count : 1, sizeof(i_owned_tensor)));
+  std::vector<float*> out_ptrs;
+  bool ok = tensors != nullptr;
+  for (size_t o = 0; ok && o < count; ++o) {
+    size_t len = 1;
+    for (size_t d : shapes[o]) len *= d;
+    tensors[o].rank = shapes[o].size();
+    tensors[o].len = len;
+    tensors[o].data = static_cast<float*>(std::calloc(len ? len : 1, sizeof(float)));  // zero-filled, as the reference
+    tensors[o].shape = static_cast<size_t*>(std::calloc(shapes[o].size() ? shapes[o].size() : 1, sizeof(size_t)));
+    ok = tensors[o].data && tensors[o].shape;
+    if (ok) std::copy(shapes[o].begin(), shapes[o].end(), tensors[o].shape);
+    out_ptrs.push_back(tensors[o].data);
+  }
+  i_outputs result{tensors, count};
+  std::string err = ok ? run_host(p, inputs, input_count, out_ptrs) : std::string("out of memory");
+  if (!err.empty()) {
+    i_outputs_free(result);
+    icore::set_error(err);
+    return none;
+  }
+  return result;
+}
+
+int i_exec_into_device(const i_program* program, const i_device_tensor* inputs, size_t input_count,
+                       const i_device_tensor* outputs, size_t output_count, void* stream) {
+  if (!program) return fail("null program");
+  if (input_count > 0 && !inputs) return fail("null inputs");
+  if (output_count != ihipc::output_count(*program->inner)) return fail("wrong output count");
+  if (output_count > 0 && !outputs) return fail("null outputs");
+  auto convert = [](const i_device_tensor* t, size_t n, std::vector<ihipc::DeviceTensor>* out) -> bool {
+    for (size_t i = 0; i < n; ++i) {
+      if (t[i].dtype != I_DTYPE_F32 && t[i].dtype != I_DTYPE_BF16) return false;
+      ihipc::DeviceTensor d;
+      d.data = t[i].data;
+      d.dtype = t[i].dtype == I_DTYPE_BF16 ? ihipc::DType::BF16 : ihipc::DType::F32;
+      if (t[i].rank > 0 && !t[i].shape) return false;
+      d.shape.assign(t[i].shape, t[i].shape + t[i].rank);
+      out->push_back(std::move(d));
+    }
+    return true;
+  };
+  std::vector<ihipc::DeviceTensor> in, out;
+  if (!convert(inputs, input_count, &in) || !convert(outputs, output_count, &out)) return fail("bad device tensor (dtype or shape)");
+  try {
+    const std::string err = ihipc::execute(*program->inner, in, out, static_cast<hipStream_t>(stream));
+    return err.empty() ? 0 : fail(err);
+  } catch (const std::exception& e) {
+    return fail(e.what());
+  }
+}
+
 void i_component_free(i_component* component) { delete component; }
+
+void i_program_free(i_program* program) { delete program; }
+
+void i_outputs_free(i_outputs outputs) {
+  if (!outputs.tensors) return;
+  for (size_t i = 0; i < outputs.count; ++i) {
+    std::free(outputs.tensors[i].data);
+    std::free(outputs.tensors[i].shape);
+  }
+  std::free(outputs.tensors);
+}
 
 void i_string_free(char* s) { std::free(s); }
 
 const char* i_error(void) { return icore::last_error(); }
 
 }  // extern "C"
+#pragma GCC visibility pop

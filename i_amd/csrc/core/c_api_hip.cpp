@@ -12,13 +12,14 @@ int finish(const ihip::Err& e) {
 bool dtype_ok(int d) { return d == I_DTYPE_F32 || d == I_DTYPE_BF16; }
 }  // namespace
 
+#pragma GCC visibility push(default)
 extern "C" {
 
 int i_hip_attention(const void* q, const void* k, const void* v, void* o, int in_dtype, int out_dtype, size_t bh,
                     size_t nq, size_t nk, size_t d, size_t dv, float scale, void* stream) {
   if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype)) return finish("unknown dtype");
   return finish(ihip::launch_attention(q, k, v, o, (ihip::DType)in_dtype, (ihip::DType)out_dtype, bh, nq, nk, d, dv,
-                                       scale, (hipStream_t)stream));
+                                       nullptr, scale, (hipStream_t)stream));
 }
 
 int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k, void* stream) {
@@ -36,3 +37,4 @@ int i_hip_convert(const void* src, void* dst, int from_dtype, int to_dtype, size
 
 
 }  // extern "C"
+#pragma GCC visibility pop

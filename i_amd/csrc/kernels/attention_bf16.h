@@ -64,6 +64,12 @@ __device__ __forceinline__ void attn_fwd_bf16_body(const AttnParams& p) {
   const bf16_t* __restrict__ K = reinterpret_cast<const bf16_t*>(p.k) + (size_t)head * p.nk * p.d;
   const bf16_t* __restrict__ V = reinterpret_cast<const bf16_t*>(p.v) + (size_t)head * p.nk * p.dv;
 
+  // A negative scale is folded into Q (sign flip is exact), so the running max
+  // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
+  const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
+  const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
+  const float scale_log2 = fabsf(scale_raw) * I_LOG2_E32;
+
   // Q^T fragments (B operand): lane (c, h) holds q[row][16*ks + 8*h .. +8].
   const uint32_t qrow = qt * BM + wave * 32 + c;
   bf16x8 qf[KSTEPS];
@@ -72,6 +78,7 @@ __device__ __forceinline__ void attn_fwd_bf16_body(const AttnParams& p) {
     u32x4 z = {0, 0, 0, 0};
     const uint32_t col = 16 * ks + 8 * h;
     if (qrow < p.nq && col < p.d) z = ldg128(Q + (size_t)qrow * p.d + col);
+    z ^= sign_flip;
     qf[ks] = __builtin_bit_cast(bf16x8, z);
   }
 
@@ -80,7 +87,7 @@ __device__ __forceinline__ void attn_fwd_bf16_body(const AttnParams& p) {
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[t][i] = 0.0f;
-  float m_run = -INFINITY;  // running max of the raw scores (scale > 0)
+  float m_run = -INFINITY;  // running max of the raw scores
   float l_run = 0.0f;       // running sum over this half-wave's keys
 
   u32x4 kreg[K_ITERS];
@@ -180,8 +187,9 @@ __device__ __forceinline__ void attn_fwd_bf16_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
     mx = fmaxf(mx, xhalf(mx));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = fast_exp2((m_run - m_new) * p.scale_log2);  // exp-shift correction
-    const float mb = m_new * p.scale_log2;
+    // exp-shift correction; the first tile (m_run = -inf) contributes nothing to rescale
+    const float alpha = m_run == -INFINITY ? 0.0f : fast_exp2((m_run - m_new) * scale_log2);
+    const float mb = m_new * scale_log2;
     m_run = m_new;
 
     // ---- P = exp(S - m), running sum with correction
@@ -190,7 +198,7 @@ __device__ __forceinline__ void attn_fwd_bf16_body(const AttnParams& p) {
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float e = fast_exp2(__builtin_fmaf(s[kt][i], p.scale_log2, -mb));
+        const float e = fast_exp2(__builtin_fmaf(s[kt][i], scale_log2, -mb));
         s[kt][i] = e;
         psum += e;
       }

@@ -41,12 +41,16 @@ __device__ __forceinline__ void attn_fwd_f32_body(const AttnParams& p) {
   const float* __restrict__ K = reinterpret_cast<const float*>(p.k) + (size_t)head * p.nk * p.d;
   const float* __restrict__ V = reinterpret_cast<const float*>(p.v) + (size_t)head * p.nk * p.dv;
 
+  const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
+  const float qsign = scale_raw < 0.0f ? -1.0f : 1.0f;  // negative scale folded into Q
+  const float scale_log2 = fabsf(scale_raw) * I_LOG2_E32;
+
   const uint32_t qrow = qt * BM + wave * 32 + c;
   float qf[KSTEPS];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
     const uint32_t col = 2 * ks + h;
-    qf[ks] = (qrow < p.nq && col < p.d) ? Q[(size_t)qrow * p.d + col] : 0.0f;
+    qf[ks] = (qrow < p.nq && col < p.d) ? qsign * Q[(size_t)qrow * p.d + col] : 0.0f;
   }
 
   f32x16 o[DT];
@@ -97,8 +101,8 @@ __device__ __forceinline__ void attn_fwd_f32_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
     mx = fmaxf(mx, xhalf(mx));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = fast_exp2((m_run - m_new) * p.scale_log2);
-    const float mb = m_new * p.scale_log2;
+    const float alpha = m_run == -INFINITY ? 0.0f : fast_exp2((m_run - m_new) * scale_log2);
+    const float mb = m_new * scale_log2;
     m_run = m_new;
 
     float psum = 0.0f;
@@ -106,7 +110,7 @@ __device__ __forceinline__ void attn_fwd_f32_body(const AttnParams& p) {
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float e = fast_exp2(__builtin_fmaf(s[kt][i], p.scale_log2, -mb));
+        const float e = fast_exp2(__builtin_fmaf(s[kt][i], scale_log2, -mb));
         s[kt][i] = e;
         psum += e;
       }

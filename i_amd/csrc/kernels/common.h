@@ -36,6 +36,12 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 __device__ __forceinline__ u32x4 ldg128(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 
+// Effective score scale in the log2 domain.  exp is spelled pow(2.71828175f, x)
+// by the reference, i.e. exp2(x * I_LOG2_E32).
+__device__ __forceinline__ float load_scale(const float* ptr, float value) {
+  return (ptr ? *ptr : 1.0f) * value;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.
 // Map the linear workgroup id so that ids sharing an XCD walk consecutive
 // tiles of one `group` (e.g. one attention head, whose K/V then stay in that

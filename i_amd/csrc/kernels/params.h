@@ -13,7 +13,9 @@ struct AttnParams {
   uint32_t bh, nq, nk, d, dv;
   uint32_t nqt;        // query tiles per head
   uint32_t out_bf16;   // 0: f32 output, 1: bf16 output
-  float scale_log2;    // score scale * log2(2.71828175f); scale > 0
+  // score scale = scale_value * (scale_ptr ? *scale_ptr : 1), any finite value
+  const float* scale_ptr;  // optional rank-0 f32 operand in device memory
+  float scale_value;
 };
 
 struct GemmParams {

@@ -8,23 +8,22 @@
 
 namespace ihip {
 namespace {
-constexpr float kLog2E32 = 1.44269499718f;  // log2(2.71828175f)
 constexpr size_t kMaxGrid = 0x7fffffffu;
 
 bool fits_u32(size_t v) { return v <= 0xffffffffull; }
 }  // namespace
 
-bool attention_supported(DType in_dtype, size_t d, size_t dv, float scale) {
-  if (!(scale > 0.0f) || !std::isfinite(scale)) return false;
+bool attention_supported(DType in_dtype, size_t d, size_t dv) {
   if (d == 0 || dv == 0 || d > 128 || dv > 128) return false;
   if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
   return true;
 }
 
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
-                     size_t nq, size_t nk, size_t d, size_t dv, float scale, hipStream_t stream) {
-  if (!attention_supported(in_dtype, d, dv, scale))
-    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, scale > 0; bf16 needs d, dv % 8 == 0)";
+                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream) {
+  if (!attention_supported(in_dtype, d, dv))
+    return "attention kernel: unsupported operands (need 0 < d, dv <= 128; bf16 needs d, dv % 8 == 0)";
+  if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
   if (in_dtype == F32 && out_dtype != F32) return "attention kernel: f32 inputs produce f32 output";
   if (bh == 0 || nq == 0) return {};
   if (nk == 0) return "attention kernel: no keys";
@@ -38,7 +37,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.bh = (uint32_t)bh; p.nq = (uint32_t)nq; p.nk = (uint32_t)nk; p.d = (uint32_t)d; p.dv = (uint32_t)dv;
   p.nqt = (uint32_t)((nq + bm - 1) / bm);
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
-  p.scale_log2 = scale * kLog2E32;
+  p.scale_ptr = scale_ptr;
+  p.scale_value = scale;
 
   const char* name;
   if (in_dtype == BF16) name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";

@@ -10,11 +10,12 @@ namespace ihip {
 
 enum DType { F32 = 0, BF16 = 1 };
 
-// o[bh,nq,dv] = softmax(scale * q[bh,nq,d] k[bh,nk,d]^T) v[bh,nk,dv]
+// o[bh,nq,dv] = softmax(s * q[bh,nq,d] k[bh,nk,d]^T) v[bh,nk,dv],  s = scale * (scale_ptr ? *scale_ptr : 1)
 // in_dtype applies to q, k, v; out_dtype to o (F32 or BF16; BF16 only with bf16 inputs).
+// scale_ptr, when given, is a rank-0 f32 operand in device memory, read by the kernel.
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
-                     size_t nq, size_t nk, size_t d, size_t dv, float scale, hipStream_t stream);
-bool attention_supported(DType in_dtype, size_t d, size_t dv, float scale);
+                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream);
+bool attention_supported(DType in_dtype, size_t d, size_t dv);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,n,k]^T, a and b bf16
 Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,

@@ -7,6 +7,8 @@
  * (compiler/src/backends/c/stmt.rs:36-41).  The entry points below are the
  * GPU counterparts of those two things and do not change any i.h signature:
  *
+ *   i_exec_into_device  run a compiled program on device-resident operands,
+ *            f32 or bf16, asynchronously on a stream.
  *   i_hip_*  kernel launchers: the hand-written kernels a compiled program
  *            dispatches to, callable directly on device memory (the `fK`
  *            level of the generated-library ABI, ABI.md:4-9).
@@ -23,15 +25,40 @@
 extern "C" {
 #endif
 
+#include "i.h"
+
 enum { I_DTYPE_F32 = 0, I_DTYPE_BF16 = 1 };
+
+/* A dense row-major tensor in DEVICE memory: the device-side twin of
+ * i_tensor / i_tensor_mut (core/i.h:8-18) plus an element type tag. */
+typedef struct {
+  void* data;
+  const size_t* shape;
+  size_t rank;
+  int dtype; /* I_DTYPE_* */
+} i_device_tensor;
+
+/*
+ * i_exec_into for operands that already live on the GPU (reference host form:
+ * core/src/lib.rs:200-225).  Enqueues the whole program on `stream` and returns
+ * without waiting; temporaries are stream-ordered allocations.  Rank-0 operands
+ * (scalars) must be f32.  bf16 operands select the bf16-in / f32-accumulate
+ * kernels where a kernel has one and are widened on the device otherwise;
+ * each output is written in its own dtype.  Output shapes, when given
+ * (rank > 0), are checked against i_output_shapes.
+ */
+int i_exec_into_device(const i_program* program,
+                       const i_device_tensor* inputs, size_t input_count,
+                       const i_device_tensor* outputs, size_t output_count,
+                       void* stream);
 
 /*
  * FlashAttention forward,  o = softmax(scale * q k^T) v  per (batch*head):
  * the fused kernel for  mm_t >> [scale] >> row_max_shift >> exp >> row_normalize >> mm
  * (reference emission of the same component: ilang-python/annotated-flashattn.c:52-310,
  * `f0`).  q [bh,nq,d], k [bh,nk,d], v [bh,nk,dv], o [bh,nq,dv], row-major.
- * in_dtype applies to q/k/v, out_dtype to o.  Requires 0 < d,dv <= 128, scale > 0,
- * and d,dv multiples of 8 for bf16.
+ * in_dtype applies to q/k/v, out_dtype to o.  Requires 0 < d,dv <= 128, a finite
+ * scale, and d,dv multiples of 8 for bf16.
  */
 int i_hip_attention(const void* q, const void* k, const void* v, void* o,
                     int in_dtype, int out_dtype,

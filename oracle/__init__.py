@@ -182,3 +182,69 @@ def bf16_bits(x):
     """uint16 bf16 bit patterns of f32 values that are already bf16-representable."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     return (x.view(np.uint32) >> 16).astype(np.uint16).reshape(x.shape)
+
+
+# ---------------------------------------------------------------- C text backend (arbitrary components)
+_CB = HERE / "liboracle_cbackend.so"
+_cb = None
+
+
+def _cbackend():
+    global _cb
+    if _cb is None:
+        if not _CB.exists():
+            build()
+        _cb = ctypes.CDLL(str(_CB))
+        _cb.oracle_emit_c.restype = ctypes.c_void_p
+        _cb.oracle_emit_c.argtypes = [ctypes.c_void_p]
+        _cb.oracle_c_error.restype = ctypes.c_char_p
+    return _cb
+
+
+def emit_c(component_ptr):
+    """C source the reference C backend would print for a component handle
+    (an ``i_component*`` made through libi_core's i_parse / combinators)."""
+    lib_ = _cbackend()
+    raw = lib_.oracle_emit_c(component_ptr)
+    if not raw:
+        raise RuntimeError(lib_.oracle_c_error().decode())
+    try:
+        return ctypes.cast(raw, ctypes.c_char_p).value.decode()
+    finally:
+        ctypes.CDLL(None).free(ctypes.c_void_p(raw))
+
+
+class CProgram:
+    """Emitted C compiled the reference's way (cc -O3 -shared -fPIC -lm,
+    core/src/lib.rs:400-406) and driven through count/ranks/shapes/exec."""
+
+    def __init__(self, source):
+        import tempfile
+
+        self.source = source
+        self._dir = tempfile.TemporaryDirectory(prefix="ilang_oracle_")
+        c_path = Path(self._dir.name) / "prog.c"
+        so_path = Path(self._dir.name) / "prog.so"
+        c_path.write_text(source)
+        subprocess.run(["cc", "-O3", "-shared", "-fPIC", str(c_path), "-o", str(so_path), "-lm"], check=True)
+        self._lib = ctypes.CDLL(str(so_path))
+        self._lib.count.restype = _sz
+
+    def run(self, *inputs):
+        arrs = [_c(a) for a in inputs]
+        shapes = [(_sz * max(a.ndim, 1))(*a.shape) for a in arrs]
+        ins = (_Tensor * len(arrs))(*[_Tensor(_p(a), s, a.ndim) for a, s in zip(arrs, shapes)])
+        n = self._lib.count()
+        ranks = (_sz * n)()
+        self._lib.ranks(ranks)
+        oshapes = [(_sz * max(ranks[i], 1))() for i in range(n)]
+        optrs = (ctypes.POINTER(_sz) * n)(*[ctypes.cast(s, ctypes.POINTER(_sz)) for s in oshapes])
+        self._lib.shapes(ins, optrs)
+        outs = [np.full(tuple(oshapes[i][d] for d in range(ranks[i])), 123.0, dtype=np.float32) for i in range(n)]
+        otens = (_Tensor * n)(*[_Tensor(_p(o), s, ranks[i]) for i, (o, s) in enumerate(zip(outs, oshapes))])
+        self._lib.exec(ins, otens)
+        return outs[0] if n == 1 else tuple(outs)
+
+
+def compile_component(component_ptr):
+    return CProgram(emit_c(component_ptr))
