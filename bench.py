@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the north-star path on one MI355X.
+
+One step = one forward pass of the 𝚒 FlashAttention component
+(mm_t >> scale >> row_max_shift >> exp >> row_normalize >> mm), compiled from
+its expression strings through i_parse/i_compile and run with
+i_exec_into_device on operands resident in HBM: B=8, H=32, N=4096, d=128,
+bf16 inputs, f32 accumulation, f32 output, scores scaled by 1/sqrt(d).
+
+Prints ONE JSON line.  Besides the headline TFLOP/s it carries
+  roofline      achieved vs MI355X dense bf16 MFMA peak for the attention kernel,
+                from HIP events recorded on the launch stream
+  cpu_baseline  the CPU oracle (scalar port of the reference C backend's loop
+                nest) timed on one host core on a bounded sample
+  secondary     row-softmax [16384,4096] f32 (HBM bound) and mm_t 4096^3 bf16
+"""
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def flash_component(i, I, split):
+    mm_t = i(f"bhik*bhjk~bhijk | {split} | bhjii'j'k") >> i(f"+bhijk~bhij | {split} | bhjii'j'k0")
+    scale = i(f"bhij*.~bhij | {split} | bhji0i'j'")
+    row_max_shift = (I & i(f">bhij~bhi | {split} | bhji0i'j'")) >> i(f"bhij-bhi~bhij | {split} | bhji01i'j'")
+    exp = i(f"^bhij~bhij | {split} | bhji0i'j'")
+    row_normalize = (I & i(f"+bhij~bhi | {split} | bhji0i'j'")) >> i(f"bhij/bhi~bhij | {split} | bhji01i'j'")
+    mm = i(f"bhij*bhjk~bhikj | {split} | bhji0i'kj'") >> i(f"+bhikj~bhik | {split} | bhjii'kj'0")
+    return mm_t >> scale >> row_max_shift >> exp >> row_normalize >> mm
+
+
+def softmax_component(i, I):
+    # row-staged single-kernel schedule: max and sum fold to scalars, the row stays on chip
+    return (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
+            >> ((I & i("+ij~i|i:16|ii'0j")) >> i("ij/i~ij|i:16|ii'01j")))
+
+
+def mm_t_component(i):
+    return i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")
+
+
+def time_steps(torch, fn, steps, warmup):
+    """Wall time over exactly `steps` calls plus per-launch durations from events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s in range(steps):
+        starts[s].record()
+        fn()
+        ends[s].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    kernel_ms = sum(a.elapsed_time(b) for a, b in zip(starts, ends)) / steps
+    return wall_ms, kernel_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import numpy as np
+    import torch
+
+    from i_amd import Component as i, I
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    B, H, N, D = 8, 32, 4096, 128
+    gen = torch.Generator(device=dev).manual_seed(1)
+    q, k, v = (torch.randn(B, H, N, D, device=dev, generator=gen).bfloat16() for _ in range(3))
+    scale = torch.tensor(1.0 / np.sqrt(D), dtype=torch.float32, device=dev)
+    out = torch.empty(B, H, N, D, dtype=torch.float32, device=dev)
+    attn = flash_component(i, I, "i:128,j:64")
+    attn.into(out, q, k, scale, v)  # compile + first run outside the timed region
+    wall_ms, kernel_ms = time_steps(torch, lambda: attn.into(out, q, k, scale, v), args.steps, args.warmup)
+    flop = 4.0 * B * H * N * N * D
+    tflops = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (kernel_ms * 1e-3) / 1e12
+
+    # ---- secondary: row softmax (HBM bound) and mm_t (MFMA bound)
+    rows, cols = 16384, 4096
+    x = torch.randn(rows, cols, device=dev, generator=gen)
+    y = torch.empty_like(x)
+    sm = softmax_component(i, I)
+    sm.into(y, x)
+    _, sm_ms = time_steps(torch, lambda: sm.into(y, x), max(args.steps, 20), args.warmup)
+    sm_bytes = 2.0 * rows * cols * 4
+    sm_gbs = sm_bytes / (sm_ms * 1e-3) / 1e9
+
+    M = 4096
+    a = (torch.rand(M, M, device=dev, generator=gen) * 2 - 1).bfloat16()
+    b = (torch.rand(M, M, device=dev, generator=gen) * 2 - 1).bfloat16()
+    c = torch.empty(M, M, device=dev)
+    mm = mm_t_component(i)
+    mm.into(c, a, b)
+    _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), max(args.steps, 20), args.warmup)
+    mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
+
+    # ---- CPU baseline: the oracle on one host core, one (b, h) slice of the same workload
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+
+        qs, ks, vs = (t[0, 0].float().cpu().numpy() for t in (q, k, v))
+        t0 = time.perf_counter()
+        ref = oracle.attention_tiled(qs, ks, vs, float(scale), 16, 16)
+        cpu_s = time.perf_counter() - t0
+        got = out[0, 0].cpu().numpy()
+        rel = float(np.abs(got - ref).max() / np.abs(ref).max())
+        cpu = {
+            "value": 4.0 * N * N * D / cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"one (b,h) slice of the workload (N={N}, d={D}; 1 of {B * H}), {cpu_s:.1f} s; "
+                      f"GPU vs oracle on that slice: rel err {rel:.1e}",
+        }
+
+    line = {
+        "metric": "attn TFLOP/s & %MFMA peak (B8,H32,N4096,d128); row-softmax HBM GB/s",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "flash_attention_fwd B8 H32 N4096 d128, bf16 in / f32 accumulate / f32 out, "
+                               "1/sqrt(d) scale, non-causal (BASELINE configs[3]); compiled from 𝚒 component strings",
+                   "schedule": "i:128,j:64", "entry": "i_exec_into_device"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "attn_fwd_bf16_d128_bn64", "kernel_ms": kernel_ms},
+        "cpu_baseline": cpu,
+        "secondary": [
+            {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1])", "value": sm_gbs, "unit": "GB/s",
+             "roofline": {"bound": "hbm", "achieved": sm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                          "frac": sm_gbs / PEAK_HBM_GBS, "traffic": None, "kernel": "row_softmax_wave_v16",
+                          "kernel_ms": sm_ms}},
+            {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
+             "roofline": {"bound": "mfma", "achieved": mm_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "gemm_nt_bf16_128x128x64",
+                          "kernel_ms": mm_ms}},
+        ],
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -114,6 +114,19 @@ __device__ __forceinline__ void attn_fwd_f32_body(const AttnParams& p) {
         s[kt][i] = e;
         psum += e;
       }
+    // keys past nk take no weight (spelled out rather than left to exp(-inf): a zero scale
+    // turns the masked score into 0 * inf)
+    if (key0 + BN > p.nk) {
+      psum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t key = key0 + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
+          if (key >= p.nk) s[kt][i] = 0.0f;
+          psum += s[kt][i];
+        }
+    }
     l_run = l_run * alpha + psum;
 
 #pragma unroll

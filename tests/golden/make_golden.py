@@ -51,6 +51,18 @@ def main():
     np.savez_compressed(Path(__file__).with_name("flashattn_ref.npz"), **blobs)
     print("wrote", len(CASES), "cases")
 
+    # checksum of the reference's emitted C for the demo component, comments and
+    # whitespace removed: pins the whole lowering pipeline + C printer byte for byte
+    import hashlib
+    import re
+
+    text = Path("/root/reference/ilang-python/annotated-flashattn.c").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    text = re.sub(r"\s+", "", text)
+    Path(__file__).with_name("flashattn_emitted.sha256").write_text(
+        f"{hashlib.sha256(text.encode()).hexdigest()}  {len(text)}\n")
+
 
 if __name__ == "__main__":
     main()

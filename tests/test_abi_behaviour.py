@@ -1,0 +1,115 @@
+"""Behaviour of the C ABI that needs no GPU: handle ownership, NULL handling and
+error reporting as in the reference runtime (core/src/lib.rs:61-351), shape
+queries, and loud failure when no device can run the program."""
+import ctypes
+import threading
+
+import numpy as np
+import pytest
+
+from i_amd import Component as i, I
+from i_amd import _native as nat
+from i_amd import ilang
+
+core = nat.core
+
+
+def test_null_handles_report_reference_errors():
+    assert not core.i_chain(None, I._ptr) and nat.last_error() == "null left component"
+    assert not core.i_chain(I._ptr, None) and nat.last_error() == "null right component"
+    assert not core.i_swap(None) and nat.last_error() == "null component"
+    assert not core.i_code(None) and nat.last_error() == "null component"
+    assert not core.i_compile(None) and nat.last_error() == "null component"
+    assert core.i_output_count(None) == 0 and nat.last_error() == "null program"
+    assert core.i_output_ranks(None, None) == -1 and nat.last_error() == "null program"
+    assert core.i_exec_into(None, None, 0, None, 0) == -1 and nat.last_error() == "null program"
+    out = core.i_exec(None, None, 0)
+    assert out.count == 0 and not out.tensors and nat.last_error() == "null program"
+    # frees accept NULL
+    core.i_component_free(None)
+    core.i_program_free(None)
+    core.i_string_free(None)
+    core.i_outputs_free(ilang._COutputs(None, 0))
+
+
+def test_error_is_thread_local_and_sticky():
+    assert not core.i_swap(None)
+    assert nat.last_error() == "null component"
+    assert i("ij~ij")._ptr  # success does not clear the slot
+    assert nat.last_error() == "null component"
+    seen = {}
+
+    def other():
+        err = core.i_error()
+        seen["fresh"] = err
+        core.i_swap(None)
+        seen["after"] = core.i_error()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["fresh"] is None and seen["after"] == b"null component"
+
+
+def test_combinators_clone_operands():
+    a, b = i("ij~ij"), i("+ij~i")
+    c = a >> b
+    del a, b  # operands freed; the combined tree must stay valid
+    assert "1 kernel(s)" in c._code() or "2 kernel(s)" in c._code()
+
+
+def test_output_shapes_and_ranks_without_running():
+    mm = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    a, b = np.zeros((33, 20), np.float32), np.zeros((17, 20), np.float32)
+    assert mm.output_shapes(a, b) == [(33, 17)]
+    two = i("+ij~i") & i(">ij~j")
+    assert two.output_shapes(np.zeros((4, 9), np.float32)) == [(4,), (9,)]
+    assert (~two).output_shapes(np.zeros((4, 9), np.float32)) == [(9,), (4,)]
+    scalar = i("+ij~.")
+    assert scalar.output_shapes(np.zeros((4, 9), np.float32)) == [()]
+
+
+def test_output_shapes_rejects_low_rank_inputs():
+    mm = i("ik*kj~ijk") >> i("+ijk~ij")
+    with pytest.raises(RuntimeError) as err:
+        mm.output_shapes(np.zeros((4,), np.float32), np.zeros((4, 3), np.float32))
+    assert "rank" in str(err.value)
+
+
+def test_exec_into_checks_output_count_before_touching_the_device():
+    prog = i("+ij~i")
+    program = prog._compile()
+    x = np.zeros((4, 9), np.float32)
+    arr, keep = ilang._inputs([x])
+    assert core.i_exec_into(program, arr, 1, None, 0) == -1
+    assert nat.last_error() == "wrong output count"
+    assert core.i_exec_into(program, None, 1, None, 1) == -1
+    assert nat.last_error() == "null inputs"
+    assert core.i_exec_into(program, arr, 1, None, 1) == -1
+    assert nat.last_error() == "null outputs"
+
+
+def test_identity_program_is_rejected_like_the_reference():
+    # a program output that is a program input has no kernel to produce it
+    with pytest.raises(RuntimeError) as err:
+        I._compile()
+    assert "output 0 references Input buffer 0" in str(err.value)
+
+
+def test_no_device_fails_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    x = np.ones((4, 9), np.float32)
+    with pytest.raises(RuntimeError) as err:
+        i("+ij~i").exec_numpy(x)
+    assert "hip" in str(err.value).lower()
+    with pytest.raises(RuntimeError):
+        i("+ij~i").exec(x.tolist())
+
+
+def test_generated_source_builds_for_gfx950_without_a_gpu():
+    # i_compile runs hipcc for kernels that have no hand-written form
+    prog = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")
+    assert prog._compile()

@@ -1,0 +1,324 @@
+"""End-to-end through the drop-in boundary on the GPU: component strings ->
+i_parse / combinators -> i_compile -> i_exec / i_exec_into / i_exec_into_device.
+
+The cases are the reference's own integration tests (ilang-python/test.py:131-150,
+ilang-python/flash-attn.py:31-77) plus the BASELINE configurations, each
+checked against the CPU oracle: the emitted C of the same component where the
+oracle finishes in seconds, oracle.c / NumPy closed forms otherwise.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from i_amd import Component as i, I, Tensor
+
+pytestmark = pytest.mark.gpu
+RTOL_F32, RTOL_BF16 = 1e-4, 2e-2
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+
+    assert torch.cuda.is_available()
+    return torch
+
+
+def rnd(shape, seed):
+    return np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+
+
+def close(got, ref, rtol):
+    got, ref = np.asarray(got), np.asarray(ref)
+    assert got.shape == ref.shape and np.isfinite(got).all()
+    scale = max(float(np.abs(ref).max()), 1e-30)
+    assert float(np.abs(got - ref).max()) / scale <= rtol
+    return True
+
+
+def as_numpy(t):
+    return np.asarray(t.data, dtype=np.float32).reshape(t.shape)
+
+
+def flash(split="i:16,j:16", prefix="", scaled=False):
+    p = prefix
+    mm_t = i(f"{p}ik*{p}jk~{p}ijk | {split} | {p}jii'j'k") >> i(f"+{p}ijk~{p}ij | {split} | {p}jii'j'k0")
+    row_max_shift = (I & i(f">{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij-{p}i~{p}ij | {split} | {p}ji01i'j'")
+    exp = i(f"^{p}ij~{p}ij | {split} | {p}ji0i'j'")
+    row_normalize = (I & i(f"+{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij/{p}i~{p}ij | {split} | {p}ji01i'j'")
+    mm = i(f"{p}ij*{p}jk~{p}ikj | {split} | {p}ji0i'kj'") >> i(f"+{p}ikj~{p}ik | {split} | {p}jii'kj'0")
+    if scaled:
+        return mm_t >> i(f"{p}ij*.~{p}ij | {split} | {p}ji0i'j'") >> row_max_shift >> exp >> row_normalize >> mm
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
+def naive(split="i:16,j:16"):
+    mm_t = i(f"ik*jk~ijk | {split} | jii'j'k") >> i(f"+ijk~ij | {split} | jii'j'k0")
+    row_max_shift = (I & i(f">ij~i | {split} | jii'j'")) >> i(f"ij-i~ij | {split} | 1jii'j'")
+    exp = i(f"^ij~ij | {split} | jii'j'")
+    row_normalize = (I & i(f"+ij~i | {split} | jii'j'")) >> i(f"ij/i~ij | {split} | 1jii'j'")
+    mm = i(f"ij*jk~ikj | {split} | jii'kj'") >> i(f"+ikj~ik | {split} | jii'kj'0")
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
+def softmax_rowstaged():
+    return (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
+            >> ((I & i("+ij~i|i:16|ii'0j")) >> i("ij/i~ij|i:16|ii'01j")))
+
+
+def softmax_naive():
+    s = "i:16,j:16"
+    return (((I & i(f">ij~i|{s}|jii'j'")) >> i(f"ij-i~ij|{s}|1jii'j'")) >> i(f"^ij~ij|{s}|jii'j'")
+            >> ((I & i(f"+ij~i|{s}|jii'j'")) >> i(f"ij/i~ij|{s}|1jii'j'")))
+
+
+# ------------------------------------------------------------------ the reference's test.py cases (Tensor in, Tensor out)
+def test_reference_matmul_case(torch):
+    a, b = rnd((8, 16), 1), rnd((16, 7), 2)
+    f = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")
+    got = as_numpy(f.exec(Tensor(a.tolist()), Tensor(b.tolist())))
+    assert np.allclose(got, a @ b, rtol=1e-5, atol=1e-6)
+
+
+def test_reference_batched_attention_case(torch):
+    q, k, v = rnd((2, 3, 4, 8), 1), rnd((2, 3, 4, 8), 2), rnd((2, 3, 4, 8), 3)
+    mm_t = i("bhij*bhkj~bhikj | i:16,k:16 | bhkii'k'j") >> i("+bhikj~bhik | i:16,k:16 | bhkii'k'j0")
+    row_max_shift = (I & i(">bhik~bhi | i:16,k:16 | bhkii'k'")) >> i("bhik-bhi~bhik | i:16,k:16 | bh1kii'k'")
+    exp = i("^bhik~bhik | i:16,k:16 | bhkii'k'")
+    row_normalize = (I & i("+bhik~bhi | i:16,k:16 | bhkii'k'")) >> i("bhik/bhi~bhik | i:16,k:16 | bh1kii'k'")
+    mm = i("bhik*bhkj~bhijk | i:16,k:16 | bhkii'jk'") >> i("+bhijk~bhij | i:16,k:16 | bhkii'jk'0")
+    attn = mm_t >> row_max_shift >> exp >> row_normalize >> mm
+    got = as_numpy(attn.exec(*(Tensor(x.tolist()) for x in (q, k, v))))
+    assert np.allclose(got, oracle.np_attention64(q, k, v), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("src,fn", [(">ij~i", np.max), ("<ij~i", np.min), ("+ij~i", np.sum)])
+def test_reference_row_reductions(torch, src, fn):
+    x = rnd((16, 8), 1)
+    got = as_numpy(i(src).exec(Tensor(x.tolist())))
+    assert np.allclose(got, fn(x, axis=1), rtol=1e-5, atol=1e-6)
+
+
+def test_reference_mlp_case_with_pair(torch):
+    # test.py's mlp spells the pairing with an operator the frontend lacks; `|` is the pair combinator
+    x, w1, w2 = rnd((8,), 1), rnd((16, 8), 2), rnd((7, 16), 3)
+    mvp = i("ij*j~ij") >> i("+ij~i")
+    amvp = mvp >> i(">i~i")
+    f = (i("ij~ij") | amvp) >> mvp
+    got = as_numpy(f.exec(*(Tensor(t.tolist()) for t in (w2, w1, x))))
+    assert np.allclose(got, w2 @ np.maximum(w1 @ x, 0), rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------ flash-attn.py
+def test_reference_demo_flash_and_naive_attention(torch):
+    q, k, v = rnd((32, 2048), 1), rnd((32, 2048), 2), rnd((32, 2048), 3)
+    ref = oracle.np_attention64(q, k, v)
+    for comp in (flash(), naive()):
+        got = comp.exec_numpy(q, k, v)
+        assert np.allclose(got, ref, rtol=3e-4, atol=5e-5, equal_nan=True)  # the demo's own tolerance
+
+
+# ------------------------------------------------------------------ BASELINE config 1
+@pytest.mark.parametrize("split", ["i:16,j:16", "i:32,j:8", "i:128,j:64"])
+def test_config1_demo_attention_f32_vs_emitted_c(torch, split):
+    q, k, v = (np.random.default_rng(s).uniform(-1, 1, (512, 64)).astype(np.float32) for s in (1, 2, 3))
+    comp = flash(split)
+    ref = oracle.compile_component(comp._ptr).run(q, k, v)  # the C the reference backend would emit for these strings
+    close(comp.exec_numpy(q, k, v), ref, RTOL_F32)
+    close(comp.exec_torch(*(torch.from_numpy(a) for a in (q, k, v))).numpy(), ref, RTOL_F32)
+
+
+def test_config1_golden_reference_outputs(torch, golden):
+    comp = flash()
+    for case in ("u_48x24", "u_64x64", "u_100x40", "n_48x24", "n_33x17", "n_16x130"):
+        q, k, v, o = (golden[f"{case}.{x}"] for x in "qkvo")
+        close(comp.exec_numpy(q, k, v), o, RTOL_F32)
+
+
+def test_generated_and_hand_written_forms_agree(torch):
+    q, k, v = (np.random.default_rng(s).uniform(-1, 1, (200, 48)).astype(np.float32) for s in (1, 2, 3))
+    hand = flash().exec_numpy(q, k, v)
+    os.environ["ILANG_HIP_GENERATED_ONLY"] = "1"
+    try:
+        gen = flash().exec_numpy(q, k, v)
+        x = rnd((70, 300), 1)
+        sm_gen = softmax_rowstaged().exec_numpy(x)
+        a, b = rnd((50, 24), 1), rnd((30, 24), 2)
+        mm_gen = (i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")).exec_numpy(a, b)
+    finally:
+        del os.environ["ILANG_HIP_GENERATED_ONLY"]
+    ref = oracle.attention_tiled(q, k, v)
+    close(hand, ref, RTOL_F32)
+    close(gen, ref, RTOL_F32)
+    close(sm_gen, oracle.row_softmax(x), RTOL_F32)
+    close(mm_gen, oracle.mm_t(a, b), RTOL_F32)
+
+
+# ------------------------------------------------------------------ BASELINE config 2
+@pytest.mark.parametrize("comp_fn", [softmax_rowstaged, softmax_naive])
+def test_config2_row_softmax_small_vs_emitted_c(torch, comp_fn):
+    x = rnd((50, 70), 1)
+    comp = comp_fn()
+    close(comp.exec_numpy(x), oracle.compile_component(comp._ptr).run(x), RTOL_F32)
+
+
+def test_config2_row_softmax_full_size_device(torch):
+    x = rnd((16384, 4096), 1)
+    xd = torch.from_numpy(x).cuda()
+    y = softmax_rowstaged().exec_torch(xd)
+    assert (y.sum(dim=-1) - 1).abs().max().item() < 1e-4
+    rows = np.r_[0:8, 16376:16384]
+    close(y[rows].cpu().numpy(), oracle.row_softmax(x[rows]), RTOL_F32)
+
+
+# ------------------------------------------------------------------ BASELINE config 3
+def test_config3_mm_t_bf16_device(torch):
+    n = 4096
+    a = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (n, n)).astype(np.float32))
+    b = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (n, n)).astype(np.float32))
+    comp = i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")
+    c = comp.exec_torch(torch.from_numpy(a).cuda().bfloat16(), torch.from_numpy(b).cuda().bfloat16())
+    rows = np.r_[0:4, n - 4:n]
+    close(c[rows].cpu().numpy(), oracle.mm_t(a[rows], b), RTOL_BF16)
+    cols = np.r_[0:4, n - 4:n]
+    close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
+
+
+def test_mm_t_f32_small_vs_emitted_c(torch):
+    a, b = rnd((100, 40), 1), rnd((70, 40), 2)
+    comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
+
+
+# ------------------------------------------------------------------ BASELINE configs 4 and 5 (bf16 in, f32 accumulate)
+def test_config4_attention_slice_vs_oracle(torch):
+    """B8 H32 N4096 d128 recipe; two heads on the GPU, one (b,h) slice of query rows against the oracle."""
+    B, H, N, D = 1, 2, 4096, 128
+    q, k, v = (oracle.to_bf16_f32(rnd((B, H, N, D), s)) for s in (1, 2, 3))
+    scale = np.float32(1.0 / np.sqrt(D))
+    comp = flash("i:128,j:64", prefix="bh", scaled=True)
+    qd, kd, vd = (torch.from_numpy(a).cuda().bfloat16() for a in (q, k, v))
+    sd = torch.tensor(scale, device="cuda")
+    got = comp.exec_torch(qd, kd, sd, vd).cpu().numpy()
+    rows = np.r_[0:64, N - 64:N]
+    ref = oracle.attention_tiled(q[:, 1:2, rows], k[:, 1:2], v[:, 1:2], scale)
+    close(got[:, 1:2, rows], ref, RTOL_BF16)
+    got16 = comp.exec_torch(qd, kd, sd, vd, out_dtype=torch.bfloat16).float().cpu().numpy()
+    close(got16[:, 1:2, rows], ref, RTOL_BF16)
+
+
+def test_config4_full_size_properties(torch):
+    B, H, N, D = 8, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k, v = (torch.randn(B, H, N, D, device="cuda", generator=g).bfloat16() for _ in range(3))
+    v[..., 5] = -0.75            # a constant column must come out constant: rows are convex combinations
+    q[3, 7], k[3, 7], v[3, 7] = q[0, 1], k[0, 1], v[0, 1]
+    sd = torch.tensor(D ** -0.5, device="cuda")
+    out = flash("i:128,j:64", prefix="bh", scaled=True).exec_torch(q, k, sd, v)
+    assert out.shape == (B, H, N, D) and torch.isfinite(out).all()
+    assert (out[..., 5] + 0.75).abs().max().item() < 1e-2
+    assert torch.equal(out[3, 7], out[0, 1])
+    assert (out <= v.float().amax(dim=2, keepdim=True) + 1e-3).all()
+
+
+def test_config5_long_sequence_slice_vs_oracle(torch):
+    """B1 H16 N32768 d64, inputs x2.0: full length on the GPU, a few query rows against the oracle."""
+    N, D = 32768, 64
+    q, k, v = (oracle.to_bf16_f32(rnd((1, 1, N, D), s) * 2.0) for s in (1, 2, 3))
+    scale = np.float32(1.0 / np.sqrt(D))
+    comp = flash("i:128,j:64", prefix="bh", scaled=True)
+    got = comp.exec_torch(*(torch.from_numpy(a).cuda().bfloat16() for a in (q, k)), torch.tensor(scale, device="cuda"),
+                          torch.from_numpy(v).cuda().bfloat16()).cpu().numpy()
+    rows = np.r_[0:16, N - 16:N]
+    ref = oracle.attention_tiled(q[:, :, rows], k, v, scale)
+    close(got[:, :, rows], ref, RTOL_BF16)
+
+
+def test_rescale_stress_max_in_last_tile(torch):
+    # every key tile raises the running max of every row
+    nq, nk, d = 100, 700, 16
+    q = np.ones((nq, d), np.float32)
+    k = (np.arange(nk, dtype=np.float32)[:, None] * np.ones((1, d), np.float32)) * 0.125
+    v = rnd((nk, d), 3)
+    close(flash().exec_numpy(q, k, v), oracle.attention_tiled(q, k, v), RTOL_F32)
+    qb, kb, vb = (torch.from_numpy(oracle.to_bf16_f32(a)).cuda().bfloat16() for a in (q, k, v))
+    ref = oracle.attention_tiled(*(oracle.to_bf16_f32(a) for a in (q, k, v)))
+    close(flash().exec_torch(qb, kb, vb).cpu().numpy(), ref, RTOL_BF16)
+
+
+# ------------------------------------------------------------------ edge cases and the ABI on a live device
+def test_multi_output_and_swap(torch):
+    x = rnd((9, 14), 1)
+    two = i("+ij~i") & i(">ij~j")
+    a, b = two.exec_numpy(x)
+    assert np.allclose(a, x.sum(1), rtol=1e-5, atol=1e-5) and np.array_equal(b, x.max(0))
+    b2, a2 = (~two).exec_numpy(x)
+    assert np.array_equal(b2, b) and np.array_equal(a2, a)
+
+
+def test_scalar_output_and_scalar_input(torch):
+    x = rnd((6, 11), 1)
+    assert np.allclose(i("+ij~.").exec_numpy(x), x.sum(dtype=np.float64), rtol=1e-5, atol=1e-5)
+    got = i("ij*.~ij").exec_numpy(x, np.array(2.5, np.float32))
+    assert np.array_equal(got, x * np.float32(2.5))
+
+
+def test_all_pointwise_ops(torch):
+    x, y = rnd((5, 7), 1), rnd((5, 7), 2)
+    ax, ay = np.abs(x) + 0.5, np.abs(y) + 0.5
+    cases = [("ij+ij~ij", x + y), ("ij*ij~ij", x * y), ("ij-ij~ij", x - y), ("ij/ij~ij", x / ay if False else None),
+             ("ij>ij~ij", np.maximum(x, y)), ("ij<ij~ij", np.minimum(x, y)), ("ij>>ij~ij", (x > y) * 1.0),
+             ("ij>=ij~ij", (x >= y) * 1.0), ("ij<<ij~ij", (x < y) * 1.0), ("ij<=ij~ij", (x <= y) * 1.0),
+             ("ij==ij~ij", (x == y) * 1.0), ("ij!=ij~ij", (x != y) * 1.0)]
+    for src, ref in cases:
+        if ref is not None:
+            assert np.allclose(i(src).exec_numpy(x, y), ref.astype(np.float32), rtol=1e-6, atol=0), src
+    assert np.allclose(i("ij/ij~ij").exec_numpy(x, ay), x / ay, rtol=1e-6)
+    assert np.allclose(i("ij^ij~ij").exec_numpy(ax, y), np.power(ax, y), rtol=1e-5)
+    bx, by = (x > 0) * 1.0, (y > 0) * 1.0
+    assert np.array_equal(i("ij&&ij~ij").exec_numpy(bx, by), np.logical_and(bx, by) * 1.0)
+    assert np.array_equal(i("ij||ij~ij").exec_numpy(bx, by), np.logical_or(bx, by) * 1.0)
+    assert np.array_equal(i("ij^^ij~ij").exec_numpy(bx, by), np.logical_xor(bx, by) * 1.0)
+    unary = [("-ij~ij", -x), ("/ij~ij", 1 / ax), (">ij~ij", np.maximum(x, 0)), ("<ij~ij", np.minimum(x, 0)),
+             ("^ij~ij", np.exp(x)), ("$ij~ij", np.log(ax)), ("!!ij~ij", (bx == 0) * 1.0), (">>ij~ij", (x > 0) * 1.0)]
+    for src, ref in unary:
+        arg = ax if src[0] in "/$" else bx if src.startswith("!!") else x
+        assert np.allclose(i(src).exec_numpy(arg), ref.astype(np.float32), rtol=1e-5, atol=1e-6), src
+
+
+def test_empty_and_ragged_extents(torch):
+    mm = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    assert mm.exec_numpy(np.zeros((0, 5), np.float32), np.zeros((3, 5), np.float32)).shape == (0, 3)
+    a, b = rnd((1, 1), 1), rnd((1, 1), 2)
+    assert np.allclose(mm.exec_numpy(a, b), a @ b.T)
+    q, k, v = rnd((17, 3), 1), rnd((1, 3), 2), rnd((1, 5), 3)
+    close(flash().exec_numpy(q, k, v), np.broadcast_to(v, (17, 5)), RTOL_F32)  # one key: output is that value row
+
+
+def test_exec_rejects_wrong_rank_and_missing_inputs(torch):
+    mm = i("ik*kj~ijk") >> i("+ijk~ij")
+    with pytest.raises(RuntimeError):
+        mm.exec_numpy(np.zeros((4,), np.float32), np.zeros((4, 3), np.float32))
+    with pytest.raises(RuntimeError):
+        mm.exec_numpy(np.zeros((4, 4), np.float32))
+
+
+def test_device_entry_is_stream_ordered_and_repeatable(torch):
+    x = torch.randn(64, 256, device="cuda")
+    sm = softmax_naive()  # three generated kernels with two stream-ordered intermediates
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        outs = [sm.exec_torch(x) for _ in range(5)]
+    side.synchronize()
+    ref = torch.softmax(x, -1)
+    for o in outs:
+        assert (o - ref).abs().max().item() < 1e-5
+
+
+def test_non_f32_host_inputs_are_converted_like_the_reference(torch):
+    x = np.arange(12, dtype=np.int64).reshape(3, 4)
+    assert np.array_equal(i("+ij~i").exec_numpy(x), x.sum(1).astype(np.float32))
+    xt = np.asfortranarray(rnd((5, 6), 1))
+    assert np.allclose(i("+ij~i").exec_numpy(xt), xt.sum(1), rtol=1e-5, atol=1e-6)

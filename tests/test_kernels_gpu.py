@@ -157,8 +157,21 @@ def test_attention_rejects_unsupported(env):
                                       1.0, env.stream())
     assert rc == -1 and "unsupported" in env.nat.last_error()
     rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 0, 0, 1, 8, 8, 64, 64,
-                                      -1.0, env.stream())
-    assert rc == -1
+                                      float("inf"), env.stream())
+    assert rc == -1 and "scale" in env.nat.last_error()
+    rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, 60, 60,
+                                      1.0, env.stream())
+    assert rc == -1  # bf16 rows must be 16-byte multiples
+
+
+def test_attention_negative_and_zero_scale(env):
+    q, k, v = rnd((2, 70, 32), 1), rnd((2, 90, 32), 2), rnd((2, 90, 32), 3)
+    for scale in (-0.4, 0.0):
+        ref = oracle.np_attention64(q, k, v, scale).astype(np.float32)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=False), ref, RTOL_F32)
+    qb, kb, vb = (oracle.to_bf16_f32(a) for a in (q, k, v))
+    ref = oracle.np_attention64(qb, kb, vb, -0.4).astype(np.float32)
+    assert_close(gpu_attention(env, qb, kb, vb, -0.4, bf16=True), ref, RTOL_BF16)
 
 
 # ------------------------------------------------------------------ mm_t
