@@ -23,6 +23,29 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Exchange a value between lane l and lane l^32.
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
+// Both half-waves' copies of a value: after the call lo = x[lane & 31], hi = x[(lane & 31) + 32]
+// in every lane.  v_permlane32_swap exchanges the upper half of its first register with the
+// lower half of its second.  It is issued as inline assembly on two registers that both hold x
+// (the compiler builtin mis-assigns the second result on this toolchain); the s_nop cover the
+// VALU-write -> permlane read wait states the compiler would otherwise insert itself.
+__device__ __forceinline__ void both_halves(float x, float& lo, float& hi) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  lo = a;
+  hi = b;
+}
+// max / sum of a value over the two half-waves (lanes l and l^32), result in both.
+__device__ __forceinline__ float half_max(float x) {
+  float lo, hi;
+  both_halves(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_sum(float x) {
+  float lo, hi;
+  both_halves(x, lo, hi);
+  return lo + hi;
+}
+
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));

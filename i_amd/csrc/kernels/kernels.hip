@@ -6,9 +6,13 @@
 #include "gemm_nt_bf16.h"
 #include "row_softmax.h"
 
-#define ATTN_BF16(DPAD, BN, NW, OCC)                                                          \
-  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN(AttnParams p) { \
-    attn_fwd_bf16_body<DPAD, BN, NW>(p);                                                      \
+// attn_fwd_bf16_d<D>_bn<BN>: d == dv == D exactly; ..._any: d, dv <= D (multiples of 8), guarded columns
+#define ATTN_BF16(DPAD, BN, NW, OCC)                                                                          \
+  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN(AttnParams p) {   \
+    attn_fwd_bf16_body<DPAD, BN, NW, true>(p);                                                                \
+  }                                                                                                           \
+  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN##_any(AttnParams p) { \
+    attn_fwd_bf16_body<DPAD, BN, NW, false>(p);                                                               \
   }
 ATTN_BF16(64, 64, 4, 2)
 ATTN_BF16(128, 64, 4, 2)

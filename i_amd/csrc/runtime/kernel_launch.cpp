@@ -41,7 +41,10 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.scale_value = scale;
 
   const char* name;
-  if (in_dtype == BF16) name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
+  if (in_dtype == BF16) {
+    if (d == dv && (d == 64 || d == 128)) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
+    else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
+  }
   else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
 
   const size_t groups = (bh + 7) / 8 * 8;  // heads padded to the XCD count
