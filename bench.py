@@ -147,7 +147,7 @@ def main():
                    "schedule": "i:128,j:64", "entry": "i_exec_into_device"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
-                     "kernel": "attn_fwd_bf16_d128_bn64", "kernel_ms": kernel_ms},
+                     "kernel": "attn_fwd_bf16_d128_bn64_direct_w8", "kernel_ms": kernel_ms},
         "cpu_baseline": cpu,
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1])", "value": sm_gbs, "unit": "GB/s",

@@ -1,0 +1,527 @@
+// FlashAttention forward, bf16 in / f32 accumulate, for d == dv == DPAD:
+// K and V tiles go from global memory straight into LDS (no register staging).
+//
+// Same mapping of work as attention_bf16.h (one query per lane, S^T = K Q^T,
+// O^T += V^T P^T, running max / sum with exp-shift corrections).  What differs
+// is how the K/V tiles reach the matrix cores:
+//
+//   global -> LDS   global_load_lds_dwordx4: every lane fetches 16 bytes and
+//                   the wave deposits them as one contiguous 1 KiB run of LDS.
+//                   A tile is a contiguous BN * 2*DPAD byte piece of K (or V),
+//                   so wave-load w of a tile fills LDS bytes [1024 w, 1024 w + 1024).
+//   swizzle         rows are 256 (DPAD 128) or 128 (DPAD 64) bytes, so unpadded
+//                   rows would collide in the banks.  The 16-byte chunk index is
+//                   XOR-ed with a function of the row, applied on the GLOBAL side
+//                   (a lane chooses which chunk it fetches for its fixed LDS slot):
+//                     K: chunk ^= (row / RPB) % CH          16 consecutive rows, same
+//                                                           chunk -> 16 different bank groups
+//                     V: chunk ^= 4 * ((row / RPB) % (CH/4)) 4 consecutive rows, same
+//                                                           64-byte group -> 4 different groups
+//                   (RPB = rows per 256 bytes, CH = chunks per row).
+//   LDS -> K operand  ds_read_b128 of row (32 kt + c), chunk (2 ks + h): the A operand of
+//                   v_mfma_f32_32x32x16_bf16 exactly as in attention_bf16.h.
+//   LDS -> V operand  V stays row-major [key][dv]; ds_read_b64_tr_b16 transposes while
+//                   reading.  Within a 16-lane block, lane 4j+q supplies the address of
+//                   V[kb + j][dv0 + 4q .. +4) and lane i receives V[kb + 0..3][dv0 + i].
+//                   Two such reads (kb = 16 s4 + 4 h and + 8) give the 8 keys that the
+//                   P^T B-operand (the S^T accumulator layout) holds in the same lane.
+//
+// The transfers cost neither vector registers nor LDS-write instructions.  They are
+// software-pipelined against the arithmetic: while the softmax of tile j runs on the
+// vector pipe, the scores of tile j+1 are computed on the matrix pipe, so K is consumed
+// one trip before V.  K(j+2) and V(j+1) are requested early in trip j, into the buffer
+// of K(j) and of V(j-1) (both last read before the barrier that opens the trip), and are
+// awaited (vmcnt(0) + barrier) at the end of the trip.  One barrier per tile.
+//
+// Other differences from attention_bf16.h:
+//   * the reference max of a row is only moved when the tile max exceeds it by more than
+//     2^8 in the exponent, so the correction pass over the O accumulators is rare;
+//   * the row sum is taken over the bf16-rounded probabilities with v_dot2c_f32_bf16
+//     (two terms per instruction), i.e. over exactly the weights the PV product uses.
+#pragma once
+#include <type_traits>
+
+#include "common.h"
+#include "params.h"
+
+// One 16-byte-per-lane global -> LDS transfer.  `lds_base` (wave-uniform) is where lane 0's
+// 16 bytes land; lane l lands at lds_base + 16 l.  `base` is wave-uniform, `voff` per lane.
+// The compiler is not told that LDS is written: completion is awaited explicitly with
+// dma_wait_all() before the barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(voff), "s"(base), "s"(lds_base)
+      : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// extra operand-fetch lead of the steady-state loop, in MFMA slots (see fast_step)
+#ifndef ATTN_XLEAD
+#define ATTN_XLEAD 1
+#endif
+
+template <int DPAD, int BN, int NWAVES>
+__device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
+  constexpr int BM = 32 * NWAVES;
+  constexpr int KSTEPS = DPAD / 16;       // k-steps of the QK^T contraction
+  constexpr int KT = BN / 32;             // 32-key accumulator tiles
+  constexpr int DT = DPAD / 32;           // 32-column output tiles
+  constexpr int RB = 2 * DPAD;            // bytes per K/V row
+  constexpr int CH = RB / 16;             // 16-byte chunks per row (= lanes per row of a wave-load)
+  constexpr int RPB = 256 / RB;           // rows per 256 bytes
+  constexpr int RPW = 64 / CH;            // rows per wave-load
+  constexpr int TILE_BYTES = BN * RB;
+  constexpr int WL = TILE_BYTES / 1024;   // wave-loads per tile
+  constexpr int WLW = WL / NWAVES;        // ... per wave
+  static_assert(RB == 128 || RB == 256, "row size");
+  static_assert(WL % NWAVES == 0 && WLW >= 1, "tile / wave shape");
+  __shared__ __attribute__((aligned(1024))) char smem[2][2][TILE_BYTES];  // [buffer][K, V]
+
+  uint32_t head, qt;
+  xcd_map(blockIdx.x, p.nqt, head, qt);
+  if (head >= p.bh) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31;  // query column within the wave / A-operand row
+  const int h = lane >> 5;  // half-wave
+  constexpr uint32_t d = DPAD;
+
+  const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)head * p.nq * d;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RB;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RB;
+
+  // A negative scale is folded into Q (sign flip is exact), so the running max
+  // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
+  const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
+  const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
+  const float scale_log2 = fabsf(scale_raw) * I_LOG2_E32;
+
+  // Q^T fragments (B operand): lane (c, h) holds q[row][16*ks + 8*h .. +8].
+  const uint32_t qrow = qt * BM + wave * 32 + c;
+  bf16x8 qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    u32x4 z = {0, 0, 0, 0};
+    if (qrow < p.nq) z = ldg128(Q + (size_t)qrow * d + 16 * ks + 8 * h);
+    z ^= sign_flip;
+    qf[ks] = __builtin_bit_cast(bf16x8, z);
+  }
+
+  f32x16 o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[t][i] = 0.0f;
+  float m_run = -INFINITY;  // running max of the raw scores
+  float l_run = 0.0f;       // running sum over this half-wave's keys
+
+  // ---- global -> LDS: this lane's slot in wave-load w is tile row w*RPW + lane/CH, chunk lane%CH
+  const uint32_t lrow = lane / CH, lch = lane % CH;
+  const uint32_t smem0 = lds_address(&smem[0][0][0]);
+
+  // For a full tile the per-lane part of the address is the same for every tile and every wave-load
+  // (the swizzle term does not depend on `it` because NWAVES * RPW rows is a multiple of the swizzle
+  // period); everything that varies is wave-uniform and is folded into the scalar base address.
+  static_assert((NWAVES * RPW / RPB) % CH == 0, "swizzle period");
+  const uint32_t lane_row = wave * RPW + lrow;
+  const uint32_t koff_lane = lrow * RB + 16 * (lch ^ ((lane_row / RPB) % CH));
+  const uint32_t voff_lane = lrow * RB + 16 * (lch ^ (4 * ((lane_row / RPB) % (CH / 4))));
+  // one wave-load of a full tile: `it` of K (want_k) or of V
+  auto request_full_one = [&](uint32_t tile, int buf, int it, auto want_k) {
+    const uint32_t w = wave + NWAVES * it;
+    const size_t byte0 = (size_t)tile * TILE_BYTES + w * 1024;
+    if constexpr (decltype(want_k)::value) dma16(K + byte0, koff_lane, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+    else dma16(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+  };
+
+  // PARTIAL: the tile runs past nk; rows past the end re-read the last row (their scores are masked).
+  auto request_tile = [&](uint32_t key0, int buf, auto partial_tag, auto want_k, auto want_v) {
+    constexpr bool PARTIAL = decltype(partial_tag)::value;
+#pragma unroll
+    for (int it = 0; it < WLW; ++it) {
+      const uint32_t w = wave + NWAVES * it;
+      const uint32_t row = w * RPW + lrow;  // row within the tile
+      const uint32_t kch = lch ^ ((row / RPB) % CH);
+      const uint32_t vch = lch ^ (4 * ((row / RPB) % (CH / 4)));
+      uint32_t key = key0 + row;
+      if constexpr (PARTIAL) key = key < p.nk ? key : p.nk - 1;
+      if constexpr (decltype(want_k)::value) dma16(K, key * RB + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+      if constexpr (decltype(want_v)::value) dma16(V, key * RB + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+    }
+  };
+
+  // ---- LDS -> operands: per-lane byte offsets inside a tile
+  // K: row c (+ 32 kt), chunk (2 ks + h) ^ fk, where fk depends on c only
+  const uint32_t fk = (c / RPB) % CH;
+  uint32_t kaddr[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) kaddr[ks] = c * RB + 16 * ((2 * ks + h) ^ fk);
+  // V: 16-lane block b = lane / 16 covers columns 16 (b & 1) .. +16 of a 32-column tile; lane 4 jj + q of
+  // the block points at key (4 h + jj), columns 4 q .. +4
+  const uint32_t blk = lane >> 4, jj = (lane >> 2) & 3, qq = lane & 3;
+  const uint32_t gv = 4 * (((4 * h + jj) / RPB) % (CH / 4));
+  uint32_t vaddr[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+    vaddr[t] = (4 * h + jj) * RB + 16 * (((4 * t) ^ gv) + 2 * (blk & 1) + (qq >> 1)) + 8 * (qq & 1);
+
+  const f32x16 zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+  // ---- S^T = K_tile * Q^T for the K tile in buffer kbuf
+  auto qk = [&](f32x16 (&s)[KT], int kbuf) {
+    const char* sk = &smem[kbuf][0][0];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        bf16x8 a = *reinterpret_cast<const bf16x8*>(sk + 32 * kt * RB + kaddr[ks]);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], ks == 0 ? zero16 : s[kt], 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- running max / sum with exp-shift correction, then O^T += V_tile^T * P^T (V tile in buffer vbuf).
+  // The reference max is moved only when a row's tile max exceeds it by more than 2^RESCALE_LOG2 in the
+  // exponent: until then P = exp(S - m_run) is at most 2^RESCALE_LOG2, well inside f32 / bf16 range, and
+  // sum and output stay consistently scaled, so the normalised result is the same while the correction
+  // pass over the O accumulators is skipped for almost every tile.
+  constexpr float RESCALE_LOG2 = 8.0f;
+  auto softmax_pv = [&](f32x16 (&s)[KT], uint32_t j, int vbuf, bool masked) {
+    if (masked) {  // tail guard: keys past nk do not take part in the max
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t key = j * BN + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
+          if (key >= p.nk) s[kt][i] = -INFINITY;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
+    mx = half_max(mx);
+    // the first tile (m_run = -inf) always sets the reference; written so that a zero scale (inf * 0) is covered
+    const bool first = m_run == -INFINITY;
+    const bool move = first || (mx - m_run) * scale_log2 > RESCALE_LOG2;
+    const float m_new = move ? mx : m_run;
+    const float alpha = first ? 0.0f : fast_exp2((m_run - m_new) * scale_log2);  // 1 when the reference stays
+    const float mb = m_new * scale_log2;
+    m_run = m_new;
+
+    // P = exp(S - m) rounded to bf16 (the PV operand); the row sum is taken over the rounded values
+    bf16x8 pb[KT][2];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float e = fast_exp2(__builtin_fmaf(s[kt][i], scale_log2, -mb));
+        if (masked) {
+          // spelled out rather than left to exp(-inf): a zero scale turns the masked score into 0 * inf
+          const uint32_t key = j * BN + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
+          if (key >= p.nk) e = 0.0f;
+        }
+        pb[kt][i >> 3][i & 7] = (bf16_t)e;
+      }
+    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+    float psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          psum[w] = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[kt][u][2 * w], pb[kt][u][2 * w + 1]}, ones, psum[w], false);
+      }
+    l_run = l_run * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
+
+    // O correction (skipped unless some row of this wave moved its reference)
+    if (__builtin_amdgcn_ballot_w64(move)) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+    }
+
+    const char* sv = &smem[vbuf][1][0];
+#pragma unroll
+    for (int s4 = 0; s4 < BN / 16; ++s4) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        const char* va = sv + 16 * s4 * RB + vaddr[t];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * RB));
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb[s4 >> 1][s4 & 1], o[t], 0,
+                                                       0, 0);
+      }
+    }
+  };
+
+  using No = std::integral_constant<bool, false>;
+  using Yes = std::integral_constant<bool, true>;
+  const uint32_t ntiles = (p.nk + BN - 1) / BN;
+  const uint32_t nfull = p.nk / BN;  // tiles that lie entirely inside nk
+
+  // Software pipeline: the scores of tile j+1 are computed (matrix pipe) in the same iteration as the
+  // softmax of tile j (vector pipe).  K is therefore consumed one iteration before V: K(j+2) and V(j+1)
+  // are requested at the top of iteration j, into the buffers of K(j) (last read in iteration j-1) and of
+  // V(j-1) (last read in iteration j-1); one wait + barrier per iteration publishes both.
+  auto request_k = [&](uint32_t t, int buf) {
+    if (t < nfull) request_tile(t * BN, buf, No{}, Yes{}, No{});
+    else request_tile(t * BN, buf, Yes{}, Yes{}, No{});
+  };
+  auto request_v = [&](uint32_t t, int buf) {
+    if (t < nfull) request_tile(t * BN, buf, No{}, No{}, Yes{});
+    else request_tile(t * BN, buf, Yes{}, No{}, Yes{});
+  };
+
+  request_k(0, 0);
+  request_v(0, 0);
+  if (ntiles > 1) request_k(1, 1);
+  dma_wait_all();
+  __syncthreads();
+  f32x16 sa[KT], sb[KT];
+  qk(sa, 0);
+
+  // Steady state (tiles j, j+1, j+2 are all full tiles).  One trip runs from barrier to barrier and is
+  // written as NQK + NPV MFMA slots, everything else dealt out between the MFMAs a few vector
+  // instructions per slot, so that the matrix pipe and the vector pipe of the SIMD are fed by the same
+  // wave at the same time.  A scheduling fence after every slot keeps this order:
+  //   DT slots       last 16-key group of O += V(j-1)^T P(j-1)^T, operands and probabilities carried in
+  //                  registers across the barrier; carry the global -> LDS requests for K(j+2), V(j+1)
+  //   NQK slots      S(j+1) = K(j+1) Q^T; carry the rest of the requests and the first PQK pairs of
+  //                  P(j) = exp(S(j) - m)
+  //   NPV - DT slots O += V(j)^T P(j)^T for all but the last 16-key group; carry the remaining pairs of
+  //                  P(j) (each before the slot that needs its group) and the row max of S(j+1)
+  // LDS operands are fetched in slot order, DT + ATTN_XLEAD slots ahead of their MFMA; the fetches for
+  // the carried group are the last ones before the barrier, so the barrier sits in the middle of a
+  // stream of MFMAs instead of at a point where the matrix pipe has drained.
+  constexpr int NQK = KSTEPS * KT;      // MFMAs of the score tile
+  constexpr int NPV = (BN / 16) * DT;   // MFMAs of the output update
+  constexpr int NSLOT = NQK + NPV;
+  constexpr int NPAIR = KT * 8;         // score pairs per lane; pairs 4 g .. 4 g + 3 are the 16-key group g
+  constexpr int PQK = 10;               // pairs exponentiated during the QK slots
+  constexpr int NMAIN = NPV - DT;       // PV slots of the trip that owns the tile
+  constexpr int MAXSLOTS = NPV / 2;     // PV slots that carry the row max (the last ones before the barrier)
+  constexpr int EPS = KT * 16 / MAXSLOTS;  // scores folded into the max per such slot
+  constexpr int XLEAD = ATTN_XLEAD;
+  static_assert(NPAIR == 16 && (KT * 16) % MAXSLOTS == 0 && 2 * WLW <= DT + NQK && NPAIR - PQK <= NMAIN &&
+                    MAXSLOTS <= NMAIN && XLEAD >= 0 && XLEAD < NQK,
+                "slot shape");
+  // pair PQK + m is produced in main PV slot m and first used in main PV slot ((PQK + m) / 4) * DT
+  // (the last group is used by the carried slots of the next trip): every pair must be ready in time
+  constexpr bool pairs_in_time = [] {
+    for (int m = 0; m < NPAIR - PQK; ++m)
+      if ((PQK + m) / 4 < NPAIR / 4 - 1 && m >= ((PQK + m) / 4) * DT) return false;
+    return true;
+  }();
+  static_assert(pairs_in_time, "a probability pair would be produced after the MFMA that consumes it");
+
+  struct Carry {
+    bf16x8 a[DT];  // V^T operands of the last 16-key group
+    u32x4 p;       // its probabilities
+  };
+
+  auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], float& mx_tile,
+                       const Carry& cin, Carry& cout) {
+    const char* sk = &smem[buf ^ 1][0][0];  // K(j+1)
+    const char* sv = &smem[buf][1][0];      // V(j)
+
+    // operand k of this trip: K rows for k < NQK, transposed V columns after that
+    bf16x8 opnd[NSLOT];
+    auto fetch = [&](int k) {
+      if (k < NQK) {
+        const int ks = k / KT, kt = k % KT;
+        opnd[k] = *reinterpret_cast<const bf16x8*>(sk + 32 * kt * RB + kaddr[ks]);
+      } else {
+        const int s4 = (k - NQK) / DT, t = (k - NQK) % DT;
+        const char* va = sv + 16 * s4 * RB + vaddr[t];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * RB));
+        opnd[k] = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+    // slot g of the trip issues fetch g + XLEAD (slot 0 also issues 0 .. XLEAD - 1)
+    auto fetch_for_slot = [&](int g) {
+      if (g == 0) {
+#pragma unroll
+        for (int k = 0; k < XLEAD; ++k) fetch(k);
+      }
+      if (g + XLEAD < NSLOT) fetch(g + XLEAD);
+    };
+    // request r of the 2 WLW global -> LDS requests of the trip
+    auto request_for_slot = [&](int g) {
+      if (g < 2 * WLW) {
+        if (g < WLW) request_full_one(j + 2, buf, g, Yes{});
+        else request_full_one(j + 1, buf ^ 1, g - WLW, No{});
+      }
+    };
+
+    // packed probability pairs: pq[g][w] holds scores 2 (4 g + w), + 1 of the lane in (kt, i) order, so pq[g] is
+    // the B operand of 16-key group g.  The empty asm statements tie each slot's vector work to its slot.
+    u32x4 pq[NPAIR / 4];
+    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+    float psum[2] = {0.0f, 0.0f};
+    float mb = 0.0f, alpha = 1.0f;
+    bool move = false;
+    auto exp_pair = [&](int pr) {
+      const int pkt = pr / 8, i = 2 * (pr % 8);
+      const float e0 = fast_exp2(__builtin_fmaf(s_cur[pkt][i], scale_log2, -mb));
+      const float e1 = fast_exp2(__builtin_fmaf(s_cur[pkt][i + 1], scale_log2, -mb));
+      const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
+      psum[pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[pr & 1], false);
+      uint32_t packed = __builtin_bit_cast(uint32_t, pair);
+      asm volatile("" : "+v"(packed), "+v"(psum[pr & 1]));
+      pq[pr / 4][pr % 4] = packed;
+    };
+
+    // ---- carried slots: last key group of tile j-1
+#pragma unroll
+    for (int g = 0; g < DT; ++g) {
+      fetch_for_slot(g);
+      o[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cin.a[g], __builtin_bit_cast(bf16x8, cin.p), o[g], 0, 0, 0);
+      request_for_slot(g);
+      if (g == 0) {
+        // reference max for tile j (mx_tile = row max of S(j), found during the previous trip)
+        const bool first = m_run == -INFINITY;
+        move = first || (mx_tile - m_run) * scale_log2 > RESCALE_LOG2;
+        const float m_new = move ? mx_tile : m_run;
+        alpha = first ? 0.0f : fast_exp2((m_run - m_new) * scale_log2);
+        mb = m_new * scale_log2;
+        m_run = m_new;
+        asm volatile("" : "+v"(mb), "+v"(alpha));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- score slots of tile j+1
+#pragma unroll
+    for (int n = 0; n < NQK; ++n) {
+      fetch_for_slot(DT + n);
+      const int ks = n / KT, kt = n % KT;
+      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[ks], ks == 0 ? zero16 : s_next[kt], 0, 0, 0);
+      request_for_slot(DT + n);
+#pragma unroll
+      for (int pr = n * PQK / NQK; pr < (n + 1) * PQK / NQK; ++pr) exp_pair(pr);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // O correction for tile j (after the carried slots, which still belong to tile j-1)
+    if (__builtin_amdgcn_ballot_w64(move)) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- output slots of tile j, all key groups but the last
+    float mx = s_next[0][0];
+#pragma unroll
+    for (int m = 0; m < NMAIN; ++m) {
+      fetch_for_slot(DT + NQK + m);
+      const int s4 = m / DT, t = m % DT;
+      o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[NQK + m], __builtin_bit_cast(bf16x8, pq[s4]), o[t], 0, 0, 0);
+      if (m < NPAIR - PQK) exp_pair(PQK + m);
+      if (m >= NMAIN - MAXSLOTS) {
+#pragma unroll
+        for (int e = 0; e < EPS; ++e) {
+          const int idx = (m - (NMAIN - MAXSLOTS)) * EPS + e;
+          mx = fmaxf(mx, s_next[idx / 16][idx % 16]);
+        }
+        asm volatile("" : "+v"(mx));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    l_run = l_run * alpha + (psum[0] + psum[1]);
+    mx_tile = half_max(mx);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) cout.a[t] = opnd[NQK + NMAIN + t];
+    cout.p = pq[NPAIR / 4 - 1];
+    dma_wait_all();
+    __syncthreads();
+  };
+
+  float mx_tile = sa[0][0];
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
+  mx_tile = half_max(mx_tile);
+  uint32_t j = 0;
+  if (nfull >= 4) {
+    // the first trip has no predecessor: its carried slots add zero
+    Carry ca, cb;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) ca.a[t] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+    ca.p = u32x4{0, 0, 0, 0};
+    for (; j + 4 <= nfull; j += 2) {  // j + 3 <= nfull - 1
+      fast_step(j, 0, sa, sb, mx_tile, ca, cb);
+      fast_step(j + 1, 1, sb, sa, mx_tile, cb, ca);
+    }
+    // last key group of the last steady-state tile
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ca.a[t], __builtin_bit_cast(bf16x8, ca.p), o[t], 0, 0, 0);
+  }
+  // the last tiles (no successor, or a partial one): same steps with run-time conditions; sa holds S(j)
+  for (; j < ntiles; ++j) {
+    const int buf = j & 1;
+    if (j + 2 < ntiles) request_k(j + 2, buf);
+    if (j + 1 < ntiles) {
+      request_v(j + 1, buf ^ 1);
+      qk(sb, buf ^ 1);
+    }
+    softmax_pv(sa, j, buf, j >= nfull);
+    dma_wait_all();
+    __syncthreads();
+    if (j + 1 < ntiles) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) sa[kt] = sb[kt];
+    }
+  }
+
+  // ---- epilogue: normalise and store.  Lane (c, h) holds O[q = c][32 t + 8 g + 4 h + e].
+  const float inv = 1.0f / half_sum(l_run);
+  if (qrow < p.nq) {
+    if (p.out_bf16) {
+      bf16_t* O = reinterpret_cast<bf16_t*>(p.o) + ((size_t)head * p.nq + qrow) * d;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          bf16x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(o[t][4 * g + e] * inv);
+          *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+        }
+    } else {
+      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * d;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
+          *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+        }
+    }
+  }
+}

@@ -2,6 +2,7 @@
 // Every entry point is extern "C" so the host side can look it up by name with
 // hipModuleGetFunction; each takes one parameter block by value (params.h).
 #include "attention_bf16.h"
+#include "attention_bf16_direct.h"
 #include "attention_f32.h"
 #include "gemm_nt_bf16.h"
 #include "row_softmax.h"
@@ -16,6 +17,18 @@
   }
 ATTN_BF16(64, 64, 4, 2)
 ATTN_BF16(128, 64, 4, 2)
+
+// attn_fwd_bf16_d<D>_bn<BN>_direct: d == dv == D, K/V tiles loaded from global memory straight into LDS;
+// ..._w8: eight waves (256 queries) per workgroup, one workgroup per CU
+#define ATTN_BF16_DIRECT(DPAD, BN, NW, OCC)                                                                        \
+  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN##_direct(AttnParams p) { \
+    attn_fwd_bf16_direct_body<DPAD, BN, NW>(p);                                                                    \
+  }
+ATTN_BF16_DIRECT(64, 64, 4, 2)
+ATTN_BF16_DIRECT(128, 64, 4, 2)
+extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d128_bn64_direct_w8(AttnParams p) {
+  attn_fwd_bf16_direct_body<128, 64, 8>(p);
+}
 
 #define ATTN_F32(DPAD, BN, NW)                                                             \
   extern "C" __global__ void __launch_bounds__(NW * 64) attn_fwd_f32_d##DPAD##_bn##BN(AttnParams p) { \

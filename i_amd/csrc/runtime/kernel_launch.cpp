@@ -1,6 +1,7 @@
 #include "kernel_launch.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstdint>
 #include <string>
 
@@ -31,7 +32,24 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   if (!q || !k || !v || !o) return "attention kernel: null device pointer";
 
   const size_t dmax = d > dv ? d : dv;
-  const unsigned bm = 128;
+  // Kernel choice for bf16:
+  //   d == dv in {64, 128}: direct-to-LDS kernel; for d = 128 a 256-query workgroup (8 waves) halves the
+  //     L2 -> LDS traffic per query and is used when it still leaves at least two workgroups per CU
+  //   otherwise: register-staged kernel with guarded columns
+  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the d = 128 direct kernel and ILANG_ATTN_NO_DIRECT=1
+  // forces the register-staged kernel; both exist so that tests can reach every kernel with small inputs.
+  unsigned bm = 128;
+  const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
+  // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
+  const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+  if (direct && d == 128) {
+    if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
+    if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
+      const int waves = std::atoi(w);
+      if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8";
+      bm = 32u * (unsigned)waves;
+    }
+  }
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o;
   p.bh = (uint32_t)bh; p.nq = (uint32_t)nq; p.nk = (uint32_t)nk; p.d = (uint32_t)d; p.dv = (uint32_t)dv;
@@ -42,7 +60,9 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 
   const char* name;
   if (in_dtype == BF16) {
-    if (d == dv && (d == 64 || d == 128)) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
+    if (direct)
+      name = d == 64 ? "attn_fwd_bf16_d64_bn64_direct" : bm == 256 ? "attn_fwd_bf16_d128_bn64_direct_w8" : "attn_fwd_bf16_d128_bn64_direct";
+    else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   }
   else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
@@ -52,7 +72,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   if (grid > kMaxGrid) return "attention kernel: grid too large";
   hipFunction_t fn;
   if (Err e = builtin_function(name, &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+  return launch(fn, (unsigned)grid, 1, 1, 2 * bm, &p, sizeof(p), stream);
 }
 
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }

@@ -72,8 +72,10 @@ def test_output_shapes_and_ranks_without_running():
 def test_output_shapes_rejects_low_rank_inputs():
     mm = i("ik*kj~ijk") >> i("+ijk~ij")
     with pytest.raises(RuntimeError) as err:
-        mm.output_shapes(np.zeros((4,), np.float32), np.zeros((4, 3), np.float32))
+        mm.output_shapes(np.zeros((4, 3), np.float32), np.zeros((4,), np.float32))
     assert "rank" in str(err.value)
+    # like the reference's emitted `shapes`, only the dimensions an output is sized by are read
+    assert mm.output_shapes(np.zeros((4,), np.float32), np.zeros((4, 3), np.float32)) == [(4, 3)]
 
 
 def test_exec_into_checks_output_count_before_touching_the_device():

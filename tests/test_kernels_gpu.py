@@ -105,6 +105,64 @@ def test_attention_bf16_vs_oracle(env, bh, nq, nk, d):
     assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("force", [None, "waves8", "staged"])
+def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
+    """The launcher picks between the direct-to-LDS kernel (4 or 8 waves per workgroup) and the
+    register-staged kernel; force each of them on one ragged problem (7 full key tiles + a partial
+    one, so the steady-state loop, its drain and the masked tail all run)."""
+    if force == "waves8":
+        if d != 128:
+            pytest.skip("the 8-wave workgroup exists for d = 128 only")
+        monkeypatch.setenv("ILANG_ATTN_WAVES", "8")
+    elif force == "staged":
+        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+    bh, nq, nk = 2, 300, 450
+    q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    ref = oracle.attention_tiled(q, k, v, scale)
+    assert_close(gpu_attention(env, q, k, v, scale, bf16=True), ref, RTOL_BF16)
+    assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
+
+
+def test_attention_bf16_workgroup_sizes_agree_bitwise(env, monkeypatch):
+    """A wave does the same arithmetic whether its workgroup has 4 or 8 waves."""
+    bh, n, d = 16, 1024, 128
+    q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s in (1, 2, 3))
+    monkeypatch.setenv("ILANG_ATTN_WAVES", "4")
+    a = gpu_attention(env, q, k, v, 0.1, bf16=True)
+    monkeypatch.setenv("ILANG_ATTN_WAVES", "8")
+    b = gpu_attention(env, q, k, v, 0.1, bf16=True)
+    assert np.array_equal(a, b)
+    monkeypatch.setenv("ILANG_ATTN_WAVES", "3")
+    t = env.torch
+    x = t.zeros(1, 8, 128, device="cuda", dtype=t.bfloat16)
+    rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 1, 1, 8, 8, 128, 128,
+                                      1.0, env.stream())
+    assert rc == -1 and "ILANG_ATTN_WAVES" in env.nat.last_error()
+
+
+@pytest.mark.parametrize("span", [20.0, 45.0, 90.0])
+def test_attention_bf16_reference_max_moves_slowly_and_fast(env, span):
+    """Scores rise steadily along the keys by `span` nats in total over 10 tiles.  The direct kernel
+    moves a row's reference max only when a tile exceeds it by 2^8: span 20 never reaches that after
+    the first tile, 45 reaches it every other tile, 90 at every tile."""
+    nq, nk, d = 64, 640, 64
+    q = np.ones((1, nq, d), np.float32)
+    k = oracle.to_bf16_f32((np.arange(nk, dtype=np.float32)[None, :, None] * np.ones((1, 1, d), np.float32))
+                           * np.float32(span / (nk * d)))
+    v = oracle.to_bf16_f32(rnd((1, nk, d), 3))
+    ref = oracle.attention_tiled(q, k, v, 1.0)
+    assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
+
+
+def test_attention_bf16_direct_negative_and_zero_scale(env):
+    q, k, v = (oracle.to_bf16_f32(rnd((2, n, 64), s)) for s, n in ((1, 70), (2, 400), (3, 400)))
+    for scale in (-0.3, 0.0):
+        ref = oracle.np_attention64(q, k, v, scale).astype(np.float32)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True), ref, RTOL_BF16)
+
+
 def test_attention_bf16_config4_slice_vs_oracle(env):
     """One (b, h) slice of B8 H32 N4096 d128 at full sequence length, against the oracle on 256 query rows."""
     n, d = 4096, 128
