@@ -156,7 +156,7 @@ def main():
                           "kernel_ms": sm_ms}},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
              "roofline": {"bound": "mfma", "achieved": mm_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "gemm_nt_bf16_128x128x64",
+                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "gemm_nt_bf16_256x256x64_direct",
                           "kernel_ms": mm_ms}},
         ],
     }

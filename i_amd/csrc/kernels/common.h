@@ -75,3 +75,22 @@ __device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_
   group = (slot / per_group) * 8u + xcd;
   tile = slot % per_group;
 }
+
+// One 16-byte-per-lane global -> LDS transfer.  `lds_base` (wave-uniform) is where lane 0's
+// 16 bytes land; lane l lands at lds_base + 16 l.  `base` is wave-uniform, `voff` per lane.
+// The compiler is not told that LDS is written: completion is awaited explicitly with
+// dma_wait_all() before the barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(voff), "s"(base), "s"(lds_base)
+      : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}

@@ -1,0 +1,172 @@
+// C[m,n] = sum_k A[m,k] * B[n,k]  (bf16 in, f32 accumulate and f32 out) on gfx950,
+// large-tile form: a 256 x 256 output tile per workgroup, K in slabs of 64, operand
+// slabs moved from global memory straight into LDS.
+//
+// Device form of the fused 𝚒 nest  i("ik*jk~ijk") >> i("+ijk~ij ... k0")
+// (README.md:16; annotated-flashattn.c:57-89 shows the same pair with a tile-local
+// output): tile loops i, j -> workgroups, the k loop is sequential per workgroup,
+// i', j' -> MFMA lanes, and the product never exists outside a register.
+//
+//   workgroup   8 waves as 2 (m) x 4 (n); a wave owns 128 x 64 of the tile =
+//               4 x 2 accumulators of v_mfma_f32_32x32x16_bf16 (128 registers)
+//   slabs       A and B slabs are both [256 rows][64 k] bf16 = 128-byte rows.  One
+//               global_load_lds_dwordx4 of a wave deposits 8 rows (1 KiB) contiguously
+//               in LDS; the 16-byte chunk a lane fetches is XOR-ed with (row / 2) % 8 so
+//               that the 16 rows one quarter-wave reads for an MFMA operand fall into
+//               16 different bank groups.  Two slab buffers: slab s+1 is requested at the
+//               top of iteration s and awaited (vmcnt(0) + barrier) at its end.
+//   operands    both A rows and B rows are K-contiguous, so both MFMA operands are plain
+//               ds_read_b128 of (row, chunk 2 ks + h)
+//   L2          the workgroup ids that land on one XCD (id % 8) fill a block of 4 x 8
+//               tiles, so at any time an XCD streams 1024 rows of A and 2048 rows of B
+//   M, N edges  rows past the end re-read the last valid row and are not stored
+// Requires k % 64 == 0 (the launcher falls back to gemm_nt_bf16.h otherwise).
+#pragma once
+#include "common.h"
+#include "params.h"
+
+__device__ __forceinline__ void gemm_nt_bf16_direct_body(const GemmParams& p) {
+  constexpr int BMT = 256, BNT = 256, BK = 64;
+  constexpr int WM = 2, WN = 4, NWAVES = WM * WN;
+  constexpr int TM = BMT / WM / 32;  // 4
+  constexpr int TN = BNT / WN / 32;  // 2
+  constexpr int RB = 2 * BK;         // bytes per slab row
+  constexpr int CH = RB / 16;        // chunks per row (= lanes per row of a wave-load)
+  constexpr int RPW = 64 / CH;       // rows per wave-load
+  constexpr int SLAB = BMT * RB;     // bytes of one operand slab (BMT == BNT)
+  constexpr int WL = SLAB / 1024;    // wave-loads per slab
+  constexpr int WLW = WL / NWAVES;   // ... per wave
+  constexpr int KS = BK / 16;
+  static_assert(BMT == BNT && WL % NWAVES == 0, "slab shape");
+  __shared__ __attribute__((aligned(1024))) char smem[2][2][SLAB];  // [buffer][A, B]
+
+  // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
+  constexpr uint32_t SBM = 4, SBN = 8, SB = SBM * SBN;
+  const uint32_t nsb_m = (p.tiles_m + SBM - 1) / SBM, nsb_n = (p.tiles_n + SBN - 1) / SBN;
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t sb = (slot / SB) * 8u + xcd, within = slot % SB;
+  if (sb >= nsb_m * nsb_n) return;
+  const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
+  const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
+  if (tm >= p.tiles_m || tn >= p.tiles_n) return;
+  const uint32_t batch = blockIdx.y;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  const int c = lane & 31, h = lane >> 5;
+
+  const size_t row_bytes = (size_t)p.k * 2;
+  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
+  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;
+  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
+  const uint32_t m0 = tm * BMT, n0 = tn * BNT;
+
+  // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
+  // (row 8 w + lane / 8, chunk lane % 8) and it fetches chunk (lane % 8) ^ ((row / 2) % 8) of that row.
+  // w = wave + 8 it, so (row / 2) % 8 = (4 (wave % 2) + lane / 16) % 8 does not depend on `it`.
+  const uint32_t lrow = lane / CH, lch = lane % CH;
+  const uint32_t gch = lch ^ ((4 * (wave & 1) + lane / 16) % CH);
+  const uint32_t smem0 = lds_address(&smem[0][0][0]);
+  // per-lane byte offsets from the slab's first row of this wave-load; edge tiles clamp the row
+  uint32_t aoff[WLW], boff[WLW];
+#pragma unroll
+  for (int it = 0; it < WLW; ++it) {
+    const uint32_t r = (wave + NWAVES * it) * RPW + lrow;
+    const uint32_t ra = m0 + r < p.m ? m0 + r : p.m - 1;
+    const uint32_t rb = n0 + r < p.n ? n0 + r : p.n - 1;
+    aoff[it] = (ra - m0) * (uint32_t)row_bytes + 16 * gch;
+    boff[it] = (rb - n0) * (uint32_t)row_bytes + 16 * gch;
+  }
+  const char* a_tile = A + (size_t)m0 * row_bytes;
+  const char* b_tile = B + (size_t)n0 * row_bytes;
+  auto request_slab = [&](uint32_t s, int buf) {
+    const size_t k_byte = (size_t)s * RB;
+#pragma unroll
+    for (int it = 0; it < WLW; ++it) {
+      const uint32_t w = wave + NWAVES * it;
+      dma16(a_tile + k_byte, aoff[it], smem0 + (2 * buf + 0) * SLAB + w * 1024);
+      dma16(b_tile + k_byte, boff[it], smem0 + (2 * buf + 1) * SLAB + w * 1024);
+    }
+  };
+
+  // ---- LDS -> operands: row (32 i + c) of the wave's rows, chunk (2 ks + h) ^ ((row / 2) % 8)
+  const uint32_t fr = (c / 2) % CH;
+  uint32_t addr[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) addr[ks] = c * RB + 16 * ((2 * ks + h) ^ fr);
+  const uint32_t a_rows = wm * TM * 32 * RB, b_rows = wn * TN * 32 * RB;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const uint32_t nslabs = p.k / BK;
+  request_slab(0, 0);
+  dma_wait_all();
+  __syncthreads();
+
+  // One slab: 4 k-steps of 8 MFMAs.  The operands of k-step ks+1 are fetched while the MFMAs of k-step
+  // ks issue, and the requests for the next slab are dealt out one per MFMA; scheduling fences keep
+  // that order.  The first k-step's operands are fetched right after the barrier.
+  auto fetch = [&](const char* sa, const char* sb, int ks, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * RB + addr[ks]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bfr[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
+  };
+  auto step = [&](uint32_t s, int buf, bool more) {
+    const char* sa = &smem[buf][0][0] + a_rows;
+    const char* sb = &smem[buf][1][0] + b_rows;
+    const size_t k_byte = (size_t)(s + 1) * RB;
+    bf16x8 af[2][TM], bfr[2][TN];
+    fetch(sa, sb, 0, af[0], bfr[0]);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) fetch(sa, sb, ks + 1, af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+          const int slot = (ks * TM + i) * TN + j;  // 0 .. 31
+          if (more && slot % 2 == 0 && slot / 2 < 2 * WLW) {
+            const int r = slot / 2, it = r % WLW;
+            const uint32_t w = wave + NWAVES * it;
+            if (r < WLW) dma16(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024);
+            else dma16(b_tile + k_byte, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    dma_wait_all();
+    __syncthreads();
+  };
+  uint32_t s = 0;
+  for (; s + 3 <= nslabs; s += 2) {  // two per trip so that the buffer index is a constant
+    step(s, 0, true);
+    step(s + 1, 1, true);
+  }
+  for (; s < nslabs; ++s) step(s, s & 1, s + 1 < nslabs);
+
+  // ---- store.  Accumulator layout: column n = c, rows 8 (e / 4) + 4 h + e % 4: every store instruction
+  // writes two full 128-byte lines.  C is written once and not read again: non-temporal.
+  const bool interior = m0 + BMT <= p.m && n0 + BNT <= p.n;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + (wn * TN + j) * 32 + c;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+        if (interior || (row < p.m && col < p.n)) __builtin_nontemporal_store(acc[i][j][e], &C[(size_t)row * p.n + col]);
+      }
+    }
+}

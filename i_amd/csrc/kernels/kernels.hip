@@ -5,6 +5,7 @@
 #include "attention_bf16_direct.h"
 #include "attention_f32.h"
 #include "gemm_nt_bf16.h"
+#include "gemm_nt_bf16_direct.h"
 #include "row_softmax.h"
 
 // attn_fwd_bf16_d<D>_bn<BN>: d == dv == D exactly; ..._any: d, dv <= D (multiples of 8), guarded columns
@@ -40,6 +41,10 @@ ATTN_F32(128, 32, 4)
 
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64(GemmParams p) {
   gemm_nt_bf16_body<128, 128, 64, 2, 2>(p);
+}
+
+extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct(GemmParams p) {
+  gemm_nt_bf16_direct_body(p);
 }
 
 #define SOFTMAX_WAVE(NV)                                                                          \

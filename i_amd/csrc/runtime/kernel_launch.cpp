@@ -86,6 +86,25 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  // Large problems: 256 x 256 tiles with direct global -> LDS slabs (needs whole 64-wide k slabs and 32-bit
+  // byte offsets inside a tile's 256 rows).  Its prologue and its unoverlapped store only pay off for a long
+  // k loop on a grid that fills at least half of the CUs.  ILANG_GEMM_DIRECT=1 / 0 forces / forbids it, so
+  // that tests can reach both kernels at small sizes.
+  {
+    const size_t tm = (m + 255) / 256, tn = (n + 255) / 256;
+    bool direct = k >= 512 && tm * tn * bh >= 128;
+    if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) direct = f[0] == '1';
+    if (direct && k % 64 == 0 && k <= (size_t(1) << 22) && bh <= 65535) {
+      p.tiles_m = (uint32_t)tm;
+      p.tiles_n = (uint32_t)tn;
+      const size_t nsb = ((tm + 3) / 4) * ((tn + 7) / 8);  // super-blocks of 4 x 8 tiles, dealt to the 8 XCDs
+      const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+      if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
+      hipFunction_t fn;
+      if (Err e = builtin_function("gemm_nt_bf16_256x256x64_direct", &fn); !e.empty()) return e;
+      return launch(fn, (unsigned)grid, (unsigned)bh, 1, 512, &p, sizeof(p), stream);
+    }
+  }
   p.tiles_m = (uint32_t)((m + 127) / 128);
   p.tiles_n = (uint32_t)((n + 127) / 128);
   const size_t tiles = (size_t)p.tiles_m * p.tiles_n;

@@ -246,6 +246,23 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
     assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
+                                      (3, 257, 255, 320)])
+@pytest.mark.parametrize("direct", ["1", "0"])
+def test_gemm_nt_bf16_both_kernels_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
+    """The launcher picks the 256 x 256 direct-to-LDS kernel for long-k problems on big grids; force it (and
+    forbid it) on small ragged problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
+    t = env.torch
+    a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
+    ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+    cd = t.full((bh, m, n), float("nan"), device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nt_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+    t.cuda.synchronize()
+    assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
+
+
 def test_gemm_nt_bf16_full_size_linearity(env):
     """M=N=K=4096: C(A1+A2, B) == C(A1,B) + C(A2,B) for bf16-exact sums, and row block vs oracle."""
     t = env.torch
