@@ -12,10 +12,16 @@ Prints ONE JSON line.  Besides the headline TFLOP/s it carries
                 from HIP events recorded on the launch stream
   cpu_baseline  the CPU oracle (scalar port of the reference C backend's loop
                 nest) timed on one host core on a bounded sample
-  secondary     row-softmax [16384,4096] f32 (HBM bound) and mm_t 4096^3 bf16
+  secondary     row-softmax [16384,4096] f32 (HBM bound), mm_t 4096^3 bf16 and the
+                long-sequence attention B1 H16 N32768 d64 (inputs x 2.0)
+
+roofline.traffic is the HBM traffic per launch measured with rocprofv3
+(FETCH_SIZE + WRITE_SIZE passes, scaled by a plain copy of known size); it is read
+from the committed summary under profiles/ and is null when that is missing.
 """
 import argparse
 import json
+import re
 import sys
 import time
 from pathlib import Path
@@ -45,6 +51,16 @@ def softmax_component(i, I):
 
 def mm_t_component(i):
     return i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")
+
+
+def measured_traffic(summary):
+    """HBM bytes per launch from a committed rocprofv3 summary, or None."""
+    try:
+        text = (ROOT / "profiles" / summary).read_text()
+    except OSError:
+        return None
+    m = re.search(r"Scaled traffic per launch: (\d+) MiB fetched \+ (\d+) MiB written", text)
+    return (int(m.group(1)) + int(m.group(2))) * 2 ** 20 if m else None
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -115,6 +131,15 @@ def main():
     _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), max(args.steps, 20), args.warmup)
     mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
 
+    # long-sequence attention (heavy running-max movement): B1 H16 N32768 d64, inputs x 2.0
+    B5, H5, N5, D5 = 1, 16, 32768, 64
+    q5, k5, v5 = ((torch.randn(B5, H5, N5, D5, device=dev, generator=gen) * 2.0).bfloat16() for _ in range(3))
+    scale5 = torch.tensor(1.0 / np.sqrt(D5), dtype=torch.float32, device=dev)
+    out5 = torch.empty(B5, H5, N5, D5, dtype=torch.float32, device=dev)
+    attn.into(out5, q5, k5, scale5, v5)
+    _, c5_ms = time_steps(torch, lambda: attn.into(out5, q5, k5, scale5, v5), max(args.steps // 2, 5), 2)
+    c5_tflops = 4.0 * B5 * H5 * N5 * N5 * D5 / (c5_ms * 1e-3) / 1e12
+
     if args.calibrate_copy:
         y.copy_(x)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
@@ -146,18 +171,26 @@ def main():
                                "1/sqrt(d) scale, non-causal (BASELINE configs[3]); compiled from 𝚒 component strings",
                    "schedule": "i:128,j:64", "entry": "i_exec_into_device"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": measured_traffic("flash_attention_B8_H32_N4096_d128_bf16.md"),
                      "kernel": "attn_fwd_bf16_d128_bn64_direct_w8", "kernel_ms": kernel_ms},
         "cpu_baseline": cpu,
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1])", "value": sm_gbs, "unit": "GB/s",
              "roofline": {"bound": "hbm", "achieved": sm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                          "frac": sm_gbs / PEAK_HBM_GBS, "traffic": None, "kernel": "row_softmax_wave_v16",
+                          "frac": sm_gbs / PEAK_HBM_GBS, "traffic": measured_traffic("row_softmax_16384x4096_f32.md"),
+                          "kernel": "row_softmax_wave_v16",
                           "kernel_ms": sm_ms}},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
              "roofline": {"bound": "mfma", "achieved": mm_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "gemm_nt_bf16_256x256x64_direct",
-                          "kernel_ms": mm_ms}},
+                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("gemm_nt_4096x4096x4096_bf16.md"),
+                          "kernel": "gemm_nt_bf16_256x256x64_direct", "kernel_ms": mm_ms}},
+            {"workload": "flash_attention_fwd B1 H16 N32768 d64, bf16 inputs x 2.0 (BASELINE configs[4])",
+             "value": c5_tflops, "unit": "TFLOP/s",
+             "roofline": {"bound": "mfma", "achieved": c5_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                          "frac": c5_tflops / PEAK_BF16_TFLOPS,
+                          "traffic": measured_traffic("flash_attention_B1_H16_N32768_d64_bf16.md"),
+                          "kernel": "attn_fwd_bf16_d64_bn64_direct", "kernel_ms": c5_ms}},
         ],
     }
     print(json.dumps(line))
