@@ -188,7 +188,8 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
         return e;
       }
       return ihip::launch_attention(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), run.raw_ptr(r.c.buffer), out,
-                                    bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream);
+                                    bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream,
+                                    r.tile_i);
     }
     case Recognized::GemmNT: {
       const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
@@ -202,7 +203,7 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       void* out = nullptr;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
-                                       a[nb], b[nb], a[nb + 1], run.stream);
+                                       a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j);
     }
     case Recognized::RowSoftmax: {
       const auto x = run.shape_of(r.a.buffer);

@@ -255,9 +255,11 @@ struct Matcher {
 }  // namespace
 
 std::string Recognized::describe() const {
+  std::string tiles;
+  if (tile_i || tile_j) tiles = "; schedule tile " + std::to_string(tile_i) + " x " + std::to_string(tile_j);
   switch (kind) {
-    case Attention: return has_scale ? "hand-written FlashAttention kernel (scaled scores)" : "hand-written FlashAttention kernel";
-    case GemmNT: return "hand-written MFMA GEMM (transposed right operand)";
+    case Attention: return (has_scale ? "hand-written FlashAttention kernel (scaled scores)" : "hand-written FlashAttention kernel") + tiles;
+    case GemmNT: return "hand-written MFMA GEMM (transposed right operand)" + tiles;
     case RowSoftmax: return "hand-written row-softmax kernel";
     default: return "generated HIP kernel";
   }
@@ -284,7 +286,30 @@ std::vector<Recognized> recognize_kernels(const Lowered& low) {
     TreeBuilder tb{sp};
     const int root = tb.build(stage, {});
     Matcher m{tb, refs};
-    out.push_back(m.match_root(root, refs[sp.graph.inputs + stage]));
+    Recognized rec = m.match_root(root, refs[sp.graph.inputs + stage]);
+    if (rec.kind == Recognized::Attention || rec.kind == Recognized::GemmNT) {
+      // the schedule's tile sizes, read off the root stage: its output is [B.., I, E] (attention, J reduced)
+      // or [B.., I, J] (GEMM)
+      const Stage& st = sp.graph.nodes[stage].inner;
+      auto tile_of = [&](size_t index) -> size_t {
+        for (const SAxis& a : st.axes)
+          if (!a.pruned && a.index == index && a.kind.kind == ExtentKind::Base) {
+            size_t t = 1;
+            for (size_t f : a.kind.factors) t *= f;
+            return a.kind.factors.empty() ? 0 : t;
+          }
+        return 0;
+      };
+      const auto& shape = st.output.shape;
+      if (shape.size() >= 2) {
+        rec.tile_i = tile_of(shape[shape.size() - 2]);
+        if (rec.kind == Recognized::GemmNT) rec.tile_j = tile_of(shape.back());
+        else
+          for (const SAxis& a : st.axes)
+            if (std::find(shape.begin(), shape.end(), a.index) == shape.end()) rec.tile_j = tile_of(a.index);
+      }
+    }
+    out.push_back(rec);
   }
   return out;
 }

@@ -30,6 +30,9 @@ struct Recognized {
   Operand scale;               // rank-0 operand
   ic::BufferRef out;
   size_t batch_rank = 0;       // number of leading shared dims
+  // Tile sizes the schedule asks for (product of the split factors of the index in the kernel's root
+  // stage, 0 when the index is not split): Attention: query rows I / keys J; GemmNT: rows I / columns J.
+  size_t tile_i = 0, tile_j = 0;
   std::string describe() const;
 };
 

@@ -21,7 +21,8 @@ bool attention_supported(DType in_dtype, size_t d, size_t dv) {
 }
 
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
-                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream) {
+                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
+                     size_t query_tile) {
   if (!attention_supported(in_dtype, d, dv))
     return "attention kernel: unsupported operands (need 0 < d, dv <= 128; bf16 needs d, dv % 8 == 0)";
   if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
@@ -34,7 +35,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   const size_t dmax = d > dv ? d : dv;
   // Kernel choice for bf16:
   //   d == dv in {64, 128}: direct-to-LDS kernel; for d = 128 a 256-query workgroup (8 waves) halves the
-  //     L2 -> LDS traffic per query and is used when it still leaves at least two workgroups per CU
+  //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
+  //     larger workgroup is used when it still leaves at least two workgroups per CU
   //   otherwise: register-staged kernel with guarded columns
   // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the d = 128 direct kernel and ILANG_ATTN_NO_DIRECT=1
   // forces the register-staged kernel; both exist so that tests can reach every kernel with small inputs.
@@ -43,7 +45,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
   const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct && d == 128) {
-    if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
+    if (query_tile == 128 || query_tile == 256) bm = (unsigned)query_tile;  // the schedule's i split
+    else if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
       const int waves = std::atoi(w);
       if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8";
@@ -78,7 +81,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }
 
 Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream) {
+                        hipStream_t stream, size_t tile_m, size_t tile_n) {
   if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || !fits_u32(k) || !fits_u32(bh)) return "gemm_nt kernel: extent exceeds 32 bits";
@@ -93,6 +96,8 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   {
     const size_t tm = (m + 255) / 256, tn = (n + 255) / 256;
     bool direct = k >= 512 && tm * tn * bh >= 128;
+    if (tile_m == 256 && tile_n == 256) direct = true;   // the schedule's i, j splits
+    if (tile_m == 128 && tile_n == 128) direct = false;
     if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) direct = f[0] == '1';
     if (direct && k % 64 == 0 && k <= (size_t(1) << 22) && bh <= 65535) {
       p.tiles_m = (uint32_t)tm;

@@ -13,13 +13,19 @@ enum DType { F32 = 0, BF16 = 1 };
 // o[bh,nq,dv] = softmax(s * q[bh,nq,d] k[bh,nk,d]^T) v[bh,nk,dv],  s = scale * (scale_ptr ? *scale_ptr : 1)
 // in_dtype applies to q, k, v; out_dtype to o (F32 or BF16; BF16 only with bf16 inputs).
 // scale_ptr, when given, is a rank-0 f32 operand in device memory, read by the kernel.
+// query_tile is the query-row tile the schedule asks for (the product of the split factors of the row
+// index; 0 = no preference): 128 and 256 select the 4- and 8-wave workgroup of the d = 128 kernel, any other
+// value leaves the choice to the launcher.
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
-                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream);
+                     size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
+                     size_t query_tile = 0);
 bool attention_supported(DType in_dtype, size_t d, size_t dv);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,n,k]^T, a and b bf16
+// tile_m x tile_n is the output tile the schedule asks for (0 = no preference): 256 x 256 and 128 x 128 select
+// the kernel with that workgroup tile (when its requirements hold), anything else leaves the choice to the launcher.
 Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream);
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
 bool gemm_nt_bf16_supported(size_t k);
 
 // y[rows,cols] = row softmax of x, f32

@@ -402,11 +402,19 @@ def test_emitted_c_agrees_bit_for_bit_with_oracle_restatement():
 
 # ------------------------------------------------------------------ backend plan (what i_code reports)
 def test_plan_recognises_hot_path_kernels():
-    assert "f0: hand-written FlashAttention kernel [in0, in1, in2 -> out0]" in flash()._code()
+    # the plan also reports the tile sizes the schedule asks for (products of the split factors of the
+    # row index and of the key / column index); the launchers map 128 / 256 onto kernel variants
+    assert "f0: hand-written FlashAttention kernel; schedule tile 16 x 16 [in0, in1, in2 -> out0]" in flash()._code()
     mmt = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     assert "hand-written MFMA GEMM" in mmt._code()
+    big = i("ik*jk~ijk | i:256,j:256 | jii'j'k") >> i("+ijk~ij | i:256,j:256 | jii'j'k0")
+    assert "schedule tile 256 x 256" in big._code()
+    two_level = i("ik*jk~ijk | i:16:8,j:64 | jii'i''j'k") >> i("+ijk~ij | i:16:8,j:64 | jii'i''j'k0")
+    assert "schedule tile 128 x 64" in two_level._code()
+    unfused = i("ik*jk~ijk") >> i("+ijk~ij")  # no staging digit: two kernels with a full-size product, as in the reference
+    assert "2 kernel(s)" in unfused._code() and "hand-written" not in unfused._code()
     swapped = i("jk*ik~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
-    assert "hand-written MFMA GEMM (transposed right operand) [in1, in0 -> out0]" in swapped._code()
+    assert "hand-written MFMA GEMM (transposed right operand); schedule tile 16 x 16 [in1, in0 -> out0]" in swapped._code()
     sm = (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
           >> ((I & i("+ij~i|i:16|ii'0j")) >> i("ij/i~ij|i:16|ii'01j")))
     assert "hand-written row-softmax kernel [in0 -> out0]" in sm._code()

@@ -178,7 +178,7 @@ def test_config3_mm_t_bf16_device(torch):
     n = 4096
     a = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (n, n)).astype(np.float32))
     b = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (n, n)).astype(np.float32))
-    comp = i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")
+    comp = i("ik*jk~ijk | i:256,j:256 | jii'j'k") >> i("+ijk~ij | i:256,j:256 | jii'j'k0")
     c = comp.exec_torch(torch.from_numpy(a).cuda().bfloat16(), torch.from_numpy(b).cuda().bfloat16())
     rows = np.r_[0:4, n - 4:n]
     close(c[rows].cpu().numpy(), oracle.mm_t(a[rows], b), RTOL_BF16)
@@ -207,6 +207,24 @@ def test_config4_attention_slice_vs_oracle(torch):
     close(got[:, 1:2, rows], ref, RTOL_BF16)
     got16 = comp.exec_torch(qd, kd, sd, vd, out_dtype=torch.bfloat16).float().cpu().numpy()
     close(got16[:, 1:2, rows], ref, RTOL_BF16)
+
+
+def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
+    """The i split of the attention schedule picks the workgroup size (128 or 256 query rows) and the
+    i, j splits of mm_t pick the 128 x 128 or 256 x 256 kernel; the variants agree (attention bitwise)."""
+    B, H, N, D = 1, 4, 1024, 128
+    q, k, v = (torch.from_numpy(oracle.to_bf16_f32(rnd((B, H, N, D), s))).cuda().bfloat16() for s in (1, 2, 3))
+    sd = torch.tensor(np.float32(1.0 / np.sqrt(D)), device="cuda")
+    o128 = flash("i:128,j:64", prefix="bh", scaled=True).exec_torch(q, k, sd, v)
+    o256 = flash("i:256,j:64", prefix="bh", scaled=True).exec_torch(q, k, sd, v)
+    assert torch.equal(o128, o256)
+    a = torch.from_numpy(oracle.to_bf16_f32(rnd((512, 256), 1))).cuda().bfloat16()
+    b = torch.from_numpy(oracle.to_bf16_f32(rnd((300, 256), 2))).cuda().bfloat16()
+    c128 = (i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")).exec_torch(a, b)
+    c256 = (i("ik*jk~ijk | i:256,j:256 | jii'j'k") >> i("+ijk~ij | i:256,j:256 | jii'j'k0")).exec_torch(a, b)
+    ref = a.float() @ b.float().T
+    assert (c128 - ref).abs().max() <= 1e-3 * ref.abs().max()
+    assert (c256 - ref).abs().max() <= 1e-3 * ref.abs().max()
 
 
 def test_config4_full_size_properties(torch):
