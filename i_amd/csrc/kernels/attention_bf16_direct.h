@@ -105,6 +105,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     for (int i = 0; i < 16; ++i) o[t][i] = 0.0f;
   float m_run = -INFINITY;  // running max of the raw scores
   float l_run = 0.0f;       // running sum over this half-wave's keys
+  float mb_run = 0.0f;      // m_run * scale_log2, kept while the steady-state loop runs
 
   // ---- global -> LDS: this lane's slot in wave-load w is tile row w*RPW + lane/CH, chunk lane%CH
   const uint32_t lrow = lane / CH, lch = lane % CH;
@@ -319,6 +320,23 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     u32x4 p;       // its probabilities
   };
 
+  // Reference max of tile j (mx_tile = row max of S(j), found during the previous trip).  Runs between the
+  // carried slots, which still belong to tile j-1, and the first use of the reference for tile j.
+  auto move_reference = [&](float mx_tile) {
+    const bool move = __builtin_fmaf(mx_tile, scale_log2, -mb_run) > RESCALE_LOG2;
+    if (__builtin_amdgcn_ballot_w64(move)) {  // rare: some row of this wave moves its reference
+      const float m_new = move ? mx_tile : m_run;
+      const float alpha = fast_exp2((m_run - m_new) * scale_log2);  // 1 for the rows that stay
+      m_run = m_new;
+      mb_run = m_new * scale_log2;
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+    }
+  };
+
   auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], float& mx_tile,
                        const Carry& cin, Carry& cout) {
     const char* sk = &smem[buf ^ 1][0][0];  // K(j+1)
@@ -359,8 +377,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     u32x4 pq[NPAIR / 4];
     const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
     float psum[2] = {0.0f, 0.0f};
-    float mb = 0.0f, alpha = 1.0f;
-    bool move = false;
+    float mb = 0.0f;  // reference of tile j in the exponent domain, set after the carried slots
     auto exp_pair = [&](int pr) {
       const int pkt = pr / 8, i = 2 * (pr % 8);
       const float e0 = fast_exp2(__builtin_fmaf(s_cur[pkt][i], scale_log2, -mb));
@@ -378,18 +395,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       fetch_for_slot(g);
       o[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cin.a[g], __builtin_bit_cast(bf16x8, cin.p), o[g], 0, 0, 0);
       request_for_slot(g);
-      if (g == 0) {
-        // reference max for tile j (mx_tile = row max of S(j), found during the previous trip)
-        const bool first = m_run == -INFINITY;
-        move = first || (mx_tile - m_run) * scale_log2 > RESCALE_LOG2;
-        const float m_new = move ? mx_tile : m_run;
-        alpha = first ? 0.0f : fast_exp2((m_run - m_new) * scale_log2);
-        mb = m_new * scale_log2;
-        m_run = m_new;
-        asm volatile("" : "+v"(mb), "+v"(alpha));
-      }
       __builtin_amdgcn_sched_barrier(0);
     }
+    move_reference(mx_tile);
+    mb = mb_run;
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- score slots of tile j+1
 #pragma unroll
@@ -402,15 +412,6 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       for (int pr = n * PQK / NQK; pr < (n + 1) * PQK / NQK; ++pr) exp_pair(pr);
       __builtin_amdgcn_sched_barrier(0);
     }
-
-    // O correction for tile j (after the carried slots, which still belong to tile j-1)
-    if (__builtin_amdgcn_ballot_w64(move)) {
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
-    }
-    __builtin_amdgcn_sched_barrier(0);
 
     // ---- output slots of tile j, all key groups but the last
     float mx = s_next[0][0];
@@ -430,7 +431,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run = l_run * alpha + (psum[0] + psum[1]);
+    l_run += psum[0] + psum[1];
     mx_tile = half_max(mx);
 #pragma unroll
     for (int t = 0; t < DT; ++t) cout.a[t] = opnd[NQK + NMAIN + t];
@@ -447,6 +448,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   mx_tile = half_max(mx_tile);
   uint32_t j = 0;
   if (nfull >= 4) {
+    // nothing has been accumulated yet, so the first tile's max becomes the reference without any correction
+    m_run = mx_tile;
+    mb_run = m_run * scale_log2;
     // the first trip has no predecessor: its carried slots add zero
     Carry ca, cb;
 #pragma unroll
