@@ -34,8 +34,10 @@
 // awaited (vmcnt(0) + barrier) at the end of the trip.  One barrier per tile.
 //
 // Other differences from attention_bf16.h:
-//   * the reference max of a row is only moved when the tile max exceeds it by more than
-//     2^8 in the exponent, so the correction pass over the O accumulators is rare;
+//   * in the steady state no row max is taken at all: probabilities are computed against the
+//     reference the row already has and the reference is only moved (with the exp-shift
+//     correction of O and l) when a tile's row sum reaches 2^40, checked before that tile's
+//     PV product; the remaining tiles move it when the tile max exceeds it by 2^8;
 //   * the row sum is taken over the bf16-rounded probabilities with v_dot2c_f32_bf16
 //     (two terms per instruction), i.e. over exactly the weights the PV product uses.
 #pragma once
@@ -286,11 +288,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // instructions per slot, so that the matrix pipe and the vector pipe of the SIMD are fed by the same
   // wave at the same time.  A scheduling fence after every slot keeps this order:
   //   DT slots       last 16-key group of O += V(j-1)^T P(j-1)^T, operands and probabilities carried in
-  //                  registers across the barrier; carry the global -> LDS requests for K(j+2), V(j+1)
-  //   NQK slots      S(j+1) = K(j+1) Q^T; carry the rest of the requests and the first PQK pairs of
-  //                  P(j) = exp(S(j) - m)
-  //   NPV - DT slots O += V(j)^T P(j)^T for all but the last 16-key group; carry the remaining pairs of
-  //                  P(j) (each before the slot that needs its group) and the row max of S(j+1)
+  //                  registers across the barrier
+  //   NQK slots      S(j+1) = K(j+1) Q^T
+  //                  (these DT + NQK slots also carry the global -> LDS requests for K(j+2), V(j+1) and all of
+  //                  P(j) = exp(S(j) - reference), its bf16 rounding and the row sum)
+  //   NPV - DT slots O += V(j)^T P(j)^T for all but the last 16-key group
   // LDS operands are fetched in slot order, DT + ATTN_XLEAD slots ahead of their MFMA; the fetches for
   // the carried group are the last ones before the barrier, so the barrier sits in the middle of a
   // stream of MFMAs instead of at a point where the matrix pipe has drained.
@@ -298,47 +300,24 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int NPV = (BN / 16) * DT;   // MFMAs of the output update
   constexpr int NSLOT = NQK + NPV;
   constexpr int NPAIR = KT * 8;         // score pairs per lane; pairs 4 g .. 4 g + 3 are the 16-key group g
-  constexpr int PQK = 10;               // pairs exponentiated during the QK slots
+  constexpr int NPRE = DT + NQK;        // slots that carry the exponentials (all before the first PV slot of the tile)
   constexpr int NMAIN = NPV - DT;       // PV slots of the trip that owns the tile
-  constexpr int MAXSLOTS = NPV / 2;     // PV slots that carry the row max (the last ones before the barrier)
-  constexpr int EPS = KT * 16 / MAXSLOTS;  // scores folded into the max per such slot
   constexpr int XLEAD = ATTN_XLEAD;
-  static_assert(NPAIR == 16 && (KT * 16) % MAXSLOTS == 0 && 2 * WLW <= DT + NQK && NPAIR - PQK <= NMAIN &&
-                    MAXSLOTS <= NMAIN && XLEAD >= 0 && XLEAD < NQK,
-                "slot shape");
-  // pair PQK + m is produced in main PV slot m and first used in main PV slot ((PQK + m) / 4) * DT
-  // (the last group is used by the carried slots of the next trip): every pair must be ready in time
-  constexpr bool pairs_in_time = [] {
-    for (int m = 0; m < NPAIR - PQK; ++m)
-      if ((PQK + m) / 4 < NPAIR / 4 - 1 && m >= ((PQK + m) / 4) * DT) return false;
-    return true;
-  }();
-  static_assert(pairs_in_time, "a probability pair would be produced after the MFMA that consumes it");
+  static_assert(NPAIR == 16 && 2 * WLW <= NPRE && XLEAD >= 0 && XLEAD < NQK, "slot shape");
 
   struct Carry {
     bf16x8 a[DT];  // V^T operands of the last 16-key group
     u32x4 p;       // its probabilities
   };
 
-  // Reference max of tile j (mx_tile = row max of S(j), found during the previous trip).  Runs between the
-  // carried slots, which still belong to tile j-1, and the first use of the reference for tile j.
-  auto move_reference = [&](float mx_tile) {
-    const bool move = __builtin_fmaf(mx_tile, scale_log2, -mb_run) > RESCALE_LOG2;
-    if (__builtin_amdgcn_ballot_w64(move)) {  // rare: some row of this wave moves its reference
-      const float m_new = move ? mx_tile : m_run;
-      const float alpha = fast_exp2((m_run - m_new) * scale_log2);  // 1 for the rows that stay
-      m_run = m_new;
-      mb_run = m_new * scale_log2;
-      l_run *= alpha;
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
-    }
-  };
+  // No row max is taken in the steady state.  P = exp(S - reference) is computed against the reference the
+  // row already has; floating point is scale-free, so any reference gives the same normalised result as long
+  // as nothing overflows.  The tile's row sum (a by-product) is checked before the tile's PV product: if it is
+  // not below 2^40 (this includes inf and NaN) for any row of the wave, the reference is moved up to the tile
+  // max, O and l are corrected by the exp-shift factor, and the tile's probabilities are recomputed.
+  constexpr float SUM_GUARD = 1099511627776.0f;  // 2^40
 
-  auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], float& mx_tile,
-                       const Carry& cin, Carry& cout) {
+  auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], const Carry& cin, Carry& cout) {
     const char* sk = &smem[buf ^ 1][0][0];  // K(j+1)
     const char* sv = &smem[buf][1][0];      // V(j)
 
@@ -364,7 +343,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       }
       if (g + XLEAD < NSLOT) fetch(g + XLEAD);
     };
-    // request r of the 2 WLW global -> LDS requests of the trip
+    // request g of the 2 WLW global -> LDS requests of the trip
     auto request_for_slot = [&](int g) {
       if (g < 2 * WLW) {
         if (g < WLW) request_full_one(j + 2, buf, g, Yes{});
@@ -377,7 +356,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     u32x4 pq[NPAIR / 4];
     const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
     float psum[2] = {0.0f, 0.0f};
-    float mb = 0.0f;  // reference of tile j in the exponent domain, set after the carried slots
+    float mb = mb_run;
     auto exp_pair = [&](int pr) {
       const int pkt = pr / 8, i = 2 * (pr % 8);
       const float e0 = fast_exp2(__builtin_fmaf(s_cur[pkt][i], scale_log2, -mb));
@@ -388,6 +367,10 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       asm volatile("" : "+v"(packed), "+v"(psum[pr & 1]));
       pq[pr / 4][pr % 4] = packed;
     };
+    auto pairs_for_slot = [&](int g) {
+#pragma unroll
+      for (int pr = g * NPAIR / NPRE; pr < (g + 1) * NPAIR / NPRE; ++pr) exp_pair(pr);
+    };
 
     // ---- carried slots: last key group of tile j-1
 #pragma unroll
@@ -395,11 +378,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       fetch_for_slot(g);
       o[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cin.a[g], __builtin_bit_cast(bf16x8, cin.p), o[g], 0, 0, 0);
       request_for_slot(g);
+      pairs_for_slot(g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    move_reference(mx_tile);
-    mb = mb_run;
-    __builtin_amdgcn_sched_barrier(0);
 
     // ---- score slots of tile j+1
 #pragma unroll
@@ -408,31 +389,44 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const int ks = n / KT, kt = n % KT;
       s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[ks], ks == 0 ? zero16 : s_next[kt], 0, 0, 0);
       request_for_slot(DT + n);
-#pragma unroll
-      for (int pr = n * PQK / NQK; pr < (n + 1) * PQK / NQK; ++pr) exp_pair(pr);
+      pairs_for_slot(DT + n);
       __builtin_amdgcn_sched_barrier(0);
     }
 
+    // ---- guard (see above); O at this point holds everything up to and including tile j-1
+    if (__builtin_amdgcn_ballot_w64(!(psum[0] + psum[1] < SUM_GUARD))) {
+      float mx = s_cur[0][0];
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_cur[kt][i]);
+      mx = half_max(mx);
+      const bool move = mx * scale_log2 > mb_run;  // the reference only moves up
+      const float mb_new = move ? mx * scale_log2 : mb_run;
+      const float alpha = fast_exp2(mb_run - mb_new);
+      m_run = move ? mx : m_run;
+      mb_run = mb_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+      mb = mb_new;
+      psum[0] = psum[1] = 0.0f;
+#pragma unroll
+      for (int pr = 0; pr < NPAIR; ++pr) exp_pair(pr);
+    }
+    l_run += psum[0] + psum[1];
+    __builtin_amdgcn_sched_barrier(0);
+
     // ---- output slots of tile j, all key groups but the last
-    float mx = s_next[0][0];
 #pragma unroll
     for (int m = 0; m < NMAIN; ++m) {
       fetch_for_slot(DT + NQK + m);
       const int s4 = m / DT, t = m % DT;
       o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[NQK + m], __builtin_bit_cast(bf16x8, pq[s4]), o[t], 0, 0, 0);
-      if (m < NPAIR - PQK) exp_pair(PQK + m);
-      if (m >= NMAIN - MAXSLOTS) {
-#pragma unroll
-        for (int e = 0; e < EPS; ++e) {
-          const int idx = (m - (NMAIN - MAXSLOTS)) * EPS + e;
-          mx = fmaxf(mx, s_next[idx / 16][idx % 16]);
-        }
-        asm volatile("" : "+v"(mx));
-      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += psum[0] + psum[1];
-    mx_tile = half_max(mx);
 #pragma unroll
     for (int t = 0; t < DT; ++t) cout.a[t] = opnd[NQK + NMAIN + t];
     cout.p = pq[NPAIR / 4 - 1];
@@ -440,16 +434,15 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     __syncthreads();
   };
 
-  float mx_tile = sa[0][0];
-#pragma unroll
-  for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
-  mx_tile = half_max(mx_tile);
   uint32_t j = 0;
   if (nfull >= 4) {
     // nothing has been accumulated yet, so the first tile's max becomes the reference without any correction
-    m_run = mx_tile;
+    float mx_tile = sa[0][0];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
+    m_run = half_max(mx_tile);
     mb_run = m_run * scale_log2;
     // the first trip has no predecessor: its carried slots add zero
     Carry ca, cb;
@@ -457,8 +450,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     for (int t = 0; t < DT; ++t) ca.a[t] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
     ca.p = u32x4{0, 0, 0, 0};
     for (; j + 4 <= nfull; j += 2) {  // j + 3 <= nfull - 1
-      fast_step(j, 0, sa, sb, mx_tile, ca, cb);
-      fast_step(j + 1, 1, sb, sa, mx_tile, cb, ca);
+      fast_step(j, 0, sa, sb, ca, cb);
+      fast_step(j + 1, 1, sb, sa, cb, ca);
     }
     // last key group of the last steady-state tile
 #pragma unroll

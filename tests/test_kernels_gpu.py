@@ -156,6 +156,25 @@ def test_attention_bf16_reference_max_moves_slowly_and_fast(env, span):
     assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("jump_tile", [1, 6, 11])
+def test_attention_bf16_score_jump_overflows_the_stale_reference(env, d, jump_tile):
+    """All scores are ~0 except in one key tile, where they are ~+300 nats: exp against the reference of the
+    earlier tiles overflows to inf there.  The steady-state loop takes no row max; its row-sum guard has to
+    catch this before the tile's PV product and move the reference.  Rows 32.. keep small scores throughout."""
+    nq, nk = 64, 12 * 64 + 40
+    q = np.zeros((1, nq, d), np.float32)
+    q[:, :32, 0] = 1.0
+    q[:, 32:, 1] = 0.5
+    k = oracle.to_bf16_f32(rnd((1, nk, d), 2) * 0.25)
+    k[:, :, 0] = 0.0
+    k[:, 64 * jump_tile:64 * jump_tile + 64, 0] = oracle.to_bf16_f32(np.linspace(296, 304, 64, dtype=np.float32))
+    v = oracle.to_bf16_f32(rnd((1, nk, d), 3))
+    ref = oracle.attention_tiled(q, k, v, 1.0)
+    assert np.isfinite(ref).all()
+    assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
+
+
 def test_attention_bf16_direct_negative_and_zero_scale(env):
     q, k, v = (oracle.to_bf16_f32(rnd((2, n, 64), s)) for s, n in ((1, 70), (2, 400), (3, 400)))
     for scale in (-0.3, 0.0):
