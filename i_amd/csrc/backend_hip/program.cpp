@@ -136,9 +136,11 @@ bool hand_usable(const Run& run, const Recognized& r) {
       return ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back());
     }
     case Recognized::GemmNT: {
-      if (run.dtype_of(r.a.buffer) != DType::BF16 || run.dtype_of(r.b.buffer) != DType::BF16) return false;
+      const DType t = run.dtype_of(r.a.buffer);
+      if (run.dtype_of(r.b.buffer) != t) return false;
       const auto a = rows_cols(r.a);
-      return a.size() >= 2 && ihip::gemm_nt_bf16_supported(a.back());
+      if (a.size() < 2) return false;
+      return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
     }
     case Recognized::RowSoftmax: return true;
   }
@@ -202,6 +204,10 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       if (b[nb + 1] != a[nb + 1]) return "gemm operands disagree on the contracted extent";
       void* out = nullptr;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+      if (run.dtype_of(r.a.buffer) == DType::F32)
+        return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)),
+                                        static_cast<const float*>(run.raw_ptr(r.b.buffer)), static_cast<float*>(out), bh,
+                                        a[nb], b[nb], a[nb + 1], run.stream);
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
                                        a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j);
     }

@@ -21,22 +21,30 @@
 //               tiles, so at any time an XCD streams 1024 rows of A and 2048 rows of B
 //   M, N edges  rows past the end re-read the last valid row and are not stored
 // Requires k % 64 == 0 (the launcher falls back to gemm_nt_bf16.h otherwise).
+//
+// F32 = true is the same kernel for f32 operands (the reference's own arithmetic type): slabs of 32 k
+// (again 128-byte rows, so layout, swizzle and transfers are unchanged) and v_mfma_f32_32x32x2_f32, whose
+// operands are one f32 per lane with k = lane / 32: a 16-byte operand read covers k = 4 (2 ks + h) .. + 3,
+// and element e of it feeds MFMA e of the k-step.  Products and sums stay f32.  Requires k % 32 == 0.
 #pragma once
 #include "common.h"
 #include "params.h"
 
-__device__ __forceinline__ void gemm_nt_bf16_direct_body(const GemmParams& p) {
-  constexpr int BMT = 256, BNT = 256, BK = 64;
+template <bool F32>
+__device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
+  constexpr int BMT = 256, BNT = 256;
+  constexpr int ELEM = F32 ? 4 : 2;   // bytes per operand element
+  constexpr int BK = 128 / ELEM;      // k per slab: 128-byte slab rows
   constexpr int WM = 2, WN = 4, NWAVES = WM * WN;
   constexpr int TM = BMT / WM / 32;  // 4
   constexpr int TN = BNT / WN / 32;  // 2
-  constexpr int RB = 2 * BK;         // bytes per slab row
+  constexpr int RB = ELEM * BK;      // bytes per slab row
   constexpr int CH = RB / 16;        // chunks per row (= lanes per row of a wave-load)
   constexpr int RPW = 64 / CH;       // rows per wave-load
   constexpr int SLAB = BMT * RB;     // bytes of one operand slab (BMT == BNT)
   constexpr int WL = SLAB / 1024;    // wave-loads per slab
   constexpr int WLW = WL / NWAVES;   // ... per wave
-  constexpr int KS = BK / 16;
+  constexpr int KS = RB / 32;        // k-steps per slab: two 16-byte chunks (one per half-wave) each
   static_assert(BMT == BNT && WL % NWAVES == 0, "slab shape");
   __shared__ __attribute__((aligned(1024))) char smem[2][2][SLAB];  // [buffer][A, B]
 
@@ -57,7 +65,7 @@ __device__ __forceinline__ void gemm_nt_bf16_direct_body(const GemmParams& p) {
   const int wm = wave % WM, wn = wave / WM;
   const int c = lane & 31, h = lane >> 5;
 
-  const size_t row_bytes = (size_t)p.k * 2;
+  const size_t row_bytes = (size_t)p.k * ELEM;
   const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
   const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;
   float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
@@ -134,7 +142,13 @@ __device__ __forceinline__ void gemm_nt_bf16_direct_body(const GemmParams& p) {
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+          if constexpr (F32) {
+            const f32x4 av = __builtin_bit_cast(f32x4, af[ks & 1][i]), bv = __builtin_bit_cast(f32x4, bfr[ks & 1][j]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[e], bv[e], acc[i][j], 0, 0, 0);
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+          }
           const int slot = (ks * TM + i) * TN + j;  // 0 .. 31
           if (more && slot % 2 == 0 && slot / 2 < 2 * WLW) {
             const int r = slot / 2, it = r % WLW;

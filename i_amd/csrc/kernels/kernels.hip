@@ -44,7 +44,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64(Gem
 }
 
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct(GemmParams p) {
-  gemm_nt_bf16_direct_body(p);
+  gemm_nt_direct_body<false>(p);
+}
+// f32 operands, f32 MFMA: the arithmetic type of the reference
+extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_direct(GemmParams p) {
+  gemm_nt_direct_body<true>(p);
 }
 
 #define SOFTMAX_WAVE(NV)                                                                          \

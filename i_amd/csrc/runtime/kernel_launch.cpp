@@ -120,6 +120,27 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
 
+bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 32 == 0 && k <= (size_t(1) << 21); }
+
+Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                       hipStream_t stream) {
+  if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 32 (at most 2^21)";
+  if (bh == 0 || m == 0 || n == 0) return {};
+  if (!fits_u32(m) || !fits_u32(n) || bh > 65535) return "gemm_nt f32 kernel: extent too large";
+  if (!a || !b || !c) return "gemm_nt f32 kernel: null device pointer";
+  GemmParams p{};
+  p.a = a; p.b = b; p.c = c;
+  p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.tiles_m = (uint32_t)((m + 255) / 256);
+  p.tiles_n = (uint32_t)((n + 255) / 256);
+  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // super-blocks of 4 x 8 tiles
+  const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+  if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
+  hipFunction_t fn;
+  if (Err e = builtin_function("gemm_nt_f32_256x256x32_direct", &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)grid, (unsigned)bh, 1, 512, &p, sizeof(p), stream);
+}
+
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream) {
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";

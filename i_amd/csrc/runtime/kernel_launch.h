@@ -28,6 +28,11 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
                         hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
 bool gemm_nt_bf16_supported(size_t k);
 
+// c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 32 == 0
+Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                       hipStream_t stream);
+bool gemm_nt_f32_supported(size_t k);
+
 // y[rows,cols] = row softmax of x, f32
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream);
 

@@ -74,6 +74,13 @@ int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c,
                        size_t bh, size_t m, size_t n, size_t k, void* stream);
 
 /*
+ * The same mm_t with f32 a, b, c and f32 products and sums (f32 MFMA), the reference's own
+ * arithmetic type: what the host f32 ABI of i.h dispatches to.  Requires k % 32 == 0.
+ */
+int i_hip_gemm_nt_f32(const float* a, const float* b, float* c,
+                      size_t bh, size_t m, size_t n, size_t k, void* stream);
+
+/*
  * Row softmax over the last axis of an f32 [rows, cols] matrix: the fused
  * kernel for  row_max_shift >> exp >> row_normalize  (README.md:19-25).
  */

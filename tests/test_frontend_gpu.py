@@ -186,10 +186,25 @@ def test_config3_mm_t_bf16_device(torch):
     close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
 
 
-def test_mm_t_f32_small_vs_emitted_c(torch):
-    a, b = rnd((100, 40), 1), rnd((70, 40), 2)
+@pytest.mark.parametrize("k", [40, 64])  # 40: generated kernel; 64: f32 MFMA kernel
+def test_mm_t_f32_small_vs_emitted_c(torch, k):
+    a, b = rnd((100, k), 1), rnd((70, k), 2)
     comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
+
+
+def test_config3_mm_t_through_the_host_f32_abi(torch):
+    """BASELINE configs[2] the way the unchanged reference frontend would run it: host f32 arrays holding
+    bf16-representable values through i_exec_into (upload, f32 MFMA kernel, download)."""
+    n = 4096
+    a = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (n, n)).astype(np.float32))
+    b = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (n, n)).astype(np.float32))
+    comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    c = comp.exec_numpy(a, b)
+    rows = np.r_[0:4, n - 4:n]
+    close(c[rows], oracle.mm_t(a[rows], b), RTOL_F32)
+    cols = np.r_[0:4, n - 4:n]
+    close(c[:, cols], oracle.mm_t(a, b[cols]), RTOL_F32)
 
 
 # ------------------------------------------------------------------ BASELINE configs 4 and 5 (bf16 in, f32 accumulate)

@@ -282,6 +282,27 @@ def test_gemm_nt_bf16_both_kernels_vs_oracle(env, monkeypatch, bh, m, n, k, dire
     assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 32), (1, 300, 260, 96), (2, 600, 520, 160), (1, 1, 1, 64),
+                                      (3, 257, 255, 320), (1, 100, 70, 64)])
+def test_gemm_nt_f32_vs_oracle(env, bh, m, n, k):
+    """f32 operands, f32 MFMA: the reference's own arithmetic type, against the scalar oracle at the f32 bar."""
+    t = env.torch
+    a, b = rnd((bh, m, k), 1, "uniform"), rnd((bh, n, k), 2, "uniform")
+    ad, bd = t.from_numpy(a).cuda(), t.from_numpy(b).cuda()
+    cd = t.full((bh, m, n), float("nan"), device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nt_f32(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+    t.cuda.synchronize()
+    assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_F32)
+
+
+def test_gemm_nt_f32_rejects_ragged_k(env):
+    t = env.torch
+    x = t.zeros(64, 40, device="cuda")
+    c = t.zeros(64, 64, device="cuda")
+    rc = env.nat.core.i_hip_gemm_nt_f32(x.data_ptr(), x.data_ptr(), c.data_ptr(), 1, 64, 64, 40, env.stream())
+    assert rc == -1 and "multiple of 32" in env.nat.last_error()
+
+
 def test_gemm_nt_bf16_full_size_linearity(env):
     """M=N=K=4096: C(A1+A2, B) == C(A1,B) + C(A2,B) for bf16-exact sums, and row block vs oracle."""
     t = env.torch
