@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <set>
 #include <sstream>
@@ -150,14 +151,15 @@ std::set<size_t> exclusive_intermediates(const ExecPlan& plan, size_t kernel) {
   return out;
 }
 
-void analyze(const ExecPlan& plan, size_t k, GenericKernel& info) {
-  const Kernel<Param>& kernel = plan.kernels[k];
+// Parallel loops and private buffers of one phase.  `body` is the phase's statement list (the spine is followed
+// while it is a single loop); buffers in `shared` are touched by other phases and must stay in memory.
+void analyze(const ExecPlan& plan, size_t k, const Block<Param>& body, const std::set<Param>& shared, GenericPhase& info) {
   const Step* dispatch = nullptr;
   for (const Step& s : plan.exec)
     if (s.kind == Step::Dispatch && s.id == k) dispatch = &s;
   const std::set<size_t> exclusive = exclusive_intermediates(plan, k);
 
-  const Block<Param>* block = &kernel.body;
+  const Block<Param>* block = &body;
   std::set<Param> privatized;
   while (block->size() == 1 && (*block)[0].kind == PAct::Loop) {
     const PAct& loop = (*block)[0];
@@ -174,7 +176,7 @@ void analyze(const ExecPlan& plan, size_t k, GenericKernel& info) {
           none_use &= !uses;
         }
       if (all_use) continue;  // distinct iterations touch distinct elements
-      const bool can_privatize = none_use && w.writeable && dispatch && w.ind < dispatch->writes.size() &&
+      const bool can_privatize = none_use && !shared.count(w) && w.writeable && dispatch && w.ind < dispatch->writes.size() &&
                                  dispatch->writes[w.ind].kind == BufferRef::Intermediate &&
                                  exclusive.count(dispatch->writes[w.ind].id);
       if (can_privatize) want_private.insert(w);
@@ -201,6 +203,26 @@ void analyze(const ExecPlan& plan, size_t k, GenericKernel& info) {
     if (pb.is_static && pb.static_size > 4096) pb.is_static = false;
     info.privates.push_back(pb);
   }
+}
+
+// Top-level statements of a kernel grouped into phases: every loop is a phase of its own, a run of
+// other statements (initialisations of scalars) is one phase.  Returns [first, last) index ranges.
+std::vector<std::pair<size_t, size_t>> phase_ranges(const Block<Param>& body) {
+  std::vector<std::pair<size_t, size_t>> out;
+  size_t i = 0;
+  while (i < body.size()) {
+    if (body[i].kind == PAct::Loop) {
+      out.push_back({i, i + 1});
+      ++i;
+    } else {
+      size_t j = i;
+      while (j < body.size() && body[j].kind != PAct::Loop) ++j;
+      out.push_back({i, j});
+      i = j;
+    }
+  }
+  if (out.empty()) out.push_back({0, 0});
+  return out;
 }
 
 // ------------------------------------------------------------------ statement printer
@@ -265,57 +287,87 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
     info.name = "f" + std::to_string(k);
     info.n_reads = plan.kernels[k].reads.size();
     info.n_writes = plan.kernels[k].writes.size();
-    analyze(plan, k, info);
+    const Block<Param>& body = plan.kernels[k].body;
     const MFn& fn = module.kernels[k];
+    // one statement of the module per action of the plan kernel (a trailing return aside)
+    size_t fn_stmts = fn.body.size();
+    while (fn_stmts > 0 && fn.body[fn_stmts - 1].kind == MStmt::Return) --fn_stmts;
+    // Splitting into phases is opt-in (ILANG_HIP_PHASES=1): it is verified on the CPU emulation of the runtime
+    // only, see tests/test_generated_kernels_cpu.py.
+    const char* want_phases = std::getenv("ILANG_HIP_PHASES");
+    auto ranges = phase_ranges(body);
+    if (fn_stmts != body.size() || !want_phases || want_phases[0] != '1') ranges = {{0, body.size()}};  // one phase, whole body
+    // buffers touched by more than one phase stay in memory
+    std::map<Param, size_t> touched;
+    std::vector<Block<Param>> bodies;
+    for (const auto& [first, last] : ranges) {
+      bodies.emplace_back(body.begin() + first, body.begin() + last);
+      Uses u;
+      collect(bodies.back(), u);
+      std::set<Param> seen;
+      for (const auto* a : u.all) seen.insert(a->buffer);
+      for (const Param& b : seen) ++touched[b];
+    }
+    std::set<Param> shared;
+    for (const auto& [b, n] : touched)
+      if (n > 1) shared.insert(b);
 
     const size_t nr = std::max<size_t>(info.n_reads, 1), nw = std::max<size_t>(info.n_writes, 1);
     src << "struct Args_" << info.name << " { View readonlys[" << nr << "]; View writeables[" << nw << "]; };\n";
-    src << "extern \"C\" __global__ void __launch_bounds__(64) " << info.name << "(Args_" << info.name << " args) {\n";
-    src << "  const View* readonlys = args.readonlys;\n";
-    src << "  View writeables[" << nw << "];\n";
-    src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
-    src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
-    src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
-    for (const PrivateBuffer& pb : info.privates) {
-      if (pb.is_static) {
-        src << "  float priv" << pb.writeable << "[" << pb.static_size << "];\n";
-        src << "  writeables[" << pb.writeable << "].data = priv" << pb.writeable << ";\n";
+    for (size_t ph = 0; ph < ranges.size(); ++ph) {
+      GenericPhase phase;
+      phase.name = ranges.size() == 1 ? info.name : info.name + "_p" + std::to_string(ph);
+      analyze(plan, k, bodies[ph], shared, phase);
+      const std::vector<MStmt> stmts(fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].first : 0),
+                                     fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].second : fn_stmts));
+      src << "extern \"C\" __global__ void __launch_bounds__(64) " << phase.name << "(Args_" << info.name << " args) {\n";
+      src << "  const View* readonlys = args.readonlys;\n";
+      src << "  View writeables[" << nw << "];\n";
+      src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
+      src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
+      src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
+      for (const PrivateBuffer& pb : phase.privates) {
+        if (pb.is_static) {
+          src << "  float priv" << pb.writeable << "[" << pb.static_size << "];\n";
+          src << "  writeables[" << pb.writeable << "].data = priv" << pb.writeable << ";\n";
+        } else {
+          const Step* dispatch = nullptr;
+          for (const Step& st : plan.exec)
+            if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
+          const size_t prank = plan.intermediates[dispatch->writes[pb.writeable].id].layout.size();
+          src << "  { size_t n = 1; for (int d = 0; d < " << prank << "; ++d) n *= writeables[" << pb.writeable
+              << "].layout[d]; writeables[" << pb.writeable << "].data += wi_first * n; }\n";
+        }
+      }
+      Printer pr;
+      if (phase.parallel_loops.empty()) {
+        src << "  if (wi_first != 0) return;\n";
+        pr.block(stmts, 1);
+        src << pr.os.str();
       } else {
-        const Step* dispatch = nullptr;
-        for (const Step& st : plan.exec)
-          if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
-        const size_t prank = plan.intermediates[dispatch->writes[pb.writeable].id].layout.size();
-        src << "  { size_t n = 1; for (int d = 0; d < " << prank << "; ++d) n *= writeables[" << pb.writeable
-            << "].layout[d]; writeables[" << pb.writeable << "].data += wi_first * n; }\n";
+        std::vector<std::string> iters;
+        for (size_t id : phase.parallel_loops) iters.push_back("i" + std::to_string(id));
+        for (const std::string& it : iters) {
+          const MStmt* loop = find_loop(stmts, it);
+          if (!loop) lower_error("parallel loop " + it + " not found in kernel body");
+          src << "  const size_t n_" << it << " = " << expr_text(*loop->value) << ";\n";
+          pr.parallel.insert(it);
+        }
+        src << "  size_t wi_total = 1;\n";
+        for (const std::string& it : iters) src << "  wi_total *= n_" << it << ";\n";
+        src << "  for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
+        src << "    size_t wi_rest = wi;\n";
+        for (size_t t = iters.size(); t-- > 0;) {
+          src << "    const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
+          src << " wi_rest /= n_" << iters[t] << ";\n";
+        }
+        pr.block(stmts, 2);
+        src << pr.os.str();
+        src << "  }\n";
       }
+      src << "}\n\n";
+      info.phases.push_back(std::move(phase));
     }
-    Printer pr;
-    if (info.parallel_loops.empty()) {
-      src << "  if (wi_first != 0) return;\n";
-      pr.block(fn.body, 1);
-      src << pr.os.str();
-    } else {
-      std::vector<std::string> iters;
-      for (size_t id : info.parallel_loops) iters.push_back("i" + std::to_string(id));
-      for (const std::string& it : iters) {
-        const MStmt* loop = find_loop(fn.body, it);
-        if (!loop) lower_error("parallel loop " + it + " not found in kernel body");
-        src << "  const size_t n_" << it << " = " << expr_text(*loop->value) << ";\n";
-        pr.parallel.insert(it);
-      }
-      src << "  size_t wi_total = 1;\n";
-      for (const std::string& it : iters) src << "  wi_total *= n_" << it << ";\n";
-      src << "  for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
-      src << "    size_t wi_rest = wi;\n";
-      for (size_t t = iters.size(); t-- > 0;) {
-        src << "    const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
-        src << " wi_rest /= n_" << iters[t] << ";\n";
-      }
-      pr.block(fn.body, 2);
-      src << pr.os.str();
-      src << "  }\n";
-    }
-    src << "}\n\n";
   }
   if (any) out.source = src.str();
   return out;

@@ -23,12 +23,26 @@ struct PrivateBuffer {
   size_t static_size = 0; // elements, when static
 };
 
-struct GenericKernel {
-  std::string name;                       // f<k>
-  size_t n_reads = 0, n_writes = 0;
+// A kernel whose body is a sequence of loop nests (e.g. a row maximum followed by the subtraction that
+// consumes it) is launched as one phase per top-level nest, in order on the stream: every phase gets its own
+// work-item space, and the stream order is the grid-wide dependency between them.
+struct GenericPhase {
+  std::string name;                       // f<k> for a single-phase kernel, f<k>_p<i> otherwise
   std::vector<size_t> parallel_loops;     // loop ids, outermost first (empty: one work-item)
   std::vector<ic::Extent<ic::Param>> parallel_extents;
-  std::vector<PrivateBuffer> privates;
+  std::vector<PrivateBuffer> privates;    // only buffers that no other phase touches
+};
+
+struct GenericKernel {
+  std::string name;                       // f<k>; empty when not emitted
+  size_t n_reads = 0, n_writes = 0;
+  std::vector<GenericPhase> phases;
+  bool is_private(size_t writeable) const {
+    for (const GenericPhase& ph : phases)
+      for (const PrivateBuffer& pb : ph.privates)
+        if (pb.writeable == writeable) return true;
+    return false;
+  }
 };
 
 struct GenericModule {

@@ -258,25 +258,6 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
   std::vector<unsigned char> args((nr + nw) * view_bytes, 0);
   if (args.size() > 4000) return "kernel " + std::to_string(k) + " takes too many buffers for one launch";
 
-  // work-item space
-  size_t total = 1;
-  for (const auto& e : gk.parallel_extents) {
-    const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
-    Extent<size_t> resolved{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind};
-    total *= run.extent(resolved);
-  }
-  if (total == 0) return {};
-  size_t threads = gk.parallel_loops.empty() ? 1 : total;
-  // dynamic private buffers cost memory per work-item slot: cap the slots
-  size_t slot_elems = 0;
-  for (const PrivateBuffer& pb : gk.privates)
-    if (!pb.is_static) slot_elems += std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
-  size_t max_threads = size_t(1) << 20;
-  if (slot_elems) max_threads = std::max<size_t>(64, std::min(max_threads, (size_t(1) << 28) / (slot_elems * 4)));
-  threads = std::min(threads, max_threads);
-  const unsigned grid = (unsigned)((threads + 63) / 64);
-  const size_t slots = (size_t)grid * 64;
-
   auto fill = [&](size_t slot, void* data, BufferRef r) {
     unsigned char* v = args.data() + slot * view_bytes;
     std::memcpy(v, &data, 8);
@@ -289,23 +270,46 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
     if (ihip::Err e = run.read_f32(dispatch.reads[i], &ptr); !e.empty()) return e;
     fill(i, ptr, dispatch.reads[i]);
   }
+  // buffers that live in memory are the same for every phase
   for (size_t i = 0; i < dispatch.writes.size(); ++i) {
-    const BufferRef r = dispatch.writes[i];
     void* ptr = nullptr;
-    const PrivateBuffer* priv = nullptr;
-    for (const PrivateBuffer& pb : gk.privates)
-      if (pb.writeable == i) priv = &pb;
-    if (priv && !priv->is_static) {
-      const size_t n = std::max<size_t>(1, product(run.layout_of(r)));
-      if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
-    } else if (!priv) {
-      if (ihip::Err e = run.write_f32(r, &ptr); !e.empty()) return e;
-    }
-    fill(nr + i, ptr, r);
+    if (!gk.is_private(i))
+      if (ihip::Err e = run.write_f32(dispatch.writes[i], &ptr); !e.empty()) return e;
+    fill(nr + i, ptr, dispatch.writes[i]);
   }
-  hipFunction_t fn;
-  if (ihip::Err e = generic_function(p, gk.name, &fn); !e.empty()) return e;
-  return ihip::launch(fn, grid, 1, 1, 64, args.data(), args.size(), run.stream);
+
+  // one launch per phase, in order on the stream
+  for (const GenericPhase& ph : gk.phases) {
+    size_t total = 1;
+    for (const auto& e : ph.parallel_extents) {
+      const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
+      Extent<size_t> resolved{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind};
+      total *= run.extent(resolved);
+    }
+    if (total == 0) continue;
+    size_t threads = ph.parallel_loops.empty() ? 1 : total;
+    // dynamic private buffers cost memory per work-item slot: cap the slots
+    size_t slot_elems = 0;
+    for (const PrivateBuffer& pb : ph.privates)
+      if (!pb.is_static) slot_elems += std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+    size_t max_threads = size_t(1) << 20;
+    if (slot_elems) max_threads = std::max<size_t>(64, std::min(max_threads, (size_t(1) << 28) / (slot_elems * 4)));
+    threads = std::min(threads, max_threads);
+    const unsigned grid = (unsigned)((threads + 63) / 64);
+    const size_t slots = (size_t)grid * 64;
+    for (const PrivateBuffer& pb : ph.privates) {
+      void* ptr = nullptr;
+      if (!pb.is_static) {
+        const size_t n = std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+        if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
+      }
+      fill(nr + pb.writeable, ptr, dispatch.writes[pb.writeable]);
+    }
+    hipFunction_t fn;
+    if (ihip::Err e = generic_function(p, ph.name, &fn); !e.empty()) return e;
+    if (ihip::Err e = ihip::launch(fn, grid, 1, 1, 64, args.data(), args.size(), run.stream); !e.empty()) return e;
+  }
+  return {};
 }
 
 const Step* find_dispatch(const ExecPlan& plan, size_t k) {
@@ -359,13 +363,17 @@ std::string program_code(const Component& component) {
     for (BufferRef r : d->reads) os << " " << ref_name(r);
     os << "; writes";
     for (BufferRef r : d->writes) os << " " << ref_name(r);
-    os << "\n//     work-items:";
-    if (gen.kernels[k].parallel_loops.empty()) os << " 1 (no independent outer loop)";
-    for (size_t id : gen.kernels[k].parallel_loops) os << " i" << id;
-    if (!gen.kernels[k].privates.empty()) {
-      os << "; work-item-private:";
-      for (const auto& pb : gen.kernels[k].privates)
-        os << " " << ref_name(d->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
+    for (const GenericPhase& ph : gen.kernels[k].phases) {
+      os << "\n//     ";
+      if (gen.kernels[k].phases.size() > 1) os << "launch " << ph.name << ", ";
+      os << "work-items:";
+      if (ph.parallel_loops.empty()) os << " 1 (no independent outer loop)";
+      for (size_t id : ph.parallel_loops) os << " i" << id;
+      if (!ph.privates.empty()) {
+        os << "; work-item-private:";
+        for (const auto& pb : ph.privates)
+          os << " " << ref_name(d->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
+      }
     }
     os << "\n";
   }
@@ -424,12 +432,10 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
     if (hand[k]) {
       for (size_t id : hand_intermediates(p.recognized[k])) needed.insert(id);
     } else {
-      std::set<size_t> priv;
-      for (const PrivateBuffer& pb : p.generic.kernels[k].privates) priv.insert(pb.writeable);
       for (BufferRef r : d->reads)
         if (r.kind == BufferRef::Intermediate) needed.insert(r.id);
       for (size_t i = 0; i < d->writes.size(); ++i)
-        if (d->writes[i].kind == BufferRef::Intermediate && !priv.count(i)) needed.insert(d->writes[i].id);
+        if (d->writes[i].kind == BufferRef::Intermediate && !p.generic.kernels[k].is_private(i)) needed.insert(d->writes[i].id);
     }
   }
 

@@ -1,0 +1,111 @@
+"""Runs components through the product's executor with every kernel in its generated form, on the CPU
+emulation of the HIP runtime (shim.cpp), and compares with the C the oracle backend emits for the same
+component.  Started as a subprocess by tests/test_generated_kernels_cpu.py with
+ILANG_CORE_LIB, ILANG_HIPCC, ILANG_HIP_GENERATED_ONLY, ILANG_NO_TORCH and ILANG_NO_DISK_CACHE set.
+Prints the case name before running it, so a crash (a guard page hit = out-of-bounds access) names its case."""
+import sys
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent.parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+import oracle  # noqa: E402
+from i_amd import Component as i, I  # noqa: E402
+
+
+def rnd(shape, seed):
+    return np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+
+
+def flash(split="i:16,j:16", p=""):
+    mm_t = i(f"{p}ik*{p}jk~{p}ijk | {split} | {p}jii'j'k") >> i(f"+{p}ijk~{p}ij | {split} | {p}jii'j'k0")
+    row_max_shift = (I & i(f">{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij-{p}i~{p}ij | {split} | {p}ji01i'j'")
+    exp = i(f"^{p}ij~{p}ij | {split} | {p}ji0i'j'")
+    row_normalize = (I & i(f"+{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij/{p}i~{p}ij | {split} | {p}ji01i'j'")
+    mm = i(f"{p}ij*{p}jk~{p}ikj | {split} | {p}ji0i'kj'") >> i(f"+{p}ikj~{p}ik | {split} | {p}jii'kj'0")
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
+def naive(split="i:16,j:16"):
+    mm_t = i(f"ik*jk~ijk | {split} | jii'j'k") >> i(f"+ijk~ij | {split} | jii'j'k0")
+    row_max_shift = (I & i(f">ij~i | {split} | jii'j'")) >> i(f"ij-i~ij | {split} | 1jii'j'")
+    exp = i(f"^ij~ij | {split} | jii'j'")
+    row_normalize = (I & i(f"+ij~i | {split} | jii'j'")) >> i(f"ij/i~ij | {split} | 1jii'j'")
+    mm = i(f"ij*jk~ikj | {split} | jii'kj'") >> i(f"+ikj~ik | {split} | jii'kj'0")
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
+def softmax_naive(s="i:16,j:16"):
+    return (((I & i(f">ij~i|{s}|jii'j'")) >> i(f"ij-i~ij|{s}|1jii'j'")) >> i(f"^ij~ij|{s}|jii'j'")
+            >> ((I & i(f"+ij~i|{s}|jii'j'")) >> i(f"ij/i~ij|{s}|1jii'j'")))
+
+
+def softmax_rowstaged():
+    return (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
+            >> ((I & i("+ij~i|i:16|ii'0j")) >> i("ij/i~ij|i:16|ii'01j")))
+
+
+def batched_naive():
+    mm_t = i("bhij*bhkj~bhikj | i:16,k:16 | bhkii'k'j") >> i("+bhikj~bhik | i:16,k:16 | bhkii'k'j0")
+    row_max_shift = (I & i(">bhik~bhi | i:16,k:16 | bhkii'k'")) >> i("bhik-bhi~bhik | i:16,k:16 | bh1kii'k'")
+    exp = i("^bhik~bhik | i:16,k:16 | bhkii'k'")
+    row_normalize = (I & i("+bhik~bhi | i:16,k:16 | bhkii'k'")) >> i("bhik/bhi~bhik | i:16,k:16 | bh1kii'k'")
+    mm = i("bhik*bhkj~bhijk | i:16,k:16 | bhkii'jk'") >> i("+bhijk~bhij | i:16,k:16 | bhkii'jk'0")
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
+CASES = {
+    "flash 33x17": (flash, [(33, 17)] * 3),
+    "flash 48x24 i:32,j:8": (lambda: flash("i:32,j:8"), [(48, 24)] * 3),
+    "flash one key": (flash, [(17, 3), (1, 3), (1, 5)]),
+    "flash batched": (lambda: flash(p="bh"), [(2, 3, 20, 8)] * 3),
+    "naive attention 32x40": (naive, [(32, 40)] * 3),
+    "naive attention ragged": (naive, [(21, 12), (37, 12), (37, 9)]),
+    "batched naive attention": (batched_naive, [(2, 3, 4, 8)] * 3),
+    "softmax naive 20x37": (softmax_naive, [(20, 37)]),
+    "softmax naive 1x1": (softmax_naive, [(1, 1)]),
+    "softmax naive i:4,j:32": (lambda: softmax_naive("i:4,j:32"), [(9, 70)]),
+    "softmax row-staged": (softmax_rowstaged, [(20, 37)]),
+    "mm_t": (lambda: i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0"), [(100, 40), (70, 40)]),
+    "mm_t empty": (lambda: i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0"), [(0, 5), (3, 5)]),
+    "matmul unfused": (lambda: i("ik*kj~ijk") >> i("+ijk~ij"), [(8, 16), (16, 7)]),
+    "matmul fused init site": (lambda: i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0"), [(8, 16), (16, 7)]),
+    "row sum": (lambda: i("+ij~i"), [(16, 8)]),
+    "column max": (lambda: i(">ij~j"), [(9, 14)]),
+    "total": (lambda: i("+ij~."), [(6, 11)]),
+    "fanout two outputs": (lambda: i("+ij~i") & i(">ij~j"), [(9, 14)]),
+    "swapped fanout": (lambda: ~(i("+ij~i") & i(">ij~j")), [(9, 14)]),
+    "scalar operand": (lambda: i("ij*.~ij"), [(6, 11), ()]),
+    "mlp with pair": (lambda: (i("ij~ij") | ((i("ij*j~ij") >> i("+ij~i")) >> i(">i~i"))) >> (i("ij*j~ij") >> i("+ij~i")),
+                      [(7, 16), (16, 8), (8,)]),
+}
+
+
+def main():
+    names = sys.argv[1:] or list(CASES)
+    failed = []
+    for name in names:
+        build, shapes = CASES[name]
+        print("CASE", name, flush=True)
+        comp = build()
+        inputs = [rnd(s, k + 1) for k, s in enumerate(shapes)]
+        got = comp.exec_numpy(*inputs)
+        ref = oracle.compile_component(comp._ptr).run(*inputs)
+        got = got if isinstance(got, tuple) else (got,)
+        ref = ref if isinstance(ref, tuple) else (ref,)
+        for g, r in zip(got, ref):
+            scale = float(np.abs(r).max()) if r.size else 1.0
+            err = float(np.abs(g - r).max()) / (scale or 1.0) if r.size else 0.0
+            ok = g.shape == r.shape and (r.size == 0 or (np.isfinite(g).all() and err <= 1e-5))
+            if not ok:
+                failed.append(name)
+                print("MISMATCH", name, g.shape, r.shape, err, flush=True)
+    print("DONE", len(names), "cases;", "failed:", failed, flush=True)
+    sys.exit(1 if failed else 0)
+
+
+if __name__ == "__main__":
+    main()

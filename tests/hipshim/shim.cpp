@@ -1,0 +1,137 @@
+// A host implementation of the dozen HIP entry points the runtime uses, for CPU tests of the generic
+// code generator and the program executor (no GPU, no HIP runtime).
+//   memory    every allocation ends exactly at an inaccessible guard page and has one before it, and is
+//             filled with NaN bit patterns: an out-of-bounds access faults, a read of unwritten memory shows
+//   modules   an "image" is a host shared object (produced by hostcc.py from the generated HIP source);
+//             anything else (the prebuilt gfx950 code object) is refused, so only generated kernels run
+//   launches  run synchronously, one work-item after the other, with blockIdx / threadIdx set per item
+#include <dlfcn.h>
+#include <elf.h>
+#include <hip/hip_runtime_api.h>
+#include <sys/mman.h>
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+namespace {
+std::mutex g_mu;
+struct Block {
+  void* map;
+  size_t map_len;
+};
+std::map<void*, Block> g_blocks;
+const size_t kPage = 4096;
+
+hipError_t guarded_alloc(void** p, size_t bytes) {
+  if (bytes == 0) bytes = 4;
+  const size_t body = (bytes + kPage - 1) / kPage * kPage;
+  const size_t len = body + 2 * kPage;
+  char* m = static_cast<char*>(mmap(nullptr, len, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0));
+  if (m == MAP_FAILED) return hipErrorOutOfMemory;
+  std::memset(m, 0xFF, len);
+  mprotect(m, kPage, PROT_NONE);
+  mprotect(m + kPage + body, kPage, PROT_NONE);
+  char* user = m + kPage + body - ((bytes + 15) / 16 * 16);  // 16-byte aligned, ends within 15 bytes of the guard
+  *p = user;
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_blocks[user] = {m, len};
+  return hipSuccess;
+}
+hipError_t guarded_free(void* p) {
+  if (!p) return hipSuccess;
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = g_blocks.find(p);
+  if (it == g_blocks.end()) return hipErrorInvalidValue;
+  munmap(it->second.map, it->second.map_len);
+  g_blocks.erase(it);
+  return hipSuccess;
+}
+struct Module {
+  void* handle;
+  std::string path;
+};
+struct BigArgs {
+  unsigned char bytes[4096];
+};
+}  // namespace
+
+extern "C" {
+hipError_t hipGetDevice(int* dev) {
+  *dev = 0;
+  return hipSuccess;
+}
+const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "emulated HIP error"; }
+hipError_t hipMalloc(void** p, size_t bytes) { return guarded_alloc(p, bytes); }
+hipError_t hipFree(void* p) { return guarded_free(p); }
+hipError_t hipMallocAsync(void** p, size_t bytes, hipStream_t) { return guarded_alloc(p, bytes); }
+hipError_t hipFreeAsync(void* p, hipStream_t) { return guarded_free(p); }
+hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t) {
+  std::memcpy(dst, src, bytes);
+  return hipSuccess;
+}
+hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+
+hipError_t hipModuleLoadData(hipModule_t* mod, const void* image) {
+  const auto* eh = static_cast<const Elf64_Ehdr*>(image);
+  if (std::memcmp(eh->e_ident, ELFMAG, SELFMAG) != 0 || eh->e_machine != EM_X86_64) return hipErrorInvalidImage;
+  const size_t size = eh->e_shoff + size_t(eh->e_shnum) * eh->e_shentsize;
+  char path[] = "/tmp/ilang_shim_XXXXXX";
+  const int fd = mkstemp(path);
+  if (fd < 0) return hipErrorInvalidImage;
+  const bool ok = write(fd, image, size) == (ssize_t)size;
+  close(fd);
+  void* h = ok ? dlopen(path, RTLD_NOW | RTLD_LOCAL) : nullptr;
+  unlink(path);
+  if (!h) {
+    std::fprintf(stderr, "hip shim: dlopen failed: %s\n", dlerror());
+    return hipErrorInvalidImage;
+  }
+  *mod = reinterpret_cast<hipModule_t>(new Module{h, path});
+  return hipSuccess;
+}
+hipError_t hipModuleUnload(hipModule_t mod) {
+  auto* m = reinterpret_cast<Module*>(mod);
+  dlclose(m->handle);
+  delete m;
+  return hipSuccess;
+}
+hipError_t hipModuleGetFunction(hipFunction_t* fn, hipModule_t mod, const char* name) {
+  auto* m = reinterpret_cast<Module*>(mod);
+  void* f = dlsym(m->handle, name);
+  void* set = dlsym(m->handle, "shim_set_ids");
+  if (!f || !set) return hipErrorNotFound;
+  // a function handle is the pair (kernel, id setter of its library)
+  *fn = reinterpret_cast<hipFunction_t>(new std::pair<void*, void*>(f, set));
+  return hipSuccess;
+}
+hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
+                                 unsigned bz, unsigned, hipStream_t, void**, void** extra) {
+  if (gy != 1 || gz != 1 || by != 1 || bz != 1 || !extra) return hipErrorInvalidValue;
+  const void* buf = nullptr;
+  size_t size = 0;
+  for (void** e = extra; *e != HIP_LAUNCH_PARAM_END; e += 2) {
+    if (*e == HIP_LAUNCH_PARAM_BUFFER_POINTER) buf = e[1];
+    else if (*e == HIP_LAUNCH_PARAM_BUFFER_SIZE) size = *static_cast<size_t*>(e[1]);
+  }
+  if (!buf || size > sizeof(BigArgs)) return hipErrorInvalidValue;
+  BigArgs args;
+  std::memset(&args, 0xEE, sizeof args);
+  std::memcpy(&args, buf, size);
+  auto* pair = reinterpret_cast<std::pair<void*, void*>*>(fn);
+  // a by-value struct larger than 16 bytes travels in memory at the start of the argument area, so a kernel
+  // that declares a smaller struct reads its prefix of this one
+  auto kernel = reinterpret_cast<void (*)(BigArgs)>(pair->first);
+  auto set_ids = reinterpret_cast<void (*)(unsigned, unsigned, unsigned, unsigned)>(pair->second);
+  for (unsigned b = 0; b < gx; ++b)
+    for (unsigned t = 0; t < bx; ++t) {
+      set_ids(b, t, bx, gx);
+      kernel(args);
+    }
+  return hipSuccess;
+}
+}
