@@ -17,7 +17,7 @@ def build():
     if OUT.exists() and all(OUT.stat().st_mtime > p.stat().st_mtime for p in srcs + list((ROOT / "i_amd" / "csrc").rglob("*.h"))):
         return OUT
     OUT.parent.mkdir(exist_ok=True)
-    subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-unused-function",
+    subprocess.run(["g++", "-O1", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-unused-function",
                     "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{ROOT / 'include'}",
                     *map(str, srcs), "-o", str(OUT), "-ldl", "-lpthread"], check=True)
     return OUT
