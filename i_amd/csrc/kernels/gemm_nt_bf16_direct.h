@@ -27,6 +27,8 @@
 // operands are one f32 per lane with k = lane / 32: a 16-byte operand read covers k = 4 (2 ks + h) .. + 3,
 // and element e of it feeds MFMA e of the k-step.  Products and sums stay f32.  Requires k % 32 == 0.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 #include "params.h"
 
@@ -119,55 +121,89 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   dma_wait_all();
   __syncthreads();
 
-  // One slab: 4 k-steps of 8 MFMAs.  The operands of k-step ks+1 are fetched while the MFMAs of k-step
-  // ks issue, and the requests for the next slab are dealt out one per MFMA; scheduling fences keep
-  // that order.  The first k-step's operands are fetched right after the barrier.
-  auto fetch = [&](const char* sa, const char* sb, int ks, bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * RB + addr[ks]);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bfr[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
+  // One trip runs from barrier to barrier.  The barrier that publishes slab s sits before the LAST k-step of
+  // slab s-1: that k-step's operands are fetched before the barrier and carried across it in registers, so
+  // the trip opens with MFMAs that need nothing from LDS while the first operands of slab s are on their
+  // way, and the matrix pipe does not drain at the barrier (both waves of a SIMD belong to this workgroup
+  // and reach the barrier together).  Within a trip the operands of the next k-step are fetched while the
+  // MFMAs of the current one issue; the global -> LDS requests for slab s+1 (into the buffer slab s-1 has
+  // just left) ride on the carried MFMAs.  Scheduling fences keep the order.
+  struct Frags {
+    bf16x8 a[TM], b[TN];
   };
-  auto step = [&](uint32_t s, int buf, bool more) {
+  auto fetch = [&](const char* sa, const char* sb, int ks, Frags& f) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * RB + addr[ks]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
+  };
+  auto mfma = [&](const Frags& f, int i, int j) {
+    if constexpr (F32) {
+      const f32x4 av = __builtin_bit_cast(f32x4, f.a[i]), bv = __builtin_bit_cast(f32x4, f.b[j]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[e], bv[e], acc[i][j], 0, 0, 0);
+    } else {
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+    }
+  };
+  static_assert(TM * TN == 2 * WLW, "one slab request per carried MFMA");
+  // The last trip has no successor; it requests its own slab once more into the other buffer, which nobody
+  // reads any more: one redundant slab per workgroup instead of a branch in every slot.
+  auto step = [&](uint32_t s, int buf, const Frags& cin, Frags& cout) {
     const char* sa = &smem[buf][0][0] + a_rows;
     const char* sb = &smem[buf][1][0] + b_rows;
-    const size_t k_byte = (size_t)(s + 1) * RB;
-    bf16x8 af[2][TM], bfr[2][TN];
-    fetch(sa, sb, 0, af[0], bfr[0]);
+    const size_t k_byte = (size_t)(s + 1 < nslabs ? s + 1 : s) * RB;
+    Frags f[2];
+    fetch(sa, sb, 0, f[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 1 < KS) fetch(sa, sb, ks + 1, af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        mfma(cin, i, j);
+        {
+          const int r = i * TN + j, it = r % WLW;
+          const uint32_t w = wave + NWAVES * it;
+          if (r < WLW) dma16(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024);
+          else dma16(b_tile + k_byte, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+    for (int ks = 0; ks + 1 < KS; ++ks) {
+      if (ks + 2 < KS) fetch(sa, sb, ks + 1, f[(ks + 1) & 1]);
+      else fetch(sa, sb, ks + 1, cout);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          if constexpr (F32) {
-            const f32x4 av = __builtin_bit_cast(f32x4, af[ks & 1][i]), bv = __builtin_bit_cast(f32x4, bfr[ks & 1][j]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[e], bv[e], acc[i][j], 0, 0, 0);
-          } else {
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
-          }
-          const int slot = (ks * TM + i) * TN + j;  // 0 .. 31
-          if (more && slot % 2 == 0 && slot / 2 < 2 * WLW) {
-            const int r = slot / 2, it = r % WLW;
-            const uint32_t w = wave + NWAVES * it;
-            if (r < WLW) dma16(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024);
-            else dma16(b_tile + k_byte, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024);
-          }
+          mfma(f[ks & 1], i, j);
           __builtin_amdgcn_sched_barrier(0);
         }
     }
     dma_wait_all();
     __syncthreads();
   };
+  Frags ca, cb;  // the first trip has no predecessor: its carried MFMAs add zero
+#pragma unroll
+  for (int i = 0; i < TM; ++i) ca.a[i] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+#pragma unroll
+  for (int j = 0; j < TN; ++j) ca.b[j] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
   uint32_t s = 0;
-  for (; s + 3 <= nslabs; s += 2) {  // two per trip so that the buffer index is a constant
-    step(s, 0, true);
-    step(s + 1, 1, true);
+  for (; s + 2 <= nslabs; s += 2) {  // two per trip so that the buffer index is a constant
+    step(s, 0, ca, cb);
+    step(s + 1, 1, cb, ca);
   }
-  for (; s < nslabs; ++s) step(s, s & 1, s + 1 < nslabs);
+  if (s < nslabs) {
+    step(s, 0, ca, cb);
+    ca = cb;
+  }
+  // last k-step of the last slab
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) mfma(ca, i, j);
 
   // ---- store.  Accumulator layout: column n = c, rows 8 (e / 4) + 4 h + e % 4: every store instruction
   // writes two full 128-byte lines.  C is written once and not read again: non-temporal.
