@@ -64,20 +64,20 @@ def measured_traffic(summary):
 
 
 def time_steps(torch, fn, steps, warmup):
-    """Wall time over exactly `steps` calls plus per-launch durations from events on the launch stream."""
+    """Wall time per step over exactly `steps` calls, and the average launch duration from one pair of events
+    on the launch stream around the timed region (the launches queue back to back on the stream)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for s in range(steps):
-        starts[s].record()
+    start.record()
+    for _ in range(steps):
         fn()
-        ends[s].record()
+    end.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    kernel_ms = sum(a.elapsed_time(b) for a, b in zip(starts, ends)) / steps
+    kernel_ms = start.elapsed_time(end) / steps
     return wall_ms, kernel_ms
 
 
