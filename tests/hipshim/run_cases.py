@@ -79,6 +79,15 @@ CASES = {
     "fanout two outputs": (lambda: i("+ij~i") & i(">ij~j"), [(9, 14)]),
     "swapped fanout": (lambda: ~(i("+ij~i") & i(">ij~j")), [(9, 14)]),
     "scalar operand": (lambda: i("ij*.~ij"), [(6, 11), ()]),
+    "two-level split mm_t": (lambda: i("ik*jk~ijk | i:4:2,j:8 | jii'i''j'k") >> i("+ijk~ij | i:4:2,j:8 | jii'i''j'k0"), [(37, 12), (21, 12)]),
+    "batched row softmax": (lambda: (((I & i(">bij~bi|i:8|bii'j")) >> i("bij-bi~bij|i:8|bii'1j")) >> i("^bij~bij|i:8|bii'0j")
+                                     >> ((I & i("+bij~bi|i:8|bii'0j")) >> i("bij/bi~bij|i:8|bii'01j"))), [(3, 11, 19)]),
+    "flash i:128,j:64 (dynamic private tiles)": (lambda: flash("i:128,j:64"), [(150, 24), (200, 24), (200, 24)]),
+    "pointwise chain": (lambda: i("ij+ij~ij") >> i("^ij~ij") >> i("$ij~ij"), [(5, 7), (5, 7)]),
+    "comparison and logic": (lambda: (i("ij>>ij~ij") & i("ij<=ij~ij")) >> i("ij^^ij~ij"), [(5, 7), (5, 7)]),
+    "column min": (lambda: i("<ij~j"), [(9, 14)]),
+    "product reduction": (lambda: i("*ij~i"), [(6, 5)]),
+    "rank-3 output": (lambda: i("ik*jk~ijk | i:7 | jii'k"), [(20, 6), (9, 6)]),
     "mlp with pair": (lambda: (i("ij~ij") | ((i("ij*j~ij") >> i("+ij~i")) >> i(">i~i"))) >> (i("ij*j~ij") >> i("+ij~i")),
                       [(7, 16), (16, 8), (8,)]),
 }
