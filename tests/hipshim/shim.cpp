@@ -127,11 +127,16 @@ hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, uns
   // that declares a smaller struct reads its prefix of this one
   auto kernel = reinterpret_cast<void (*)(BigArgs)>(pair->first);
   auto set_ids = reinterpret_cast<void (*)(unsigned, unsigned, unsigned, unsigned)>(pair->second);
-  for (unsigned b = 0; b < gx; ++b)
-    for (unsigned t = 0; t < bx; ++t) {
-      set_ids(b, t, bx, gx);
-      kernel(args);
-    }
+  // ILANG_SHIM_ORDER=reverse runs the work-items last to first: a result that depends on the order in which
+  // work-items run exposes a dependency between them that the parallelisation analysis missed
+  const char* order = std::getenv("ILANG_SHIM_ORDER");
+  const bool reverse = order && std::strcmp(order, "reverse") == 0;
+  const unsigned long total = (unsigned long)gx * bx;
+  for (unsigned long n = 0; n < total; ++n) {
+    const unsigned long id = reverse ? total - 1 - n : n;
+    set_ids((unsigned)(id / bx), (unsigned)(id % bx), bx, gx);
+    kernel(args);
+  }
   return hipSuccess;
 }
 }

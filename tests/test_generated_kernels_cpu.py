@@ -45,6 +45,12 @@ def test_generated_kernels_split_into_phases_match_too(shim_lib):
     run_cases(shim_lib, {"ILANG_HIP_PHASES": "1"})
 
 
+def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
+    """Work-items run last to first: a dependency between work-items would change the result."""
+    run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse"})
+    run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
+
+
 def test_phase_plan_is_reported(shim_lib):
     env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_NO_TORCH="1")
     code = ("from i_amd import Component as i, I\n"
