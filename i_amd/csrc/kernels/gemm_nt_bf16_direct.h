@@ -32,14 +32,16 @@
 #include "common.h"
 #include "params.h"
 
-template <bool F32>
+// BT x BT output tile per workgroup of WM x WN waves: 256 with 2 x 4 waves (one workgroup per CU) for large
+// problems, 128 with 2 x 2 waves (two workgroups per CU) for problems with too few 256-tiles to fill the chip.
+template <bool F32, int BT, int WM, int WN>
 __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
-  constexpr int BMT = 256, BNT = 256;
+  constexpr int BMT = BT, BNT = BT;
   constexpr int ELEM = F32 ? 4 : 2;   // bytes per operand element
   constexpr int BK = 128 / ELEM;      // k per slab: 128-byte slab rows
-  constexpr int WM = 2, WN = 4, NWAVES = WM * WN;
-  constexpr int TM = BMT / WM / 32;  // 4
-  constexpr int TN = BNT / WN / 32;  // 2
+  constexpr int NWAVES = WM * WN;
+  constexpr int TM = BMT / WM / 32;  // 32-row accumulator tiles per wave
+  constexpr int TN = BNT / WN / 32;
   constexpr int RB = ELEM * BK;      // bytes per slab row
   constexpr int CH = RB / 16;        // chunks per row (= lanes per row of a wave-load)
   constexpr int RPW = 64 / CH;       // rows per wave-load
@@ -47,7 +49,7 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   constexpr int WL = SLAB / 1024;    // wave-loads per slab
   constexpr int WLW = WL / NWAVES;   // ... per wave
   constexpr int KS = RB / 32;        // k-steps per slab: two 16-byte chunks (one per half-wave) each
-  static_assert(BMT == BNT && WL % NWAVES == 0, "slab shape");
+  static_assert(BMT == BNT && WL % NWAVES == 0 && NWAVES % 2 == 0, "slab shape");
   __shared__ __attribute__((aligned(1024))) char smem[2][2][SLAB];  // [buffer][A, B]
 
   // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
@@ -146,7 +148,7 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
     }
   };
-  static_assert(TM * TN == 2 * WLW, "one slab request per carried MFMA");
+  constexpr int NREQ = 2 * WLW;  // slab requests per wave and trip, dealt out over the TM * TN carried MFMAs
   // The last trip has no successor; it requests its own slab once more into the other buffer, which nobody
   // reads any more: one redundant slab per workgroup instead of a branch in every slot.
   auto step = [&](uint32_t s, int buf, const Frags& cin, Frags& cout) {
@@ -161,8 +163,10 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         mfma(cin, i, j);
-        {
-          const int r = i * TN + j, it = r % WLW;
+        const int slot = i * TN + j;
+#pragma unroll
+        for (int r = slot * NREQ / (TM * TN); r < (slot + 1) * NREQ / (TM * TN); ++r) {
+          const int it = r % WLW;
           const uint32_t w = wave + NWAVES * it;
           if (r < WLW) dma16(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024);
           else dma16(b_tile + k_byte, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024);

@@ -44,11 +44,18 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64(Gem
 }
 
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct(GemmParams p) {
-  gemm_nt_direct_body<false>(p);
+  gemm_nt_direct_body<false, 256, 2, 4>(p);
+}
+// 128 x 128 tiles, 4 waves, two workgroups per CU: mid-size problems
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64_direct(GemmParams p) {
+  gemm_nt_direct_body<false, 128, 2, 2>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_direct(GemmParams p) {
+  gemm_nt_direct_body<true, 128, 2, 2>(p);
 }
 // f32 operands, f32 MFMA: the arithmetic type of the reference
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_direct(GemmParams p) {
-  gemm_nt_direct_body<true>(p);
+  gemm_nt_direct_body<true, 256, 2, 4>(p);
 }
 
 #define SOFTMAX_WAVE(NV)                                                                          \

@@ -89,25 +89,32 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
-  // Large problems: 256 x 256 tiles with direct global -> LDS slabs (needs whole 64-wide k slabs and 32-bit
-  // byte offsets inside a tile's 256 rows).  Its prologue and its unoverlapped store only pay off for a long
-  // k loop on a grid that fills at least half of the CUs.  ILANG_GEMM_DIRECT=1 / 0 forces / forbids it, so
-  // that tests can reach both kernels at small sizes.
+  // Direct global -> LDS kernels (need whole 64-wide k slabs and 32-bit byte offsets inside a tile's rows):
+  //   256 x 256 tiles  long k loops on grids that fill at least half of the CUs (its prologue and its
+  //                    unoverlapped store only pay off there)
+  //   128 x 128 tiles  problems with too few 256-tiles, two workgroups per CU
+  // and the register-staged 128 x 128 kernel for everything else (k % 8 == 0, short k, tiny grids).
+  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; ILANG_GEMM_DIRECT=256 | 128 | 0
+  // forces a kernel so that tests can reach each of them at small sizes (1 is read as 256).
   {
-    const size_t tm = (m + 255) / 256, tn = (n + 255) / 256;
-    bool direct = k >= 512 && tm * tn * bh >= 128;
-    if (tile_m == 256 && tile_n == 256) direct = true;   // the schedule's i, j splits
-    if (tile_m == 128 && tile_n == 128) direct = false;
-    if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) direct = f[0] == '1';
-    if (direct && k % 64 == 0 && k <= (size_t(1) << 22) && bh <= 65535) {
-      p.tiles_m = (uint32_t)tm;
-      p.tiles_n = (uint32_t)tn;
-      const size_t nsb = ((tm + 3) / 4) * ((tn + 7) / 8);  // super-blocks of 4 x 8 tiles, dealt to the 8 XCDs
+    const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
+    unsigned tile = 0;  // 0: register-staged kernel
+    if (k >= 512 && t256 >= 128) tile = 256;
+    else if (k >= 256 && t128 >= 64) tile = 128;
+    if (tile_m == 256 && tile_n == 256) tile = 256;
+    if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
+    if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
+    if (tile && k % 64 == 0 && k <= (size_t(1) << 22) && bh <= 65535) {
+      p.tiles_m = (uint32_t)((m + tile - 1) / tile);
+      p.tiles_n = (uint32_t)((n + tile - 1) / tile);
+      const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs
       const size_t grid = ((nsb + 7) / 8 * 8) * 32;
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
-      if (Err e = builtin_function("gemm_nt_bf16_256x256x64_direct", &fn); !e.empty()) return e;
-      return launch(fn, (unsigned)grid, (unsigned)bh, 1, 512, &p, sizeof(p), stream);
+      if (Err e = builtin_function(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct", &fn);
+          !e.empty())
+        return e;
+      return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
     }
   }
   p.tiles_m = (uint32_t)((m + 127) / 128);
@@ -131,14 +138,20 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
-  p.tiles_m = (uint32_t)((m + 255) / 256);
-  p.tiles_n = (uint32_t)((n + 255) / 256);
-  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // super-blocks of 4 x 8 tiles
+  // 256 x 256 tiles when they fill at least half of the CUs, 128 x 128 tiles otherwise
+  const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
+  unsigned tile = t256 >= 128 ? 256 : 128;
+  if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = std::atoi(f) == 128 ? 128 : 256;
+  p.tiles_m = (uint32_t)((m + tile - 1) / tile);
+  p.tiles_n = (uint32_t)((n + tile - 1) / tile);
+  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks
   const size_t grid = ((nsb + 7) / 8 * 8) * 32;
   if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
   hipFunction_t fn;
-  if (Err e = builtin_function("gemm_nt_f32_256x256x32_direct", &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, (unsigned)bh, 1, 512, &p, sizeof(p), stream);
+  if (Err e = builtin_function(tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct", &fn);
+      !e.empty())
+    return e;
+  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream) {

@@ -267,10 +267,11 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
                                       (3, 257, 255, 320)])
-@pytest.mark.parametrize("direct", ["1", "0"])
-def test_gemm_nt_bf16_both_kernels_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
-    """The launcher picks the 256 x 256 direct-to-LDS kernel for long-k problems on big grids; force it (and
-    forbid it) on small ragged problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
+@pytest.mark.parametrize("direct", ["256", "128", "0"])
+def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
+    """The launcher picks between the 256 x 256 and 128 x 128 direct-to-LDS kernels and the register-staged
+    kernel by problem size; force each of them on small ragged problems with 1 to 5 k-slabs, edge tiles on
+    both axes and several batches."""
     monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
@@ -284,8 +285,10 @@ def test_gemm_nt_bf16_both_kernels_vs_oracle(env, monkeypatch, bh, m, n, k, dire
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 32), (1, 300, 260, 96), (2, 600, 520, 160), (1, 1, 1, 64),
                                       (3, 257, 255, 320), (1, 100, 70, 64)])
-def test_gemm_nt_f32_vs_oracle(env, bh, m, n, k):
+@pytest.mark.parametrize("tile", ["256", "128"])
+def test_gemm_nt_f32_vs_oracle(env, monkeypatch, bh, m, n, k, tile):
     """f32 operands, f32 MFMA: the reference's own arithmetic type, against the scalar oracle at the f32 bar."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile)
     t = env.torch
     a, b = rnd((bh, m, k), 1, "uniform"), rnd((bh, n, k), 2, "uniform")
     ad, bd = t.from_numpy(a).cuda(), t.from_numpy(b).cuda()
