@@ -43,6 +43,17 @@ def flash_component(i, I, split):
     return mm_t >> scale >> row_max_shift >> exp >> row_normalize >> mm
 
 
+def flash_demo_component(i, I):
+    # the demo's strings (ilang-python/flash-attn.py:45-53): single head, no score scale
+    s = "i:16,j:16"
+    mm_t = i(f"ik*jk~ijk | {s} | jii'j'k") >> i(f"+ijk~ij | {s} | jii'j'k0")
+    row_max_shift = (I & i(f">ij~i | {s} | ji0i'j'")) >> i(f"ij-i~ij | {s} | ji01i'j'")
+    exp = i(f"^ij~ij | {s} | ji0i'j'")
+    row_normalize = (I & i(f"+ij~i | {s} | ji0i'j'")) >> i(f"ij/i~ij | {s} | ji01i'j'")
+    mm = i(f"ij*jk~ikj | {s} | ji0i'kj'") >> i(f"+ikj~ik | {s} | jii'kj'0")
+    return mm_t >> row_max_shift >> exp >> row_normalize >> mm
+
+
 def softmax_component(i, I):
     # row-staged single-kernel schedule: max and sum fold to scalars, the row stays on chip
     return (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
@@ -170,6 +181,34 @@ def main():
                       f"16x16 tiles as in the reference demo; GPU vs oracle on those slices: rel err {rel:.1e}",
         }
 
+    # ---- the reference's own CPU-runnable case (BASELINE configs[0]): demo attention, f32 [512,64], no scale,
+    # i:16,j:16 schedule; on the GPU through the f32 kernel, on the host through the reference's emitted C
+    # (oracle/_ref, compiled from the reference tree when it was mounted at build time) or the oracle port
+    c1 = None
+    if not args.no_cpu_baseline:
+        import oracle
+
+        rng = [np.random.default_rng(sd).uniform(-1, 1, (512, 64)).astype(np.float32) for sd in (1, 2, 3)]
+        demo = flash_demo_component(i, I)
+        dq, dk, dv_ = (torch.from_numpy(a).to(dev) for a in rng)
+        dout = torch.empty(512, 64, device=dev)
+        demo.into(dout, dq, dk, dv_)
+        _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), 50, 5)
+        use_ref = oracle.have_ref()
+        host = (lambda: oracle.ref_flash_attention(*rng)) if use_ref else (lambda: oracle.attention_tiled(*rng))
+        host()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            ref1 = host()
+        c1_cpu_s = (time.perf_counter() - t0) / 5
+        c1_flop = 4.0 * 512 * 512 * 64
+        c1_rel = float(np.abs(dout.cpu().numpy() - ref1).max() / np.abs(ref1).max())
+        c1 = {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
+              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": c1_ms,
+              "cpu_baseline": {"value": c1_flop / c1_cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1,
+                               "kind": "reference" if use_ref else "port",
+                               "sample": f"the whole workload, {c1_cpu_s * 1e3:.1f} ms per run; GPU vs host rel err {c1_rel:.1e}"}}
+
     line = {
         "metric": "attn TFLOP/s & %MFMA peak (B8,H32,N4096,d128); row-softmax HBM GB/s",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -203,7 +242,7 @@ def main():
                           "frac": c5_tflops / PEAK_BF16_TFLOPS,
                           "traffic": measured_traffic("flash_attention_B1_H16_N32768_d64_bf16.md"),
                           "kernel": "attn_fwd_bf16_d64_bn64_direct", "kernel_ms": c5_ms}},
-        ],
+        ] + ([c1] if c1 else []),
     }
     print(json.dumps(line))
 
