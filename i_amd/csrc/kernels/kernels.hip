@@ -30,6 +30,9 @@ ATTN_BF16_DIRECT(128, 64, 4, 2)
 extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d128_bn64_direct_w8(AttnParams p) {
   attn_fwd_bf16_direct_body<128, 64, 8>(p);
 }
+extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn64_direct_w8(AttnParams p) {
+  attn_fwd_bf16_direct_body<64, 64, 8>(p);
+}
 
 #define ATTN_F32(DPAD, BN, NW)                                                             \
   extern "C" __global__ void __launch_bounds__(NW * 64) attn_fwd_f32_d##DPAD##_bn##BN(AttnParams p) { \

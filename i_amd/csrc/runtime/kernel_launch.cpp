@@ -34,17 +34,17 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 
   const size_t dmax = d > dv ? d : dv;
   // Kernel choice for bf16:
-  //   d == dv in {64, 128}: direct-to-LDS kernel; for d = 128 a 256-query workgroup (8 waves) halves the
+  //   d == dv in {64, 128}: direct-to-LDS kernel; a 256-query workgroup (8 waves) halves the
   //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
   //     larger workgroup is used when it still leaves at least two workgroups per CU
   //   otherwise: register-staged kernel with guarded columns
-  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the d = 128 direct kernel and ILANG_ATTN_NO_DIRECT=1
+  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the direct kernel and ILANG_ATTN_NO_DIRECT=1
   // forces the register-staged kernel; both exist so that tests can reach every kernel with small inputs.
   unsigned bm = 128;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
   const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
-  if (direct && d == 128) {
+  if (direct) {
     if (query_tile == 128 || query_tile == 256) bm = (unsigned)query_tile;  // the schedule's i split
     else if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
@@ -64,7 +64,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   const char* name;
   if (in_dtype == BF16) {
     if (direct)
-      name = d == 64 ? "attn_fwd_bf16_d64_bn64_direct" : bm == 256 ? "attn_fwd_bf16_d128_bn64_direct_w8" : "attn_fwd_bf16_d128_bn64_direct";
+      name = d == 64 ? (bm == 256 ? "attn_fwd_bf16_d64_bn64_direct_w8" : "attn_fwd_bf16_d64_bn64_direct")
+                     : (bm == 256 ? "attn_fwd_bf16_d128_bn64_direct_w8" : "attn_fwd_bf16_d128_bn64_direct");
     else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   }

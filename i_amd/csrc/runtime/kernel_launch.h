@@ -14,7 +14,7 @@ enum DType { F32 = 0, BF16 = 1 };
 // in_dtype applies to q, k, v; out_dtype to o (F32 or BF16; BF16 only with bf16 inputs).
 // scale_ptr, when given, is a rank-0 f32 operand in device memory, read by the kernel.
 // query_tile is the query-row tile the schedule asks for (the product of the split factors of the row
-// index; 0 = no preference): 128 and 256 select the 4- and 8-wave workgroup of the d = 128 kernel, any other
+// index; 0 = no preference): 128 and 256 select the 4- and 8-wave workgroup of the direct-to-LDS kernel, any other
 // value leaves the choice to the launcher.
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
