@@ -109,6 +109,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   float l_run = 0.0f;       // running sum over this half-wave's keys
   float mb_run = 0.0f;      // m_run * scale_log2, kept while the steady-state loop runs
 
+  const uint32_t nfull_tiles = p.nk / BN;  // tiles that lie entirely inside nk
   // ---- global -> LDS: this lane's slot in wave-load w is tile row w*RPW + lane/CH, chunk lane%CH
   const uint32_t lrow = lane / CH, lch = lane % CH;
   const uint32_t smem0 = lds_address(&smem[0][0][0]);
@@ -126,6 +127,20 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     const size_t byte0 = (size_t)tile * TILE_BYTES + w * 1024;
     if constexpr (decltype(want_k)::value) dma16(K + byte0, koff_lane, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
     else dma16(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+  };
+
+  // one wave-load of K of any tile index: full tile, partial tile (rows past nk re-read the last row), or none
+  auto request_k_one = [&](uint32_t tile, int buf, int it) {
+    if (tile < nfull_tiles) {
+      const uint32_t w = wave + NWAVES * it;
+      dma16(K + (size_t)tile * TILE_BYTES + w * 1024, koff_lane, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+    } else if (tile * BN < p.nk) {
+      const uint32_t w = wave + NWAVES * it;
+      const uint32_t row = w * RPW + lrow;
+      uint32_t key = tile * BN + row;
+      key = key < p.nk ? key : p.nk - 1;
+      dma16(K, key * RB + 16 * (lch ^ ((row / RPB) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+    }
   };
 
   // PARTIAL: the tile runs past nk; rows past the end re-read the last row (their scores are masked).
@@ -317,7 +332,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // max, O and l are corrected by the exp-shift factor, and the tile's probabilities are recomputed.
   constexpr float SUM_GUARD = 1099511627776.0f;  // 2^40
 
-  auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], const Carry& cin, Carry& cout) {
+  // any_k_tag: tile j+2 may be partial or absent (the last steady-state trip); otherwise it is a full tile
+  auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], const Carry& cin, Carry& cout,
+                       auto any_k_tag) {
     const char* sk = &smem[buf ^ 1][0][0];  // K(j+1)
     const char* sv = &smem[buf][1][0];      // V(j)
 
@@ -346,8 +363,12 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     // request g of the 2 WLW global -> LDS requests of the trip
     auto request_for_slot = [&](int g) {
       if (g < 2 * WLW) {
-        if (g < WLW) request_full_one(j + 2, buf, g, Yes{});
-        else request_full_one(j + 1, buf ^ 1, g - WLW, No{});
+        if (g < WLW) {
+          if constexpr (decltype(any_k_tag)::value) request_k_one(j + 2, buf, g);
+          else request_full_one(j + 2, buf, g, Yes{});
+        } else {
+          request_full_one(j + 1, buf ^ 1, g - WLW, No{});
+        }
       }
     };
 
@@ -450,8 +471,16 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     for (int t = 0; t < DT; ++t) ca.a[t] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
     ca.p = u32x4{0, 0, 0, 0};
     for (; j + 4 <= nfull; j += 2) {  // j + 3 <= nfull - 1
-      fast_step(j, 0, sa, sb, ca, cb);
-      fast_step(j + 1, 1, sb, sa, cb, ca);
+      fast_step(j, 0, sa, sb, ca, cb, No{});
+      fast_step(j + 1, 1, sb, sa, cb, ca, No{});
+    }
+    // one more trip: tile j+1 is still a full tile, tile j+2 may be partial or absent
+    {
+      fast_step(j, 0, sa, sb, ca, cb, Yes{});
+      ++j;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) sa[kt] = sb[kt];
+      ca = cb;
     }
     // last key group of the last steady-state tile
 #pragma unroll
