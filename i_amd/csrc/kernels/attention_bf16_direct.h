@@ -305,9 +305,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   //   DT slots       last 16-key group of O += V(j-1)^T P(j-1)^T, operands and probabilities carried in
   //                  registers across the barrier
   //   NQK slots      S(j+1) = K(j+1) Q^T
-  //                  (these DT + NQK slots also carry the global -> LDS requests for K(j+2), V(j+1) and all of
-  //                  P(j) = exp(S(j) - reference), its bf16 rounding and the row sum)
+  //                  (these DT + NQK slots also carry the global -> LDS requests for K(j+2), V(j+1) and the
+  //                  second half of P(j) = exp(S(j) - reference), its bf16 rounding and the row sum)
   //   NPV - DT slots O += V(j)^T P(j)^T for all but the last 16-key group
+  //                  (from the second key group on, these slots carry the first half of P(j+1): S(j+1) is
+  //                  complete by then, and a group's registers are free once its MFMAs have been issued)
   // LDS operands are fetched in slot order, DT + ATTN_XLEAD slots ahead of their MFMA; the fetches for
   // the carried group are the last ones before the barrier, so the barrier sits in the middle of a
   // stream of MFMAs instead of at a point where the matrix pipe has drained.
@@ -331,6 +333,26 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // not below 2^40 (this includes inf and NaN) for any row of the wave, the reference is moved up to the tile
   // max, O and l are corrected by the exp-shift factor, and the tile's probabilities are recomputed.
   constexpr float SUM_GUARD = 1099511627776.0f;  // 2^40
+
+  // packed probability pairs: pq[g][w] holds scores 2 (4 g + w), + 1 of the lane in (kt, i) order, so pq[g] is
+  // the B operand of 16-key group g.  The empty asm statement ties the pair's vector work to the slot it is
+  // written in.  pq and the row-sum parts live across trips: the first NEARLY pairs of a tile (its key groups 0
+  // and 1) are computed one trip early, in the output slots of the previous tile, which otherwise carry no
+  // vector work at all, while the score slots are the crowded ones.
+  constexpr int NEARLY = 8;
+  u32x4 pq[NPAIR / 4];
+  float psum[2] = {0.0f, 0.0f};
+  const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+  auto exp_pair_from = [&](const f32x16 (&s)[KT], int pr, float mb) {
+    const int pkt = pr / 8, i = 2 * (pr % 8);
+    const float e0 = fast_exp2(__builtin_fmaf(s[pkt][i], scale_log2, -mb));
+    const float e1 = fast_exp2(__builtin_fmaf(s[pkt][i + 1], scale_log2, -mb));
+    const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
+    psum[pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[pr & 1], false);
+    uint32_t packed = __builtin_bit_cast(uint32_t, pair);
+    asm volatile("" : "+v"(packed), "+v"(psum[pr & 1]));
+    pq[pr / 4][pr % 4] = packed;
+  };
 
   // any_k_tag: tile j+2 may be partial or absent (the last steady-state trip); otherwise it is a full tile
   auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[KT], f32x16 (&s_next)[KT], const Carry& cin, Carry& cout,
@@ -372,25 +394,12 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       }
     };
 
-    // packed probability pairs: pq[g][w] holds scores 2 (4 g + w), + 1 of the lane in (kt, i) order, so pq[g] is
-    // the B operand of 16-key group g.  The empty asm statements tie each slot's vector work to its slot.
-    u32x4 pq[NPAIR / 4];
-    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
-    float psum[2] = {0.0f, 0.0f};
+    // pairs NEARLY .. NPAIR - 1 of tile j (pairs 0 .. NEARLY - 1 were computed during the previous trip)
     float mb = mb_run;
-    auto exp_pair = [&](int pr) {
-      const int pkt = pr / 8, i = 2 * (pr % 8);
-      const float e0 = fast_exp2(__builtin_fmaf(s_cur[pkt][i], scale_log2, -mb));
-      const float e1 = fast_exp2(__builtin_fmaf(s_cur[pkt][i + 1], scale_log2, -mb));
-      const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
-      psum[pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[pr & 1], false);
-      uint32_t packed = __builtin_bit_cast(uint32_t, pair);
-      asm volatile("" : "+v"(packed), "+v"(psum[pr & 1]));
-      pq[pr / 4][pr % 4] = packed;
-    };
     auto pairs_for_slot = [&](int g) {
 #pragma unroll
-      for (int pr = g * NPAIR / NPRE; pr < (g + 1) * NPAIR / NPRE; ++pr) exp_pair(pr);
+      for (int pr = NEARLY + g * (NPAIR - NEARLY) / NPRE; pr < NEARLY + (g + 1) * (NPAIR - NEARLY) / NPRE; ++pr)
+        exp_pair_from(s_cur, pr, mb);
     };
 
     // ---- carried slots: last key group of tile j-1
@@ -435,9 +444,10 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       mb = mb_new;
       psum[0] = psum[1] = 0.0f;
 #pragma unroll
-      for (int pr = 0; pr < NPAIR; ++pr) exp_pair(pr);
+      for (int pr = 0; pr < NPAIR; ++pr) exp_pair_from(s_cur, pr, mb);
     }
     l_run += psum[0] + psum[1];
+    psum[0] = psum[1] = 0.0f;
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- output slots of tile j, all key groups but the last
@@ -446,6 +456,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       fetch_for_slot(DT + NQK + m);
       const int s4 = m / DT, t = m % DT;
       o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[NQK + m], __builtin_bit_cast(bf16x8, pq[s4]), o[t], 0, 0, 0);
+      // key groups 0 and 1 of tile j+1, each once the MFMAs that read the group's old registers have been issued
+      if (m >= DT && m < 3 * DT) {
+#pragma unroll
+        for (int pr = (m - DT) * 4 / DT; pr < (m - DT + 1) * 4 / DT; ++pr) exp_pair_from(s_next, pr, mb);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -465,6 +480,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
     m_run = half_max(mx_tile);
     mb_run = m_run * scale_log2;
+#pragma unroll
+    for (int pr = 0; pr < NEARLY; ++pr) exp_pair_from(sa, pr, mb_run);
     // the first trip has no predecessor: its carried slots add zero
     Carry ca, cb;
 #pragma unroll
