@@ -1,0 +1,51 @@
+"""bench.py's command line and the one JSON line it prints."""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr
+    assert r.stdout.strip() == ""
+
+
+def test_committed_profile_summaries_give_the_traffic_figures():
+    sys.path.insert(0, str(ROOT))
+    import bench
+
+    for name in ("flash_attention_B8_H32_N4096_d128_bf16.md", "row_softmax_16384x4096_f32.md",
+                 "gemm_nt_4096x4096x4096_bf16.md", "flash_attention_B1_H16_N32768_d64_bf16.md"):
+        traffic = bench.measured_traffic(name)
+        assert isinstance(traffic, int) and traffic > 0, name
+    assert bench.measured_traffic("no_such_summary.md") is None
+
+
+@pytest.mark.gpu
+def test_one_json_line_with_roofline_and_cpu_baseline():
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--steps", "2", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 2 and rec["warmup"] == 1
+    assert rec["unit"] == "TFLOP/s" and rec["dtype"] == "bf16" and rec["vs_baseline"] is None
+    assert "workload" in rec["config"] and "model" not in rec["config"]
+    roof = rec["roofline"]
+    assert roof["bound"] == "mfma" and roof["unit"] == "TFLOP/s" and roof["peak"] == 2500.0
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
+    cpu = rec["cpu_baseline"]
+    assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    # the value is work over wall time of exactly `steps` calls
+    flop = 4.0 * 8 * 32 * 4096 * 4096 * 128
+    assert abs(rec["value"] - flop / (rec["ms_per_step"] * 1e-3) / 1e12) / rec["value"] < 1e-6
