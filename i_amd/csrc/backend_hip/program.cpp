@@ -142,6 +142,13 @@ bool hand_usable(const Run& run, const Recognized& r) {
       if (a.size() < 2) return false;
       return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
     }
+    case Recognized::GemmNN: {
+      const DType t = run.dtype_of(r.a.buffer);
+      if (run.dtype_of(r.b.buffer) != t) return false;
+      const auto a = rows_cols(r.a);
+      if (a.size() < 2) return false;
+      return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
+    }
     case Recognized::RowSoftmax: return true;
   }
   return false;
@@ -210,6 +217,30 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
                                         a[nb], b[nb], a[nb + 1], run.stream);
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
                                        a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j);
+    }
+    case Recognized::GemmNN: {
+      // b [B.., K, J] is transposed into a stream-ordered temporary [B.., J, K], then the NT kernel runs
+      const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
+      const size_t nb = r.batch_rank;
+      size_t bh = 1;
+      for (size_t d = 0; d < nb; ++d) {
+        if (b[d] != a[d]) return "gemm operands disagree on a batch extent";
+        bh *= a[d];
+      }
+      const size_t m = a[nb], k = a[nb + 1], n = b[nb + 1];
+      if (b[nb] != k) return "gemm operands disagree on the contracted extent";
+      const bool f32 = run.dtype_of(r.a.buffer) == DType::F32;
+      const size_t elem = f32 ? 4 : 2;
+      void* bt = nullptr;
+      if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;
+      if (ihip::Err e = ihip::launch_transpose(run.raw_ptr(r.b.buffer), bt, bh, k, n, elem, run.stream); !e.empty()) return e;
+      void* out = nullptr;
+      if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+      if (f32)
+        return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)), static_cast<const float*>(bt),
+                                        static_cast<float*>(out), bh, m, n, k, run.stream);
+      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, static_cast<float*>(out), bh, m, n, k, run.stream,
+                                       r.tile_i, r.tile_j);
     }
     case Recognized::RowSoftmax: {
       const auto x = run.shape_of(r.a.buffer);

@@ -102,6 +102,35 @@ struct Matcher {
   Operand operand(const Arg& a) const { return {refs[a.kp_buffer], a.dims}; }
 
   // S = sum_D q[B.., I, D] * k[B.., J, D], output dims [B.., I, J]
+  // sum_D a[B.., I, D] * b[B.., D, J]  (either operand order)
+  bool match_mm(int t, Recognized& r) const {
+    const Term& add = T(t);
+    if (add.op != Op::Add || add.red.size() != 1 || add.args.size() != 1 || add.args[0].external) return false;
+    if (add.out.size() < 2) return false;
+    const Term& mul = T(add.args[0].term);
+    if (mul.op != Op::Mul || !mul.red.empty() || mul.args.size() != 2) return false;
+    if (!mul.args[0].external || !mul.args[1].external) return false;
+    const int D = add.red[0];
+    const size_t nb = add.out.size() - 2;
+    const int I = add.out[nb], J = add.out[nb + 1];
+    std::vector<int> left(add.out.begin(), add.out.begin() + nb), right = left;
+    left.push_back(I);
+    left.push_back(D);
+    right.push_back(D);
+    right.push_back(J);
+    if (mul.args[0].dims == left && mul.args[1].dims == right) {
+      r.a = operand(mul.args[0]);
+      r.b = operand(mul.args[1]);
+    } else if (mul.args[1].dims == left && mul.args[0].dims == right) {
+      r.a = operand(mul.args[1]);
+      r.b = operand(mul.args[0]);
+    } else {
+      return false;
+    }
+    r.batch_rank = nb;
+    return true;
+  }
+
   bool match_qk(int t, Recognized& r) const {
     const Term& add = T(t);
     if (add.op != Op::Add || add.red.size() != 1 || add.args.size() != 1 || add.args[0].external) return false;
@@ -201,6 +230,12 @@ struct Matcher {
     }
     r = Recognized{};
     r.out = out;
+    if (match_mm(root, r)) {
+      r.kind = Recognized::GemmNN;
+      return r;
+    }
+    r = Recognized{};
+    r.out = out;
 
     // row softmax over an operand buffer
     {
@@ -260,6 +295,7 @@ std::string Recognized::describe() const {
   switch (kind) {
     case Attention: return (has_scale ? "hand-written FlashAttention kernel (scaled scores)" : "hand-written FlashAttention kernel") + tiles;
     case GemmNT: return "hand-written MFMA GEMM (transposed right operand)" + tiles;
+    case GemmNN: return "hand-written MFMA GEMM (right operand transposed on the device first)" + tiles;
     case RowSoftmax: return "hand-written row-softmax kernel";
     default: return "generated HIP kernel";
   }
@@ -287,7 +323,7 @@ std::vector<Recognized> recognize_kernels(const Lowered& low) {
     const int root = tb.build(stage, {});
     Matcher m{tb, refs};
     Recognized rec = m.match_root(root, refs[sp.graph.inputs + stage]);
-    if (rec.kind == Recognized::Attention || rec.kind == Recognized::GemmNT) {
+    if (rec.kind == Recognized::Attention || rec.kind == Recognized::GemmNT || rec.kind == Recognized::GemmNN) {
       // the schedule's tile sizes, read off the root stage: its output is [B.., I, E] (attention, J reduced)
       // or [B.., I, J] (GEMM)
       const Stage& st = sp.graph.nodes[stage].inner;
@@ -303,7 +339,7 @@ std::vector<Recognized> recognize_kernels(const Lowered& low) {
       const auto& shape = st.output.shape;
       if (shape.size() >= 2) {
         rec.tile_i = tile_of(shape[shape.size() - 2]);
-        if (rec.kind == Recognized::GemmNT) rec.tile_j = tile_of(shape.back());
+        if (rec.kind != Recognized::Attention) rec.tile_j = tile_of(shape.back());
         else
           for (const SAxis& a : st.axes)
             if (std::find(shape.begin(), shape.end(), a.index) == shape.end()) rec.tile_j = tile_of(a.index);

@@ -21,9 +21,10 @@ struct Operand {
 };
 
 struct Recognized {
-  enum Kind { None, Attention, GemmNT, RowSoftmax } kind = None;
+  enum Kind { None, Attention, GemmNT, GemmNN, RowSoftmax } kind = None;
   // Attention: q [B.., I, D], k [B.., J, D], v [B.., J, E] -> out [B.., I, E]; optional scalar scale
   // GemmNT:    a [B.., I, K], b [B.., J, K] -> out [B.., I, J]
+  // GemmNN:    a [B.., I, K], b [B.., K, J] -> out [B.., I, J]
   // RowSoftmax: x [R.., J] -> out [R.., J]
   Operand a, b, c;             // q,k,v | a,b,- | x,-,-
   bool has_scale = false;
@@ -31,7 +32,7 @@ struct Recognized {
   ic::BufferRef out;
   size_t batch_rank = 0;       // number of leading shared dims
   // Tile sizes the schedule asks for (product of the split factors of the index in the kernel's root
-  // stage, 0 when the index is not split): Attention: query rows I / keys J; GemmNT: rows I / columns J.
+  // stage, 0 when the index is not split): Attention: query rows I / keys J; GemmNT, GemmNN: rows I / columns J.
   size_t tile_i = 0, tile_j = 0;
   std::string describe() const;
 };

@@ -89,3 +89,26 @@ extern "C" __global__ void __launch_bounds__(256) convert_bf16_to_f32(ConvertPar
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < p.n; i += (uint64_t)gridDim.x * blockDim.x)
     d[i] = (float)s[i];
 }
+
+// Batched matrix transpose through a padded 64 x 64 LDS tile (reads and writes both run along rows).  It feeds
+// the NT GEMM kernels with the right operand of an NN product.
+template <typename T>
+__device__ __forceinline__ void transpose_body(const TransposeParams& p) {
+  __shared__ T tile[64][65];
+  const uint32_t per_batch = p.tiles_r * p.tiles_c;
+  const uint32_t b = blockIdx.x / per_batch, t = blockIdx.x % per_batch;
+  const uint32_t r0 = (t / p.tiles_c) * 64, c0 = (t % p.tiles_c) * 64;
+  const T* src = reinterpret_cast<const T*>(p.src) + (size_t)b * p.rows * p.cols;
+  T* dst = reinterpret_cast<T*>(p.dst) + (size_t)b * p.rows * p.cols;
+  const uint32_t x = threadIdx.x & 63, y0 = threadIdx.x >> 6;
+#pragma unroll 4
+  for (uint32_t y = y0; y < 64; y += 4)
+    if (r0 + y < p.rows && c0 + x < p.cols) tile[y][x] = src[(size_t)(r0 + y) * p.cols + c0 + x];
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t y = y0; y < 64; y += 4)
+    if (c0 + y < p.cols && r0 + x < p.rows) dst[(size_t)(c0 + y) * p.rows + r0 + x] = tile[x][y];
+}
+extern "C" __global__ void __launch_bounds__(256) transpose_b16(TransposeParams p) { transpose_body<uint16_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) transpose_b32(TransposeParams p) { transpose_body<uint32_t>(p); }
+

@@ -37,3 +37,12 @@ struct ConvertParams {
   void* dst;
   uint64_t n;
 };
+
+// dst[b][c][r] = src[b][r][c] for b < bh, r < rows, c < cols; elements of 2 or 4 bytes
+struct TransposeParams {
+  const void* src;
+  void* dst;
+  uint32_t bh, rows, cols;
+  uint32_t tiles_r, tiles_c;  // 64 x 64 tiles
+};
+

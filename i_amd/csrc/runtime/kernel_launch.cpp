@@ -176,6 +176,24 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
   return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
 }
 
+Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,
+                     hipStream_t stream) {
+  if (elem_bytes != 2 && elem_bytes != 4) return "transpose kernel: element size must be 2 or 4 bytes";
+  if (bh == 0 || rows == 0 || cols == 0) return {};
+  if (!fits_u32(bh) || !fits_u32(rows) || !fits_u32(cols)) return "transpose kernel: extent exceeds 32 bits";
+  if (!src || !dst) return "transpose kernel: null device pointer";
+  TransposeParams p{};
+  p.src = src; p.dst = dst;
+  p.bh = (uint32_t)bh; p.rows = (uint32_t)rows; p.cols = (uint32_t)cols;
+  p.tiles_r = (uint32_t)((rows + 63) / 64);
+  p.tiles_c = (uint32_t)((cols + 63) / 64);
+  const size_t grid = bh * p.tiles_r * p.tiles_c;
+  if (grid > kMaxGrid) return "transpose kernel: grid too large";
+  hipFunction_t fn;
+  if (Err e = builtin_function(elem_bytes == 2 ? "transpose_b16" : "transpose_b32", &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+}
+
 Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, hipStream_t stream) {
   if (n == 0) return {};
   if (from == to) return "convert kernel: identical dtypes";

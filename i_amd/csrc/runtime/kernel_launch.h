@@ -36,6 +36,10 @@ bool gemm_nt_f32_supported(size_t k);
 // y[rows,cols] = row softmax of x, f32
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream);
 
+// dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  The NN product runs as transpose + NT kernel.
+Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,
+                     hipStream_t stream);
+
 Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, hipStream_t stream);
 
 }  // namespace ihip

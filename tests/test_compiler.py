@@ -418,8 +418,14 @@ def test_plan_recognises_hot_path_kernels():
     sm = (((I & i(">ij~i|i:16|ii'j")) >> i("ij-i~ij|i:16|ii'1j")) >> i("^ij~ij|i:16|ii'0j")
           >> ((I & i("+ij~i|i:16|ii'0j")) >> i("ij/i~ij|i:16|ii'01j")))
     assert "hand-written row-softmax kernel [in0 -> out0]" in sm._code()
-    plain = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")
-    assert "f0: generated HIP kernel" in plain._code()  # B is not transposed: no hand-written form
+    plain = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")  # test.py's matmul: B is [K, J]
+    assert "f0: hand-written MFMA GEMM (right operand transposed on the device first)" in plain._code()
+    pv = i("ij*jk~ikj | i:16,j:16 | jii'kj'") >> i("+ikj~ik | i:16,j:16 | jii'kj'0")  # the demo's standalone mm
+    assert "(right operand transposed on the device first); schedule tile 16 x 0 [in0, in1 -> out0]" in pv._code()
+    batched = i("bhik*bhkj~bhijk | i:16,k:16 | bhkii'jk'") >> i("+bhijk~bhij | i:16,k:16 | bhkii'jk'0")
+    assert "right operand transposed" in batched._code()
+    outer = i("ik*jl~ijkl") >> i("+ijkl~ij")  # not a contraction over a shared index
+    assert "hand-written" not in outer._code()
 
 
 def test_plan_does_not_mistake_near_misses():

@@ -207,6 +207,49 @@ def test_config3_mm_t_through_the_host_f32_abi(torch):
     close(c[:, cols], oracle.mm_t(a, b[cols]), RTOL_F32)
 
 
+# ------------------------------------------------------------------ NN products: right operand transposed on the device, then the NT kernel
+MATMUL = "ik*kj~ijk|i:16,k:16|ii'jkk'", "+ijk~ij|i:16,k:16|ii'j!kk'0"  # test.py's matmul with larger splits
+
+
+@pytest.mark.parametrize("m,k,n", [(100, 64, 70), (64, 96, 200), (1, 32, 1), (130, 160, 65)])
+def test_matmul_nn_f32_vs_emitted_c(torch, m, k, n):
+    a, b = rnd((m, k), 1), rnd((k, n), 2)
+    comp = i(MATMUL[0]) >> i(MATMUL[1])
+    assert "right operand transposed" in comp._code()
+    close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
+
+
+@pytest.mark.parametrize("m,k,n", [(300, 256, 200), (128, 64, 128), (77, 1024, 513)])
+def test_matmul_nn_bf16_device_vs_torch(torch, m, k, n):
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(3)
+    a = (torch.rand(m, k, device=dev, generator=gen) * 2 - 1).bfloat16()
+    b = (torch.rand(k, n, device=dev, generator=gen) * 2 - 1).bfloat16()
+    comp = i(MATMUL[0]) >> i(MATMUL[1])
+    got = comp.exec_torch(a, b)
+    ref = a.double() @ b.double()
+    assert float((got.double() - ref).abs().max() / ref.abs().max()) <= RTOL_BF16
+
+
+def test_matmul_nn_batched_and_the_demo_mm(torch):
+    a, b = rnd((2, 3, 40, 64), 1), rnd((2, 3, 64, 50), 2)
+    batched = i("bhik*bhkj~bhijk | i:16,k:16 | bhkii'jk'") >> i("+bhijk~bhij | i:16,k:16 | bhkii'jk'0")
+    assert "right operand transposed" in batched._code()
+    close(batched.exec_numpy(a, b), np.einsum("bhik,bhkj->bhij", a.astype(np.float64), b.astype(np.float64)), RTOL_F32)
+    p_, v_ = rnd((48, 96), 3), rnd((96, 64), 4)
+    mm = i("ij*jk~ikj | i:16,j:16 | jii'kj'") >> i("+ikj~ik | i:16,j:16 | jii'kj'0")
+    close(mm.exec_numpy(p_, v_), oracle.compile_component(mm._ptr).run(p_, v_), RTOL_F32)
+
+
+def test_naive_attention_uses_both_gemm_forms(torch):
+    """The reference's naive attention (flash-attn.py:57-65): mm_t and mm on the MFMA kernels, the rest generated."""
+    q, k, v = rnd((96, 64), 1), rnd((96, 64), 2), rnd((96, 64), 3)
+    comp = naive()
+    code = comp._code()
+    assert "transposed right operand" in code and "right operand transposed on the device first" in code
+    assert np.allclose(comp.exec_numpy(q, k, v), oracle.np_attention64(q, k, v), rtol=3e-4, atol=5e-5)
+
+
 # ------------------------------------------------------------------ BASELINE configs 4 and 5 (bf16 in, f32 accumulate)
 def test_config4_attention_slice_vs_oracle(torch):
     """B8 H32 N4096 d128 recipe; two heads on the GPU, one (b,h) slice of query rows against the oracle."""
