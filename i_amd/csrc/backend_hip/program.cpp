@@ -149,7 +149,9 @@ bool hand_usable(const Run& run, const Recognized& r) {
       if (a.size() < 2) return false;
       return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
     }
-    case Recognized::RowSoftmax: return true;
+    case Recognized::RowSoftmax:
+    case Recognized::RowMaxShift:
+    case Recognized::RowNormalize: return true;
   }
   return false;
 }
@@ -161,7 +163,7 @@ std::set<size_t> hand_intermediates(const Recognized& r) {
   };
   add(r.out);
   add(r.a.buffer);
-  if (r.kind != Recognized::RowSoftmax) add(r.b.buffer);
+  if (r.kind == Recognized::Attention || r.kind == Recognized::GemmNT || r.kind == Recognized::GemmNN) add(r.b.buffer);
   if (r.kind == Recognized::Attention) {
     add(r.c.buffer);
     if (r.has_scale) add(r.scale.buffer);
@@ -242,14 +244,17 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, static_cast<float*>(out), bh, m, n, k, run.stream,
                                        r.tile_i, r.tile_j);
     }
-    case Recognized::RowSoftmax: {
+    case Recognized::RowSoftmax:
+    case Recognized::RowMaxShift:
+    case Recognized::RowNormalize: {
       const auto x = run.shape_of(r.a.buffer);
       size_t rows = 1;
       for (size_t d = 0; d + 1 < x.size(); ++d) rows *= x[d];
       void *in = nullptr, *out = nullptr;
       if (ihip::Err e = run.read_f32(r.a.buffer, &in); !e.empty()) return e;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
-      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream);
+      const int mode = r.kind == Recognized::RowSoftmax ? 0 : r.kind == Recognized::RowMaxShift ? 1 : 2;
+      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode);
     }
     default: return "no hand-written kernel";
   }
@@ -385,7 +390,8 @@ std::string program_code(const Component& component) {
     if (rec[k].kind != Recognized::None) {
       os << " [";
       os << ref_name(rec[k].a.buffer);
-      if (rec[k].kind != Recognized::RowSoftmax) os << ", " << ref_name(rec[k].b.buffer);
+      if (rec[k].kind == Recognized::Attention || rec[k].kind == Recognized::GemmNT || rec[k].kind == Recognized::GemmNN)
+        os << ", " << ref_name(rec[k].b.buffer);
       if (rec[k].kind == Recognized::Attention) os << ", " << ref_name(rec[k].c.buffer);
       if (rec[k].has_scale) os << ", scale " << ref_name(rec[k].scale.buffer);
       os << " -> " << ref_name(rec[k].out) << "]; generated form below runs when operands are outside its limits";

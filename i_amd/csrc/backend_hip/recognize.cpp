@@ -200,6 +200,25 @@ struct Matcher {
     return match_x(x);
   }
 
+  // X - max_J X and X / sum_J X over an operand buffer X[R.., J] (the reduction runs over a private copy of J
+  // and must read the very same X)
+  bool match_row_reduce_then(int t, Op outer, Op inner, Operand& x_out) const {
+    const Term& top = T(t);
+    if (top.op != outer || !top.red.empty() || top.args.size() != 2 || top.out.empty()) return false;
+    const Arg &x = top.args[0], &m = top.args[1];
+    if (!x.external || m.external || x.dims != top.out) return false;
+    const Term& red = T(m.term);
+    if (red.op != inner || red.red.size() != 1 || red.args.size() != 1 || !red.args[0].external) return false;
+    std::vector<int> rows(top.out.begin(), top.out.end() - 1);
+    if (red.out != rows || m.dims != rows) return false;
+    std::map<int, int> ren;
+    for (int r : rows) ren[r] = r;
+    ren[top.out.back()] = red.red[0];
+    if (!tb.unify_arg(x, red.args[0], ren)) return false;
+    x_out = operand(x);
+    return true;
+  }
+
   // P[R.., J] = E / sum_J E, the sum reading the very same E over a private copy of J
   template <class F>
   bool match_softmax(int t, F&& match_x) const {
@@ -236,6 +255,18 @@ struct Matcher {
     }
     r = Recognized{};
     r.out = out;
+
+    // the two halves of the row softmax on their own
+    {
+      Operand x;
+      const bool shift = match_row_reduce_then(root, Op::Sub, Op::Max, x);
+      if (shift || match_row_reduce_then(root, Op::Div, Op::Add, x)) {
+        r.kind = shift ? Recognized::RowMaxShift : Recognized::RowNormalize;
+        r.a = x;
+        r.batch_rank = x.dims.size() - 1;
+        return r;
+      }
+    }
 
     // row softmax over an operand buffer
     {
@@ -297,6 +328,8 @@ std::string Recognized::describe() const {
     case GemmNT: return "hand-written MFMA GEMM (transposed right operand)" + tiles;
     case GemmNN: return "hand-written MFMA GEMM (right operand transposed on the device first)" + tiles;
     case RowSoftmax: return "hand-written row-softmax kernel";
+    case RowMaxShift: return "hand-written row kernel (x - row max)";
+    case RowNormalize: return "hand-written row kernel (x / row sum)";
     default: return "generated HIP kernel";
   }
 }

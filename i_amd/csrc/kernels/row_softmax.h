@@ -5,6 +5,10 @@
 // (three kernels, ilang-python/flash-attn.py:60-62); here the row lives in
 // registers, so HBM sees exactly one read and one write per element.
 // One wavefront owns one row; reductions use cross-lane shuffles only.
+//
+// The same kernels also run the two halves on their own (SoftmaxParams::mode), which is how the reference's
+// naive three-kernel schedule reaches them:  row_max_shift  y = x - max_j x  (flash-attn.py:60) and
+// row_normalize  y = x / sum_j x  (flash-attn.py:62).
 #pragma once
 #include "common.h"
 #include "params.h"
@@ -20,19 +24,53 @@ __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
 
   f32x4 r[NV];
   float mx = -INFINITY;
+  const float pad = p.mode == 2 ? 0.0f : -INFINITY;  // neutral for the reduction of the mode
 #pragma unroll
   for (int t = 0; t < NV; ++t) {
     const uint32_t col = 4u * (lane + 64 * t);
     if (VEC) {
       if (col < p.cols) r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
-      else r[t] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      else r[t] = f32x4{pad, pad, pad, pad};
     } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : -INFINITY;
+      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : pad;
     }
     mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
   }
+  if (p.mode == 2) {  // row_normalize: x / sum(x)
+    float total = 0.0f;
+#pragma unroll
+    for (int t = 0; t < NV; ++t) total += (r[t][0] + r[t][1]) + (r[t][2] + r[t][3]);
+    total = wave_sum(total);
+    const float inv_total = 1.0f / total;
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      const uint32_t col = 4u * (lane + 64 * t);
+      if (VEC) {
+        if (col < p.cols) __builtin_nontemporal_store(r[t] * inv_total, reinterpret_cast<f32x4*>(y + col));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < p.cols) y[col + e] = r[t][e] * inv_total;
+      }
+    }
+    return;
+  }
   mx = wave_max(mx);
+  if (p.mode == 1) {  // row_max_shift: x - max(x)
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      const uint32_t col = 4u * (lane + 64 * t);
+      if (VEC) {
+        if (col < p.cols) __builtin_nontemporal_store(r[t] - mx, reinterpret_cast<f32x4*>(y + col));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < p.cols) y[col + e] = r[t][e] - mx;
+      }
+    }
+    return;
+  }
   const float mb = mx * I_LOG2_E32;
   float sum = 0.0f;
 #pragma unroll
@@ -65,6 +103,18 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
   const float* __restrict__ x = p.x + (size_t)row * p.cols;
   float* __restrict__ y = p.y + (size_t)row * p.cols;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if (p.mode == 2) {  // row_normalize
+    float total = 0.0f;
+    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) total += x[j];
+    total = wave_sum(total);
+    if (lane == 0) red[wave] = total;
+    __syncthreads();
+    total = 0.0f;
+    for (int w = 0; w < nw; ++w) total += red[w];
+    const float inv_total = 1.0f / total;
+    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] * inv_total;
+    return;
+  }
   float mx = -INFINITY;
   for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) mx = fmaxf(mx, x[j]);
   mx = wave_max(mx);
@@ -73,6 +123,10 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
   mx = red[0];
   for (int w = 1; w < nw; ++w) mx = fmaxf(mx, red[w]);
   __syncthreads();
+  if (p.mode == 1) {  // row_max_shift
+    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] - mx;
+    return;
+  }
   const float mb = mx * I_LOG2_E32;
   float sum = 0.0f;
   for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) sum += fast_exp2(__builtin_fmaf(x[j], I_LOG2_E32, -mb));

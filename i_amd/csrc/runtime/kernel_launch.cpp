@@ -155,11 +155,12 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 
-Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream) {
+Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode) {
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
-  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols};
+  if (mode < 0 || mode > 2) return "row_softmax kernel: unknown mode";
+  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, (uint32_t)mode};
   hipFunction_t fn;
   if (cols <= 8192) {
     int nv = 1;

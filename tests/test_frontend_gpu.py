@@ -241,6 +241,21 @@ def test_matmul_nn_batched_and_the_demo_mm(torch):
     close(mm.exec_numpy(p_, v_), oracle.compile_component(mm._ptr).run(p_, v_), RTOL_F32)
 
 
+@pytest.mark.parametrize("rows,cols", [(37, 100), (64, 4096), (5, 9000), (300, 33)])
+def test_row_max_shift_and_row_normalize_kernels(torch, rows, cols):
+    x = rnd((rows, cols), 1)
+    shift = (I & i(">ij~i|i:16,j:16|jii'j'")) >> i("ij-i~ij|i:16,j:16|1jii'j'")
+    assert "x - row max" in shift._code()
+    got = shift.exec_numpy(x)
+    assert np.array_equal(got, x - x.max(axis=1, keepdims=True))  # one exact subtraction per element
+    pos = np.abs(x) + 0.1
+    norm = (I & i("+ij~i|i:16,j:16|jii'j'")) >> i("ij/i~ij|i:16,j:16|1jii'j'")
+    assert "x / row sum" in norm._code()
+    close(norm.exec_numpy(pos), pos.astype(np.float64) / pos.astype(np.float64).sum(axis=1, keepdims=True), RTOL_F32)
+    # the three-kernel naive softmax of the reference's demo runs on them
+    close(softmax_naive().exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
+
+
 def test_naive_attention_uses_both_gemm_forms(torch):
     """The reference's naive attention (flash-attn.py:57-65): mm_t and mm on the MFMA kernels, the rest generated."""
     q, k, v = rnd((96, 64), 1), rnd((96, 64), 2), rnd((96, 64), 3)
