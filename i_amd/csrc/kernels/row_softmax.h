@@ -42,16 +42,16 @@ __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
 #pragma unroll
     for (int t = 0; t < NV; ++t) total += (r[t][0] + r[t][1]) + (r[t][2] + r[t][3]);
     total = wave_sum(total);
-    const float inv_total = 1.0f / total;
+    // a true division per element, as the reference's `a / b`: the kernel is HBM-bound either way
 #pragma unroll
     for (int t = 0; t < NV; ++t) {
       const uint32_t col = 4u * (lane + 64 * t);
       if (VEC) {
-        if (col < p.cols) __builtin_nontemporal_store(r[t] * inv_total, reinterpret_cast<f32x4*>(y + col));
+        if (col < p.cols) __builtin_nontemporal_store(r[t] / total, reinterpret_cast<f32x4*>(y + col));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (col + e < p.cols) y[col + e] = r[t][e] * inv_total;
+          if (col + e < p.cols) y[col + e] = r[t][e] / total;
       }
     }
     return;
@@ -111,8 +111,7 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
     __syncthreads();
     total = 0.0f;
     for (int w = 0; w < nw; ++w) total += red[w];
-    const float inv_total = 1.0f / total;
-    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] * inv_total;
+    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] / total;
     return;
   }
   float mx = -INFINITY;
