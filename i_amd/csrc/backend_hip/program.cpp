@@ -151,7 +151,8 @@ bool hand_usable(const Run& run, const Recognized& r) {
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
-    case Recognized::RowNormalize: return true;
+    case Recognized::RowNormalize:
+    case Recognized::RowExp: return true;
   }
   return false;
 }
@@ -246,14 +247,15 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
-    case Recognized::RowNormalize: {
+    case Recognized::RowNormalize:
+    case Recognized::RowExp: {
       const auto x = run.shape_of(r.a.buffer);
       size_t rows = 1;
       for (size_t d = 0; d + 1 < x.size(); ++d) rows *= x[d];
       void *in = nullptr, *out = nullptr;
       if (ihip::Err e = run.read_f32(r.a.buffer, &in); !e.empty()) return e;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
-      const int mode = r.kind == Recognized::RowSoftmax ? 0 : r.kind == Recognized::RowMaxShift ? 1 : 2;
+      const int mode = r.kind == Recognized::RowSoftmax ? 0 : r.kind == Recognized::RowMaxShift ? 1 : r.kind == Recognized::RowNormalize ? 2 : 3;
       return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode);
     }
     default: return "no hand-written kernel";

@@ -256,6 +256,15 @@ struct Matcher {
     r = Recognized{};
     r.out = out;
 
+    // exp of an operand buffer, elementwise
+    if (top.op == Op::Pow && top.red.empty() && top.args.size() == 1 && top.args[0].external && !top.out.empty() &&
+        top.args[0].dims == top.out) {
+      r.kind = Recognized::RowExp;
+      r.a = operand(top.args[0]);
+      r.batch_rank = r.a.dims.size() - 1;
+      return r;
+    }
+
     // the two halves of the row softmax on their own
     {
       Operand x;
@@ -330,6 +339,7 @@ std::string Recognized::describe() const {
     case RowSoftmax: return "hand-written row-softmax kernel";
     case RowMaxShift: return "hand-written row kernel (x - row max)";
     case RowNormalize: return "hand-written row kernel (x / row sum)";
+    case RowExp: return "hand-written row kernel (exp x)";
     default: return "generated HIP kernel";
   }
 }

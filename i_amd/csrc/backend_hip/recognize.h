@@ -21,11 +21,12 @@ struct Operand {
 };
 
 struct Recognized {
-  enum Kind { None, Attention, GemmNT, GemmNN, RowSoftmax, RowMaxShift, RowNormalize } kind = None;
+  enum Kind { None, Attention, GemmNT, GemmNN, RowSoftmax, RowMaxShift, RowNormalize, RowExp } kind = None;
   // Attention: q [B.., I, D], k [B.., J, D], v [B.., J, E] -> out [B.., I, E]; optional scalar scale
   // GemmNT:    a [B.., I, K], b [B.., J, K] -> out [B.., I, J]
   // GemmNN:    a [B.., I, K], b [B.., K, J] -> out [B.., I, J]
-  // RowSoftmax, RowMaxShift (x - max_J x), RowNormalize (x / sum_J x): x [R.., J] -> out [R.., J]
+  // RowSoftmax, RowMaxShift (x - max_J x), RowNormalize (x / sum_J x), RowExp (exp x, elementwise):
+  //            x [R.., J] -> out [R.., J]
   Operand a, b, c;             // q,k,v | a,b,- | x,-,-
   bool has_scale = false;
   Operand scale;               // rank-0 operand

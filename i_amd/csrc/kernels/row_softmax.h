@@ -8,7 +8,8 @@
 //
 // The same kernels also run the two halves on their own (SoftmaxParams::mode), which is how the reference's
 // naive three-kernel schedule reaches them:  row_max_shift  y = x - max_j x  (flash-attn.py:60) and
-// row_normalize  y = x / sum_j x  (flash-attn.py:62).
+// row_normalize  y = x / sum_j x  (flash-attn.py:62); and the elementwise exp between them (flash-attn.py:61, mode 3)
+// with the exponential the fused form uses.
 #pragma once
 #include "common.h"
 #include "params.h"
@@ -36,6 +37,23 @@ __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
       for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : pad;
     }
     mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
+  }
+  if (p.mode == 3) {  // exp(x), elementwise
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      const uint32_t col = 4u * (lane + 64 * t);
+      f32x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = fast_exp2(r[t][e] * I_LOG2_E32);
+      if (VEC) {
+        if (col < p.cols) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(y + col));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < p.cols) y[col + e] = v[e];
+      }
+    }
+    return;
   }
   if (p.mode == 2) {  // row_normalize: x / sum(x)
     float total = 0.0f;
@@ -103,6 +121,10 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
   const float* __restrict__ x = p.x + (size_t)row * p.cols;
   float* __restrict__ y = p.y + (size_t)row * p.cols;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if (p.mode == 3) {  // exp(x), elementwise
+    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = fast_exp2(x[j] * I_LOG2_E32);
+    return;
+  }
   if (p.mode == 2) {  // row_normalize
     float total = 0.0f;
     for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) total += x[j];

@@ -159,7 +159,7 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
-  if (mode < 0 || mode > 2) return "row_softmax kernel: unknown mode";
+  if (mode < 0 || mode > 3) return "row_softmax kernel: unknown mode";
   SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, (uint32_t)mode};
   hipFunction_t fn;
   if (cols <= 8192) {

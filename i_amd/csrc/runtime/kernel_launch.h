@@ -34,7 +34,7 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
 bool gemm_nt_f32_supported(size_t k);
 
 // y[rows,cols] = row softmax of x, f32
-// mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize)
+// mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize); 3: y = exp(x)
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0);
 
 // dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  The NN product runs as transpose + NT kernel.

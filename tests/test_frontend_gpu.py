@@ -252,6 +252,10 @@ def test_row_max_shift_and_row_normalize_kernels(torch, rows, cols):
     norm = (I & i("+ij~i|i:16,j:16|jii'j'")) >> i("ij/i~ij|i:16,j:16|1jii'j'")
     assert "x / row sum" in norm._code()
     close(norm.exec_numpy(pos), pos.astype(np.float64) / pos.astype(np.float64).sum(axis=1, keepdims=True), RTOL_F32)
+    ex = i("^ij~ij|i:16,j:16|jii'j'")
+    assert "exp x" in ex._code()
+    small = np.clip(x, -20.0, 5.0)
+    close(ex.exec_numpy(small), oracle.compile_component(ex._ptr).run(small), RTOL_F32)
     # the three-kernel naive softmax of the reference's demo runs on them
     close(softmax_naive().exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
 
