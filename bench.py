@@ -137,7 +137,20 @@ def main():
     y = torch.empty_like(x)
     sm = softmax_component(i, I)
     sm.into(y, x)
-    _, sm_ms = time_steps(torch, lambda: sm.into(y, x), max(args.steps, 20), args.warmup)
+    # The timed calls walk four input/output pairs (2 GiB): one pair alone (512 MiB) would be re-read partly out of
+    # the 256 MiB Infinity Cache from one step to the next, and that is not HBM bandwidth.
+    xs = [x] + [torch.randn(rows, cols, device=dev, generator=gen) for _ in range(3)]
+    ys = [y] + [torch.empty_like(x) for _ in range(3)]
+    turn = [0]
+
+    def softmax_step():
+        k_ = turn[0] % 4
+        turn[0] += 1
+        sm.into(ys[k_], xs[k_])
+
+    _, sm_ms = time_steps(torch, softmax_step, max(args.steps, 20), max(args.warmup, 4))
+    sm.into(y, x)  # the parity check below reads y
+    del xs, ys
     sm_bytes = 2.0 * rows * cols * 4
     sm_gbs = sm_bytes / (sm_ms * 1e-3) / 1e9
 
@@ -227,7 +240,7 @@ def main():
             "value": flop / (const_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": const_ms,
             "frac_of_peak": flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
         "secondary": [
-            {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1])", "value": sm_gbs, "unit": "GB/s",
+            {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
              "roofline": {"bound": "hbm", "achieved": sm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                           "frac": sm_gbs / PEAK_HBM_GBS, "traffic": measured_traffic("row_softmax_16384x4096_f32.md"),
                           "kernel": "row_softmax_wave_v16",

@@ -61,21 +61,24 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
   gemm_nt_direct_body<true, 256, 2, 4>(p);
 }
 
-#define SOFTMAX_WAVE(NV)                                                                          \
-  extern "C" __global__ void __launch_bounds__(256) row_softmax_wave_v##NV(SoftmaxParams p) {     \
-    row_softmax_wave_body<NV, true>(p);                                                           \
-  }                                                                                               \
-  extern "C" __global__ void __launch_bounds__(256) row_softmax_wave_s##NV(SoftmaxParams p) {     \
-    row_softmax_wave_body<NV, false>(p);                                                          \
+// row_<op>_wave_{v,s}<NV> and row_<op>_block for op = softmax, shift (x - row max), norm (x / row sum), exp
+#define ROW_WAVE(OP, MODE, NV)                                                                     \
+  extern "C" __global__ void __launch_bounds__(256) row_##OP##_wave_v##NV(SoftmaxParams p) {       \
+    row_softmax_wave_body<NV, true, MODE>(p);                                                      \
+  }                                                                                                \
+  extern "C" __global__ void __launch_bounds__(256) row_##OP##_wave_s##NV(SoftmaxParams p) {       \
+    row_softmax_wave_body<NV, false, MODE>(p);                                                     \
   }
-SOFTMAX_WAVE(1)
-SOFTMAX_WAVE(2)
-SOFTMAX_WAVE(4)
-SOFTMAX_WAVE(8)
-SOFTMAX_WAVE(16)
-SOFTMAX_WAVE(32)
-
-extern "C" __global__ void __launch_bounds__(1024) row_softmax_block(SoftmaxParams p) { row_softmax_block_body(p); }
+#define ROW_OP(OP, MODE)                                                                           \
+  ROW_WAVE(OP, MODE, 1) ROW_WAVE(OP, MODE, 2) ROW_WAVE(OP, MODE, 4) ROW_WAVE(OP, MODE, 8)          \
+  ROW_WAVE(OP, MODE, 16) ROW_WAVE(OP, MODE, 32)                                                    \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_block(SoftmaxParams p) {           \
+    row_softmax_block_body<MODE>(p);                                                               \
+  }
+ROW_OP(softmax, 0)
+ROW_OP(shift, 1)
+ROW_OP(norm, 2)
+ROW_OP(exp, 3)
 
 extern "C" __global__ void __launch_bounds__(256) convert_f32_to_bf16(ConvertParams p) {
   const float* s = reinterpret_cast<const float*>(p.src);

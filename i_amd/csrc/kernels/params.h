@@ -30,7 +30,6 @@ struct SoftmaxParams {
   const float* x;
   float* y;
   uint32_t rows, cols;
-  uint32_t mode;  // 0: softmax, 1: y = x - rowmax(x), 2: y = x / rowsum(x), 3: y = exp(x)
 };
 
 struct ConvertParams {

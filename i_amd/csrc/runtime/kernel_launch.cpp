@@ -160,20 +160,21 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
   if (mode < 0 || mode > 3) return "row_softmax kernel: unknown mode";
-  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, (uint32_t)mode};
+  static const char* const kOps[4] = {"softmax", "shift", "norm", "exp"};
+  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols};
   hipFunction_t fn;
   if (cols <= 8192) {
     int nv = 1;
     while ((size_t)256 * nv < cols) nv *= 2;
     const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
-    const std::string name = std::string("row_softmax_wave_") + (vec ? "v" : "s") + std::to_string(nv);
+    const std::string name = std::string("row_") + kOps[mode] + "_wave_" + (vec ? "v" : "s") + std::to_string(nv);
     if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
     const size_t grid = (rows + 3) / 4;  // four wavefronts (rows) per workgroup
     if (grid > kMaxGrid) return "row_softmax kernel: grid too large";
     return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
   }
   if (rows > kMaxGrid) return "row_softmax kernel: grid too large";
-  if (Err e = builtin_function("row_softmax_block", &fn); !e.empty()) return e;
+  if (Err e = builtin_function((std::string("row_") + kOps[mode] + "_block").c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
 }
 
