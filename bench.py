@@ -254,7 +254,7 @@ def main():
              "roofline": {"bound": "mfma", "achieved": c5_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                           "frac": c5_tflops / PEAK_BF16_TFLOPS,
                           "traffic": measured_traffic("flash_attention_B1_H16_N32768_d64_bf16.md"),
-                          "kernel": "attn_fwd_bf16_d64_bn64_direct_w8", "kernel_ms": c5_ms}},
+                          "kernel": "attn_fwd_bf16_d64_bn32_q64", "kernel_ms": c5_ms}},
         ] + ([c1] if c1 else []),
     }
     print(json.dumps(line))

@@ -3,6 +3,7 @@
 // hipModuleGetFunction; each takes one parameter block by value (params.h).
 #include "attention_bf16.h"
 #include "attention_bf16_direct.h"
+#include "attention_bf16_q64.h"
 #include "attention_f32.h"
 #include "gemm_nt_bf16.h"
 #include "gemm_nt_bf16_direct.h"
@@ -32,6 +33,10 @@ extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d128_bn64_dir
 }
 extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn64_direct_w8(AttnParams p) {
   attn_fwd_bf16_direct_body<64, 64, 8>(p);
+}
+// d = 64 with 64 queries per wave (attention_bf16_q64.h): 8 waves, 512 query rows per workgroup, 32-key tiles
+extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(AttnParams p) {
+  attn_fwd_bf16_q64_body<64, 32, 8>(p);
 }
 
 #define ATTN_F32(DPAD, BN, NW)                                                             \

@@ -38,20 +38,29 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
   //     larger workgroup is used when it still leaves at least two workgroups per CU
   //   otherwise: register-staged kernel with guarded columns
-  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the direct kernel and ILANG_ATTN_NO_DIRECT=1
-  // forces the register-staged kernel; both exist so that tests can reach every kernel with small inputs.
+  //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512): the
+  //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs
+  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
+  // d == 64 only) and ILANG_ATTN_NO_DIRECT=1 forces the register-staged kernel; both exist so that tests can
+  // reach every kernel with small inputs.
   unsigned bm = 128;
+  bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
   const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct) {
     if (query_tile == 128 || query_tile == 256) bm = (unsigned)query_tile;  // the schedule's i split
+    else if (d == 64 && (query_tile == 512 || (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256))) q64 = true;
     else if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
       const int waves = std::atoi(w);
-      if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8";
-      bm = 32u * (unsigned)waves;
+      q64 = waves == 64 && d == 64;
+      if (!q64) {
+        if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8 (or 64 for d = 64)";
+        bm = 32u * (unsigned)waves;
+      }
     }
+    if (q64) bm = 512;
   }
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o;
@@ -63,7 +72,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 
   const char* name;
   if (in_dtype == BF16) {
-    if (direct)
+    if (direct && q64) name = "attn_fwd_bf16_d64_bn32_q64";
+    else if (direct)
       name = d == 64 ? (bm == 256 ? "attn_fwd_bf16_d64_bn64_direct_w8" : "attn_fwd_bf16_d64_bn64_direct")
                      : (bm == 256 ? "attn_fwd_bf16_d128_bn64_direct_w8" : "attn_fwd_bf16_d128_bn64_direct");
     else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
@@ -76,7 +86,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   if (grid > kMaxGrid) return "attention kernel: grid too large";
   hipFunction_t fn;
   if (Err e = builtin_function(name, &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, 1, 1, 2 * bm, &p, sizeof(p), stream);
+  return launch(fn, (unsigned)grid, 1, 1, q64 ? bm : 2 * bm, &p, sizeof(p), stream);
 }
 
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }

@@ -106,13 +106,17 @@ def test_attention_bf16_vs_oracle(env, bh, nq, nk, d):
 
 
 @pytest.mark.parametrize("d", [64, 128])
-@pytest.mark.parametrize("force", [None, "waves8", "staged"])
+@pytest.mark.parametrize("force", [None, "waves8", "q64", "staged"])
 def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
-    """The launcher picks between the direct-to-LDS kernel (4 or 8 waves per workgroup) and the
-    register-staged kernel; force each of them on one ragged problem (7 full key tiles + a partial
-    one, so the steady-state loop, its drain and the masked tail all run)."""
+    """The launcher picks between the direct-to-LDS kernel (4 or 8 waves per workgroup), the 64-queries-per-wave
+    kernel (d = 64) and the register-staged kernel; force each of them on one ragged problem (7 full 64-key
+    tiles + a partial one, so the steady-state loop, its drain and the masked tail all run)."""
+    if force == "q64" and d != 64:
+        pytest.skip("the 64-queries-per-wave kernel exists for d = 64 only")
     if force == "waves8":
         monkeypatch.setenv("ILANG_ATTN_WAVES", "8")
+    elif force == "q64":
+        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
     elif force == "staged":
         monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
     bh, nq, nk = 2, 300, 450
@@ -140,11 +144,14 @@ def test_attention_bf16_workgroup_sizes_agree_bitwise(env, monkeypatch):
     assert rc == -1 and "ILANG_ATTN_WAVES" in env.nat.last_error()
 
 
+@pytest.mark.parametrize("q64", [False, True])
 @pytest.mark.parametrize("span", [20.0, 45.0, 90.0])
-def test_attention_bf16_reference_max_moves_slowly_and_fast(env, span):
+def test_attention_bf16_reference_max_moves_slowly_and_fast(env, monkeypatch, span, q64):
     """Scores rise steadily along the keys by `span` nats in total over 10 tiles.  The direct kernel
     moves a row's reference max only when a tile exceeds it by 2^8: span 20 never reaches that after
     the first tile, 45 reaches it every other tile, 90 at every tile."""
+    if q64:
+        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
     nq, nk, d = 64, 640, 64
     q = np.ones((1, nq, d), np.float32)
     k = oracle.to_bf16_f32((np.arange(nk, dtype=np.float32)[None, :, None] * np.ones((1, 1, d), np.float32))
@@ -154,12 +161,15 @@ def test_attention_bf16_reference_max_moves_slowly_and_fast(env, span):
     assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, "64 (64 queries per wave)"])
 @pytest.mark.parametrize("jump_tile", [1, 6, 11])
-def test_attention_bf16_score_jump_overflows_the_stale_reference(env, d, jump_tile):
+def test_attention_bf16_score_jump_overflows_the_stale_reference(env, monkeypatch, d, jump_tile):
     """All scores are ~0 except in one key tile, where they are ~+300 nats: exp against the reference of the
     earlier tiles overflows to inf there.  The steady-state loop takes no row max; its row-sum guard has to
     catch this before the tile's PV product and move the reference.  Rows 32.. keep small scores throughout."""
+    if d == "64 (64 queries per wave)":
+        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
+        d = 64
     nq, nk = 64, 12 * 64 + 40
     q = np.zeros((1, nq, d), np.float32)
     q[:, :32, 0] = 1.0
@@ -173,7 +183,10 @@ def test_attention_bf16_score_jump_overflows_the_stale_reference(env, d, jump_ti
     assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
 
 
-def test_attention_bf16_direct_negative_and_zero_scale(env):
+@pytest.mark.parametrize("q64", [False, True])
+def test_attention_bf16_direct_negative_and_zero_scale(env, monkeypatch, q64):
+    if q64:
+        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
     q, k, v = (oracle.to_bf16_f32(rnd((2, n, 64), s)) for s, n in ((1, 70), (2, 400), (3, 400)))
     for scale in (-0.3, 0.0):
         ref = oracle.np_attention64(q, k, v, scale).astype(np.float32)
@@ -191,8 +204,11 @@ def test_attention_bf16_config4_slice_vs_oracle(env):
     assert_close(got[:, rows], ref, RTOL_BF16)
 
 
-def test_attention_bf16_long_sequence_rescale_stress(env):
-    """Config 5 recipe (inputs x2.0, d=64) at N=8192: heavy running-max movement."""
+@pytest.mark.parametrize("waves", ["8", "64"])
+def test_attention_bf16_long_sequence_rescale_stress(env, monkeypatch, waves):
+    """Config 5 recipe (inputs x2.0, d=64) at N=8192: heavy running-max movement; the 8-wave kernel and the
+    64-queries-per-wave kernel that the launcher picks at the full size."""
+    monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
     n, d = 8192, 64
     q, k, v = (oracle.to_bf16_f32(rnd((1, n, d), s) * 2.0) for s in (1, 2, 3))
     scale = float(np.float32(1.0 / np.sqrt(d)))
