@@ -85,9 +85,18 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
+  //
+  // PRESCALE (d = 64, where the softmax and not the MFMAs sets the pace: half the MFMA work per exponential): the
+  // whole factor scale * log2(e) is folded into Q, rounded to bf16 once more, and in the steady state the score
+  // accumulators start at -reference instead of 0 (a 16-register tuple as the MFMA's addend), so that a score
+  // comes out of the matrix pipe as the argument of its exp2 and the vector pipe does one instruction less per
+  // score.  The extra rounding of Q perturbs a score by about 0.007 in the exponent (0.5 % of a probability,
+  // independent from key to key), the size of the bf16 rounding of the probability itself.
+  constexpr bool PRESCALE = DPAD == 64;
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
-  const float scale_log2 = fabsf(scale_raw) * I_LOG2_E32;
+  const float scale_log2 = PRESCALE ? 1.0f : fabsf(scale_raw) * I_LOG2_E32;
+  const float q_factor = scale_raw * I_LOG2_E32;
 
   // Q^T fragments (B operand): lane (c, h) holds q[row][16*ks + 8*h .. +8].
   const uint32_t qrow = qt * BM + wave * 32 + c;
@@ -96,8 +105,15 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   for (int ks = 0; ks < KSTEPS; ++ks) {
     u32x4 z = {0, 0, 0, 0};
     if (qrow < p.nq) z = ldg128(Q + (size_t)qrow * d + 16 * ks + 8 * h);
-    z ^= sign_flip;
-    qf[ks] = __builtin_bit_cast(bf16x8, z);
+    if constexpr (PRESCALE) {
+      bf16x8 scaled = __builtin_bit_cast(bf16x8, z);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) scaled[e] = (bf16_t)((float)scaled[e] * q_factor);
+      qf[ks] = scaled;
+    } else {
+      z ^= sign_flip;
+      qf[ks] = __builtin_bit_cast(bf16x8, z);
+    }
   }
 
   f32x16 o[DT];
@@ -340,13 +356,15 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // and 1) are computed one trip early, in the output slots of the previous tile, which otherwise carry no
   // vector work at all, while the score slots are the crowded ones.
   constexpr int NEARLY = 8;
+  f32x16 negmb16 = zero16;  // PRESCALE: -reference in every element, the addend of a score tile's first MFMA
   u32x4 pq[NPAIR / 4];
   float psum[2] = {0.0f, 0.0f};
   const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
   auto exp_pair_from = [&](const f32x16 (&s)[KT], int pr, float mb) {
     const int pkt = pr / 8, i = 2 * (pr % 8);
-    const float e0 = fast_exp2(__builtin_fmaf(s[pkt][i], scale_log2, -mb));
-    const float e1 = fast_exp2(__builtin_fmaf(s[pkt][i + 1], scale_log2, -mb));
+    // PRESCALE: the steady-state scores are already relative to the reference
+    const float e0 = PRESCALE ? fast_exp2(s[pkt][i]) : fast_exp2(__builtin_fmaf(s[pkt][i], scale_log2, -mb));
+    const float e1 = PRESCALE ? fast_exp2(s[pkt][i + 1]) : fast_exp2(__builtin_fmaf(s[pkt][i + 1], scale_log2, -mb));
     const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
     psum[pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[pr & 1], false);
     uint32_t packed = __builtin_bit_cast(uint32_t, pair);
@@ -417,7 +435,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     for (int n = 0; n < NQK; ++n) {
       fetch_for_slot(DT + n);
       const int ks = n / KT, kt = n % KT;
-      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[ks], ks == 0 ? zero16 : s_next[kt], 0, 0, 0);
+      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[ks],
+                                                           ks == 0 ? (PRESCALE ? negmb16 : zero16) : s_next[kt], 0, 0, 0);
       request_for_slot(DT + n);
       pairs_for_slot(DT + n);
       __builtin_amdgcn_sched_barrier(0);
@@ -431,9 +450,23 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_cur[kt][i]);
       mx = half_max(mx);
+      if constexpr (PRESCALE) mx += mb_run;  // the scores are relative to the reference they were computed against
       const bool move = mx * scale_log2 > mb_run;  // the reference only moves up
       const float mb_new = move ? mx * scale_log2 : mb_run;
       const float alpha = fast_exp2(mb_run - mb_new);
+      if constexpr (PRESCALE) {
+        // both score tiles in flight were accumulated against the old reference
+        const float delta = mb_new - mb_run;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            s_cur[kt][i] -= delta;
+            s_next[kt][i] -= delta;
+          }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) negmb16[i] = -mb_new;
+      }
       m_run = move ? mx : m_run;
       mb_run = mb_new;
       l_run *= alpha;
@@ -480,6 +513,15 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
     m_run = half_max(mx_tile);
     mb_run = m_run * scale_log2;
+    if constexpr (PRESCALE) {
+      // from here to the end of the steady state the score tiles are kept relative to the reference
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sa[kt][i] -= mb_run;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) negmb16[i] = -mb_run;
+    }
 #pragma unroll
     for (int pr = 0; pr < NEARLY; ++pr) exp_pair_from(sa, pr, mb_run);
     // the first trip has no predecessor: its carried slots add zero
@@ -503,6 +545,13 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 #pragma unroll
     for (int t = 0; t < DT; ++t)
       o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ca.a[t], __builtin_bit_cast(bf16x8, ca.p), o[t], 0, 0, 0);
+    if constexpr (PRESCALE) {
+      // the general loop below works on scores as they are
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sa[kt][i] += mb_run;
+    }
   }
   // the last tiles (no successor, or a partial one): same steps with run-time conditions; sa holds S(j)
   for (; j < ntiles; ++j) {
