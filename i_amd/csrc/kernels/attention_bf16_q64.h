@@ -60,8 +60,11 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
-  const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
-  const float scale_log2 = fabsf(scale_raw) * I_LOG2_E32;
+  // As in attention_bf16_direct.h for d = 64: the factor scale * log2(e) is folded into Q (one more bf16 rounding),
+  // and in the steady state a score tile's first MFMA adds -reference instead of 0, so that scores leave the
+  // matrix pipe as arguments of exp2.
+  const float scale_log2 = 1.0f;
+  const float q_factor = scale_raw * I_LOG2_E32;
 
   // Q^T fragments (B operand): lane (c, h) holds q[row][16*ks + 8*h .. +8].
   uint32_t qrow[QB];
@@ -73,8 +76,10 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
     for (int ks = 0; ks < KSTEPS; ++ks) {
       u32x4 z = {0, 0, 0, 0};
       if (qrow[b] < p.nq) z = ldg128(Q + (size_t)qrow[b] * d + 16 * ks + 8 * h);
-      z ^= sign_flip;
-      qf[b][ks] = __builtin_bit_cast(bf16x8, z);
+      bf16x8 scaled = __builtin_bit_cast(bf16x8, z);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) scaled[e] = (bf16_t)((float)scaled[e] * q_factor);
+      qf[b][ks] = scaled;
     }
   }
 
@@ -322,6 +327,10 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   constexpr int XLEAD = ATTN_Q64_XLEAD;
   static_assert(NPAIR % 4 == 0 && 2 * WLW <= NPRE && XLEAD >= 0 && XLEAD < NQK, "slot shape");
 
+  f32x16 negmb16[QB];  // -reference in every element: the addend of a score tile's first MFMA
+#pragma unroll
+  for (int b = 0; b < QB; ++b) negmb16[b] = zero16;
+
   struct Carry {
     bf16x8 a[DT];  // V^T operands of the last 16-key group
     u32x4 p[QB];   // its probabilities, per query block
@@ -391,8 +400,8 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
     auto exp_pair = [&](int n) {
       const int b = n / NPAIR, pr = n % NPAIR;
       const int pkt = pr / 8, i = 2 * (pr % 8);
-      const float e0 = fast_exp2(__builtin_fmaf(s_cur[b][pkt][i], scale_log2, -mb[b]));
-      const float e1 = fast_exp2(__builtin_fmaf(s_cur[b][pkt][i + 1], scale_log2, -mb[b]));
+      const float e0 = fast_exp2(s_cur[b][pkt][i]);  // relative to the reference already
+      const float e1 = fast_exp2(s_cur[b][pkt][i + 1]);
       const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
       psum[b][pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[b][pr & 1], false);
       uint32_t packed = __builtin_bit_cast(uint32_t, pair);
@@ -425,7 +434,7 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
 #pragma unroll
       for (int b = 0; b < QB; ++b) {
         s_next[b][kt] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[b][ks], ks == 0 ? zero16 : s_next[b][kt], 0, 0, 0);
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[b][ks], ks == 0 ? negmb16[b] : s_next[b][kt], 0, 0, 0);
         request_for_slot(QB * (DT + n) + b);
         pairs_for_slot(QB * (DT + n) + b);
         __builtin_amdgcn_sched_barrier(0);
@@ -444,10 +453,23 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_cur[b][kt][i]);
-        mx = half_max(mx);
+        mx = half_max(mx) + mb_run[b];  // the scores are relative to the reference they were computed against
         const bool move = mx * scale_log2 > mb_run[b];  // the reference only moves up
         const float mb_new = move ? mx * scale_log2 : mb_run[b];
         const float alpha = fast_exp2(mb_run[b] - mb_new);
+        {
+          // both score tiles in flight were accumulated against the old reference
+          const float delta = mb_new - mb_run[b];
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              s_cur[b][kt][i] -= delta;
+              s_next[b][kt][i] -= delta;
+            }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) negmb16[b][i] = -mb_new;
+        }
         m_run[b] = move ? mx : m_run[b];
         mb_run[b] = mb_new;
         l_run[b] *= alpha;
@@ -496,6 +518,13 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
         for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[b][kt][i]);
       m_run[b] = half_max(mx_tile);
       mb_run[b] = m_run[b] * scale_log2;
+      // from here to the end of the steady state the score tiles are kept relative to the reference
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sa[b][kt][i] -= mb_run[b];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) negmb16[b][i] = -mb_run[b];
     }
     // the first trip has no predecessor: its carried slots add zero
     Carry ca, cb;
@@ -513,6 +542,13 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
 #pragma unroll
       for (int b = 0; b < QB; ++b)
         o[b][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ca.a[t], __builtin_bit_cast(bf16x8, ca.p[b]), o[b][t], 0, 0, 0);
+    // the general loop below works on scores as they are
+#pragma unroll
+    for (int b = 0; b < QB; ++b)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sa[b][kt][i] += mb_run[b];
   }
   // the last tiles (no successor, or a partial one): same steps with run-time conditions; sa holds S(j)
   for (; j < ntiles; ++j) {
