@@ -50,6 +50,10 @@
 #ifndef ATTN_XLEAD
 #define ATTN_XLEAD 1
 #endif
+// d = 128: steady state without any reference for the exponentials (see NOREF below)
+#ifndef ATTN_NOREF
+#define ATTN_NOREF 1
+#endif
 
 template <int DPAD, int BN, int NWAVES>
 __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
@@ -92,10 +96,20 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // comes out of the matrix pipe as the argument of its exp2 and the vector pipe does one instruction less per
   // score.  The extra rounding of Q perturbs a score by about 0.007 in the exponent (0.5 % of a probability,
   // independent from key to key), the size of the bf16 rounding of the probability itself.
+  //
+  // NOREF (d = 128, where the 16 registers of that tuple do not exist): Q is scaled in the same way and the steady
+  // state takes P = exp2(score) as it is, without a reference at all.  The normalised result does not depend on
+  // the reference, and with probabilities rounded to bf16 (same exponent range as f32) neither does its precision,
+  // as long as nothing overflows or the whole row underflows; scores of attention stay within a few tens.  A
+  // wave notes (without branching) whether any tile's row sum reached 2^80 and, at the end, whether a row sum
+  // fell below 2^-100; if any wave of the workgroup did, the workgroup throws the pass away and computes the item
+  // again with the general loop, which takes the running max tile by tile.
   constexpr bool PRESCALE = DPAD == 64;
+  constexpr bool NOREF = DPAD == 128 && ATTN_NOREF;
+  constexpr bool QSCALE = PRESCALE || NOREF;
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
-  const float scale_log2 = PRESCALE ? 1.0f : fabsf(scale_raw) * I_LOG2_E32;
+  const float scale_log2 = QSCALE ? 1.0f : fabsf(scale_raw) * I_LOG2_E32;
   const float q_factor = scale_raw * I_LOG2_E32;
 
   // Q^T fragments (B operand): lane (c, h) holds q[row][16*ks + 8*h .. +8].
@@ -105,7 +119,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   for (int ks = 0; ks < KSTEPS; ++ks) {
     u32x4 z = {0, 0, 0, 0};
     if (qrow < p.nq) z = ldg128(Q + (size_t)qrow * d + 16 * ks + 8 * h);
-    if constexpr (PRESCALE) {
+    if constexpr (QSCALE) {
       bf16x8 scaled = __builtin_bit_cast(bf16x8, z);
 #pragma unroll
       for (int e = 0; e < 8; ++e) scaled[e] = (bf16_t)((float)scaled[e] * q_factor);
@@ -306,13 +320,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     else request_tile(t * BN, buf, Yes{}, No{}, Yes{});
   };
 
-  request_k(0, 0);
-  request_v(0, 0);
-  if (ntiles > 1) request_k(1, 1);
-  dma_wait_all();
-  __syncthreads();
   f32x16 sa[KT], sb[KT];
-  qk(sa, 0);
 
   // Steady state (tiles j, j+1, j+2 are all full tiles).  One trip runs from barrier to barrier and is
   // written as NQK + NPV MFMA slots, everything else dealt out between the MFMAs a few vector
@@ -359,12 +367,13 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   f32x16 negmb16 = zero16;  // PRESCALE: -reference in every element, the addend of a score tile's first MFMA
   u32x4 pq[NPAIR / 4];
   float psum[2] = {0.0f, 0.0f};
+  bool bad = false;  // NOREF: some tile's row sum left the safe range
   const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
   auto exp_pair_from = [&](const f32x16 (&s)[KT], int pr, float mb) {
     const int pkt = pr / 8, i = 2 * (pr % 8);
     // PRESCALE: the steady-state scores are already relative to the reference
-    const float e0 = PRESCALE ? fast_exp2(s[pkt][i]) : fast_exp2(__builtin_fmaf(s[pkt][i], scale_log2, -mb));
-    const float e1 = PRESCALE ? fast_exp2(s[pkt][i + 1]) : fast_exp2(__builtin_fmaf(s[pkt][i + 1], scale_log2, -mb));
+    const float e0 = QSCALE ? fast_exp2(s[pkt][i]) : fast_exp2(__builtin_fmaf(s[pkt][i], scale_log2, -mb));
+    const float e1 = QSCALE ? fast_exp2(s[pkt][i + 1]) : fast_exp2(__builtin_fmaf(s[pkt][i + 1], scale_log2, -mb));
     const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
     psum[pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[pr & 1], false);
     uint32_t packed = __builtin_bit_cast(uint32_t, pair);
@@ -443,7 +452,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     }
 
     // ---- guard (see above); O at this point holds everything up to and including tile j-1
-    if (__builtin_amdgcn_ballot_w64(!(psum[0] + psum[1] < SUM_GUARD))) {
+    if constexpr (NOREF) {
+      // noted, acted upon after the pass.  With reference 0 a score may reach 2^80 / 64 as a probability
+      // (about 51 nats) before its tile counts as out of range: O then stays below 2^80 nk max|v|.
+      bad = bad || !(psum[0] + psum[1] < 0x1p80f);
+    } else if (__builtin_amdgcn_ballot_w64(!(psum[0] + psum[1] < SUM_GUARD))) {
       float mx = s_cur[0][0];
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
@@ -503,8 +516,46 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     __syncthreads();
   };
 
+  // tiles 0 and 1 of K and tile 0 of V into LDS, then S(0)
+  auto first_tiles = [&]() {
+    request_k(0, 0);
+    request_v(0, 0);
+    if (ntiles > 1) request_k(1, 1);
+    dma_wait_all();
+    __syncthreads();
+    qk(sa, 0);
+    // the first trip of either loop requests K(2) into the buffer of K(0): not before every wave has read K(0).
+    // (Without this barrier a wave that leaves qk early can overwrite rows that a late wave has yet to read,
+    // once the request is answered from L2 faster than the late wave gets through its 2 KSTEPS reads.)
+    __syncthreads();
+  };
+  // the general loop from tile j on (no successor pipelining, running max per tile, partial tiles): sa holds S(j)
+  auto general_loop = [&](uint32_t j) {
+    for (; j < ntiles; ++j) {
+      const int buf = j & 1;
+      if (j + 2 < ntiles) request_k(j + 2, buf);
+      if (j + 1 < ntiles) {
+        request_v(j + 1, buf ^ 1);
+        qk(sb, buf ^ 1);
+      }
+      softmax_pv(sa, j, buf, j >= nfull);
+      dma_wait_all();
+      __syncthreads();
+      if (j + 1 < ntiles) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) sa[kt] = sb[kt];
+      }
+    }
+  };
+  first_tiles();
+
   uint32_t j = 0;
-  if (nfull >= 4) {
+  const bool steady = nfull >= 4;
+  if (steady) {
+    if constexpr (NOREF) {
+      m_run = 0.0f;  // what has been accumulated when the steady state ends is relative to reference 0
+      mb_run = 0.0f;
+    } else {
     // nothing has been accumulated yet, so the first tile's max becomes the reference without any correction
     float mx_tile = sa[0][0];
 #pragma unroll
@@ -513,6 +564,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[kt][i]);
     m_run = half_max(mx_tile);
     mb_run = m_run * scale_log2;
+    }
     if constexpr (PRESCALE) {
       // from here to the end of the steady state the score tiles are kept relative to the reference
 #pragma unroll
@@ -553,20 +605,32 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
         for (int i = 0; i < 16; ++i) sa[kt][i] += mb_run;
     }
   }
-  // the last tiles (no successor, or a partial one): same steps with run-time conditions; sa holds S(j)
-  for (; j < ntiles; ++j) {
-    const int buf = j & 1;
-    if (j + 2 < ntiles) request_k(j + 2, buf);
-    if (j + 1 < ntiles) {
-      request_v(j + 1, buf ^ 1);
-      qk(sb, buf ^ 1);
-    }
-    softmax_pv(sa, j, buf, j >= nfull);
-    dma_wait_all();
-    __syncthreads();
-    if (j + 1 < ntiles) {
+  // the last tiles (no successor, or a partial one)
+  general_loop(j);
+  if constexpr (NOREF) {
+    if (steady) {
+      // did the pass without a reference stay inside the floating-point range, for every wave of the workgroup?
+      const float row_sum = half_sum(l_run);
+      const bool lane_bad = bad || !(row_sum > 0x1p-100f && row_sum < INFINITY);
+      // one word per wave in the tile memory, which nobody reads any more after the loop's last barrier
+      int* wave_flags = reinterpret_cast<int*>(&smem[0][0][0]);
+      if (lane == 0) wave_flags[wave] = __builtin_amdgcn_ballot_w64(lane_bad) != 0;
+      __syncthreads();
+      int redo = 0;
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) sa[kt] = sb[kt];
+      for (int w = 0; w < NWAVES; ++w) redo |= wave_flags[w];
+      if (redo != 0) {
+        __syncthreads();  // every wave has read the flags before the tile requests overwrite them
+        // throw the pass away and compute the item again, every tile through the general loop
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[t][i] = 0.0f;
+        m_run = -INFINITY;
+        l_run = 0.0f;
+        first_tiles();
+        general_loop(0);
+      }
     }
   }
 

@@ -303,6 +303,7 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   __syncthreads();
   f32x16 sa[QB][KT], sb[QB][KT];
   qk(sa, 0);
+  __syncthreads();  // K(2) is requested into the buffer of K(0): not before every wave has read K(0)
 
   // Steady state (tiles j and j+1 are full tiles).  One trip runs from barrier to barrier and is written as a
   // sequence of MFMA slots, everything else dealt out between the MFMAs a few vector instructions per slot, so
