@@ -529,22 +529,19 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     // once the request is answered from L2 faster than the late wave gets through its 2 KSTEPS reads.)
     __syncthreads();
   };
-  // the general loop from tile j on (no successor pipelining, running max per tile, partial tiles): sa holds S(j)
+  // the general loop from tile j on (running max per tile, partial tiles): sa holds S(j).  S(j+1) is computed
+  // after the softmax of tile j, into the same registers: this loop runs for the last one to three tiles (and
+  // for the second pass of an item), and a second score tile alive next to the softmax's temporaries is what
+  // would push the kernel over its register budget.
   auto general_loop = [&](uint32_t j) {
     for (; j < ntiles; ++j) {
       const int buf = j & 1;
       if (j + 2 < ntiles) request_k(j + 2, buf);
-      if (j + 1 < ntiles) {
-        request_v(j + 1, buf ^ 1);
-        qk(sb, buf ^ 1);
-      }
+      if (j + 1 < ntiles) request_v(j + 1, buf ^ 1);
       softmax_pv(sa, j, buf, j >= nfull);
+      if (j + 1 < ntiles) qk(sa, buf ^ 1);
       dma_wait_all();
       __syncthreads();
-      if (j + 1 < ntiles) {
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) sa[kt] = sb[kt];
-      }
     }
   };
   first_tiles();
