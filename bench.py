@@ -95,8 +95,10 @@ def time_steps(torch, fn, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults: the launch time keeps falling over the first two dozen launches of a process (2.2 ms -> 1.8 ms
+    # while the clocks settle), so the warm-up is longer than the launch count alone would suggest
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, a kernel of known traffic for scaling profiler counters")

@@ -2,8 +2,8 @@
 //
 // The data path is the one of attention_bf16_direct.h (K and V tiles go from global memory straight into
 // swizzled LDS tiles, K operands by ds_read_b128, V operands by the transposing ds_read_b64_tr_b16, scores
-// of tile j+1 on the matrix pipe while the softmax of tile j runs on the vector pipe, no row max in the
-// steady state).  What differs: a wave owns QB = 2 blocks of 32 query rows instead of one, so every K or V
+// of tile j+1 on the matrix pipe while the softmax of tile j runs on the vector pipe; the steady state takes no
+// row max and no reference at all, see below).  What differs: a wave owns QB = 2 blocks of 32 query rows instead of one, so every K or V
 // operand that is read from LDS feeds two MFMAs (one per block), which halves the LDS reads per flop.  At
 // d = 64 the registers allow that with two waves per SIMD (O 64 + two score tiles of 32 keys 64 + Q 32 + P 16),
 // which a wave needs because only about half of an MFMA's 32 cycles can be covered by its own vector work;
@@ -84,8 +84,7 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   }
 
   f32x16 o[QB][DT];
-  float m_run[QB], l_run[QB], mb_run[QB];  // running max of the raw scores; running sum over this half-wave's
-                                           // keys; m_run * scale_log2 (kept while the steady-state loop runs)
+  float m_run[QB], l_run[QB];  // running max of the scores; running sum over this half-wave's keys
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
 #pragma unroll
@@ -94,7 +93,6 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
       for (int i = 0; i < 16; ++i) o[b][t][i] = 0.0f;
     m_run[b] = -INFINITY;
     l_run[b] = 0.0f;
-    mb_run[b] = 0.0f;
   }
 
   const uint32_t nfull_tiles = p.nk / BN;  // tiles that lie entirely inside nk
@@ -296,14 +294,18 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
     else request_tile(t * BN, buf, Yes{}, No{}, Yes{});
   };
 
-  request_k(0, 0);
-  request_v(0, 0);
-  if (ntiles > 1) request_k(1, 1);
-  dma_wait_all();
-  __syncthreads();
   f32x16 sa[QB][KT], sb[QB][KT];
-  qk(sa, 0);
-  __syncthreads();  // K(2) is requested into the buffer of K(0): not before every wave has read K(0)
+  // tiles 0 and 1 of K and tile 0 of V into LDS, then S(0)
+  auto first_tiles = [&]() {
+    request_k(0, 0);
+    request_v(0, 0);
+    if (ntiles > 1) request_k(1, 1);
+    dma_wait_all();
+    __syncthreads();
+    qk(sa, 0);
+    __syncthreads();  // K(2) is requested into the buffer of K(0): not before every wave has read K(0)
+  };
+  first_tiles();
 
   // Steady state (tiles j and j+1 are full tiles).  One trip runs from barrier to barrier and is written as a
   // sequence of MFMA slots, everything else dealt out between the MFMAs a few vector instructions per slot, so
@@ -328,21 +330,38 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   constexpr int XLEAD = ATTN_Q64_XLEAD;
   static_assert(NPAIR % 4 == 0 && 2 * WLW <= NPRE && XLEAD >= 0 && XLEAD < NQK, "slot shape");
 
-  f32x16 negmb16[QB];  // -reference in every element: the addend of a score tile's first MFMA
+  // The steady state takes P = exp2(score) as it is, with no reference at all (Q carries scale * log2(e)).  The
+  // normalised result does not depend on the reference, and with probabilities rounded to bf16 (same exponent
+  // range as f32) neither does its precision, as long as nothing overflows or a whole row underflows.  A wave
+  // notes (without branching) whether a tile's row sum reached 2^80 and, at the end, whether a row sum fell below
+  // 2^-100; if any wave of the workgroup did, the workgroup throws the pass away and computes the item again
+  // with the general loop, which takes the running max tile by tile.
+  bool bad = false;
+  // The first NEARLY pairs of a tile and block are computed one trip early, one per output slot of the
+  // previous tile (those slots carry no other vector work, while every other slot of the trip carries one pair);
+  // they wait in `early`, and the row-sum parts live across trips with them
+  constexpr int NEARLY = 2;
+  uint32_t early[QB][NEARLY];
+  float psum[QB][2];
 #pragma unroll
-  for (int b = 0; b < QB; ++b) negmb16[b] = zero16;
+  for (int b = 0; b < QB; ++b) psum[b][0] = psum[b][1] = 0.0f;
+  const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+  // pair pr of block b of score tile s: two exponentials, their bf16 rounding, the row-sum part
+  auto exp_pair_of = [&](const f32x16 (&s)[QB][KT], int b, int pr) -> uint32_t {
+    const int pkt = pr / 8, i = 2 * (pr % 8);
+    const float e0 = fast_exp2(s[b][pkt][i]);  // relative to the reference already
+    const float e1 = fast_exp2(s[b][pkt][i + 1]);
+    const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
+    psum[b][pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[b][pr & 1], false);
+    uint32_t packed = __builtin_bit_cast(uint32_t, pair);
+    asm volatile("" : "+v"(packed), "+v"(psum[b][pr & 1]));
+    return packed;
+  };
 
   struct Carry {
     bf16x8 a[DT];  // V^T operands of the last 16-key group
     u32x4 p[QB];   // its probabilities, per query block
   };
-
-  // No row max is taken in the steady state.  P = exp(S - reference) is computed against the reference the
-  // row already has; floating point is scale-free, so any reference gives the same normalised result as long
-  // as nothing overflows.  The tile's row sum (a by-product) is checked before the tile's PV product: if it is
-  // not below 2^40 (this includes inf and NaN) for any row of the wave, the reference is moved up to the tile
-  // max, O and l are corrected by the exp-shift factor, and the tile's probabilities are recomputed.
-  constexpr float SUM_GUARD = 1099511627776.0f;  // 2^40
 
   // any_k_tag: tile j+2 may be partial or absent (the last steady-state trip); otherwise it is a full tile
   auto fast_step = [&](uint32_t j, int buf, f32x16 (&s_cur)[QB][KT], f32x16 (&s_next)[QB][KT], const Carry& cin,
@@ -389,29 +408,19 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
     // pq[b][g] is the B operand of 16-key group g of block b.  The empty asm statements tie each slot's vector
     // work to its slot.
     u32x4 pq[QB][NPAIR / 4];
-    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
-    float psum[QB][2];
-    float mb[QB];
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-      psum[b][0] = psum[b][1] = 0.0f;
-      mb[b] = mb_run[b];
-    }
-    // pair n of the trip: block n / NPAIR, pair n % NPAIR
+    for (int b = 0; b < QB; ++b)
+#pragma unroll
+      for (int w = 0; w < NEARLY; ++w) pq[b][0][w] = early[b][w];
+    // late pair n of the trip: block n / NLATE, pair NEARLY + n % NLATE
+    constexpr int NLATE = NPAIR - NEARLY;
     auto exp_pair = [&](int n) {
-      const int b = n / NPAIR, pr = n % NPAIR;
-      const int pkt = pr / 8, i = 2 * (pr % 8);
-      const float e0 = fast_exp2(s_cur[b][pkt][i]);  // relative to the reference already
-      const float e1 = fast_exp2(s_cur[b][pkt][i + 1]);
-      const bf16x2 pair = {(bf16_t)e0, (bf16_t)e1};
-      psum[b][pr & 1] = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum[b][pr & 1], false);
-      uint32_t packed = __builtin_bit_cast(uint32_t, pair);
-      asm volatile("" : "+v"(packed), "+v"(psum[b][pr & 1]));
-      pq[b][pr / 4][pr % 4] = packed;
+      const int b = n / NLATE, pr = NEARLY + n % NLATE;
+      pq[b][pr / 4][pr % 4] = exp_pair_of(s_cur, b, pr);
     };
     auto pairs_for_slot = [&](int g) {
 #pragma unroll
-      for (int n = g * (QB * NPAIR) / NPRE; n < (g + 1) * (QB * NPAIR) / NPRE; ++n) exp_pair(n);
+      for (int n = g * (QB * NLATE) / NPRE; n < (g + 1) * (QB * NLATE) / NPRE; ++n) exp_pair(n);
     };
 
     // ---- carried slots: last key group of tile j-1
@@ -435,57 +444,20 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
 #pragma unroll
       for (int b = 0; b < QB; ++b) {
         s_next[b][kt] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[b][ks], ks == 0 ? negmb16[b] : s_next[b][kt], 0, 0, 0);
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[n], qf[b][ks], ks == 0 ? zero16 : s_next[b][kt], 0, 0, 0);
         request_for_slot(QB * (DT + n) + b);
         pairs_for_slot(QB * (DT + n) + b);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 
-    // ---- guard (see above); O at this point holds everything up to and including tile j-1
-    bool safe = true;
+    // ---- the tile's row sums: noted when out of range (acted upon after the pass), then added
 #pragma unroll
-    for (int b = 0; b < QB; ++b) safe = safe && (psum[b][0] + psum[b][1] < SUM_GUARD);
-    if (__builtin_amdgcn_ballot_w64(!safe)) {
-#pragma unroll
-      for (int b = 0; b < QB; ++b) {
-        float mx = s_cur[b][0][0];
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_cur[b][kt][i]);
-        mx = half_max(mx) + mb_run[b];  // the scores are relative to the reference they were computed against
-        const bool move = mx * scale_log2 > mb_run[b];  // the reference only moves up
-        const float mb_new = move ? mx * scale_log2 : mb_run[b];
-        const float alpha = fast_exp2(mb_run[b] - mb_new);
-        {
-          // both score tiles in flight were accumulated against the old reference
-          const float delta = mb_new - mb_run[b];
-#pragma unroll
-          for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              s_cur[b][kt][i] -= delta;
-              s_next[b][kt][i] -= delta;
-            }
-#pragma unroll
-          for (int i = 0; i < 16; ++i) negmb16[b][i] = -mb_new;
-        }
-        m_run[b] = move ? mx : m_run[b];
-        mb_run[b] = mb_new;
-        l_run[b] *= alpha;
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[b][t][i] *= alpha;
-        mb[b] = mb_new;
-        psum[b][0] = psum[b][1] = 0.0f;
-      }
-#pragma unroll
-      for (int n = 0; n < QB * NPAIR; ++n) exp_pair(n);
+    for (int b = 0; b < QB; ++b) {
+      bad = bad || !(psum[b][0] + psum[b][1] < 0x1p80f);
+      l_run[b] += psum[b][0] + psum[b][1];
+      psum[b][0] = psum[b][1] = 0.0f;
     }
-#pragma unroll
-    for (int b = 0; b < QB; ++b) l_run[b] += psum[b][0] + psum[b][1];
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- output slots of tile j, all key groups but the last
@@ -496,6 +468,10 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
 #pragma unroll
       for (int b = 0; b < QB; ++b) {
         o[b][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[NQK + m], __builtin_bit_cast(bf16x8, pq[b][s4]), o[b][t], 0, 0, 0);
+        // early pairs of tile j+1, dealt out over the output slots
+#pragma unroll
+        for (int n = (QB * m + b) * (QB * NEARLY) / (QB * NMAIN); n < (QB * m + b + 1) * (QB * NEARLY) / (QB * NMAIN); ++n)
+          early[n / NEARLY][n % NEARLY] = exp_pair_of(s_next, n / NEARLY, n % NEARLY);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -508,25 +484,15 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   };
 
   uint32_t j = 0;
-  if (nfull >= 4) {
-    // nothing has been accumulated yet, so the first tile's max becomes the reference without any correction
+  const bool steady = nfull >= 4;
+  if (steady) {
+    // what has been accumulated when the steady state ends is relative to reference 0
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-      float mx_tile = sa[b][0][0];
+    for (int b = 0; b < QB; ++b) m_run[b] = 0.0f;
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
+    for (int b = 0; b < QB; ++b)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx_tile = fmaxf(mx_tile, sa[b][kt][i]);
-      m_run[b] = half_max(mx_tile);
-      mb_run[b] = m_run[b] * scale_log2;
-      // from here to the end of the steady state the score tiles are kept relative to the reference
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sa[b][kt][i] -= mb_run[b];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) negmb16[b][i] = -mb_run[b];
-    }
+      for (int w = 0; w < NEARLY; ++w) early[b][w] = exp_pair_of(sa, b, w);
     // the first trip has no predecessor: its carried slots add zero
     Carry ca, cb;
 #pragma unroll
@@ -543,30 +509,53 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
 #pragma unroll
       for (int b = 0; b < QB; ++b)
         o[b][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ca.a[t], __builtin_bit_cast(bf16x8, ca.p[b]), o[b][t], 0, 0, 0);
-    // the general loop below works on scores as they are
-#pragma unroll
-    for (int b = 0; b < QB; ++b)
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sa[b][kt][i] += mb_run[b];
   }
-  // the last tiles (no successor, or a partial one): same steps with run-time conditions; sa holds S(j)
-  for (; j < ntiles; ++j) {
-    const int buf = j & 1;
-    if (j + 2 < ntiles) request_k(j + 2, buf);
-    if (j + 1 < ntiles) {
-      request_v(j + 1, buf ^ 1);
-      qk(sb, buf ^ 1);
+  // the general loop from tile j on (running max per tile, partial tiles): sa holds S(j); S(j+1) is computed
+  // after the softmax of tile j, into the same registers
+  auto general_loop = [&](uint32_t j) {
+    for (; j < ntiles; ++j) {
+      const int buf = j & 1;
+      if (j + 2 < ntiles) request_k(j + 2, buf);
+      if (j + 1 < ntiles) request_v(j + 1, buf ^ 1);
+      softmax_pv(sa, j, buf, j >= nfull);
+      if (j + 1 < ntiles) qk(sa, buf ^ 1);
+      dma_wait_all();
+      __syncthreads();
     }
-    softmax_pv(sa, j, buf, j >= nfull);
-    dma_wait_all();
-    __syncthreads();
-    if (j + 1 < ntiles) {
+  };
+  // the last tiles (no successor, or a partial one)
+  general_loop(j);
+  {
+    if (steady) {
+      // did the pass without a reference stay inside the floating-point range, for every wave of the workgroup?
+      bool lane_bad = bad;
 #pragma unroll
-      for (int b = 0; b < QB; ++b)
+      for (int b = 0; b < QB; ++b) {
+        const float row_sum = half_sum(l_run[b]);
+        lane_bad = lane_bad || !(row_sum > 0x1p-100f && row_sum < INFINITY);
+      }
+      // one word per wave in the tile memory, which nobody reads any more after the loop's last barrier
+      int* wave_flags = reinterpret_cast<int*>(&smem[0][0][0]);
+      if (lane == 0) wave_flags[wave] = __builtin_amdgcn_ballot_w64(lane_bad) != 0;
+      __syncthreads();
+      int redo = 0;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) sa[b][kt] = sb[b][kt];
+      for (int w = 0; w < NWAVES; ++w) redo |= wave_flags[w];
+      if (redo != 0) {
+        __syncthreads();  // every wave has read the flags before the tile requests overwrite them
+        // throw the pass away and compute the item again, every tile through the general loop
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+#pragma unroll
+          for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[b][t][i] = 0.0f;
+          m_run[b] = -INFINITY;
+          l_run[b] = 0.0f;
+        }
+        first_tiles();
+        general_loop(0);
+      }
     }
   }
 
