@@ -3,4 +3,13 @@
 ``from i_amd import Component as i, Tensor, I`` mirrors the reference's
 ``from ilang import Component as i, Tensor, I``.
 """
-from .ilang import Component, I, Tensor, i  # noqa: F401
+_FRONTEND = ("Component", "I", "Tensor", "i")
+__all__ = list(_FRONTEND)
+
+
+def __getattr__(name):
+    # resolved on first use, so that ``i_amd.build`` can (re)build the native library before anything loads it
+    if name in _FRONTEND:
+        from . import ilang
+        return getattr(ilang, name)
+    raise AttributeError(f"module 'i_amd' has no attribute {name!r}")

@@ -39,6 +39,8 @@ core.i_hip_attention.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, sz,
 core.i_hip_attention.restype = ctypes.c_int
 core.i_hip_gemm_nt_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nt_bf16.restype = ctypes.c_int
+core.i_hip_gemm_nn_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
+core.i_hip_gemm_nn_bf16.restype = ctypes.c_int
 core.i_hip_gemm_nt_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nt_f32.restype = ctypes.c_int
 core.i_hip_row_softmax.argtypes = [vp, vp, sz, sz, vp]

@@ -222,7 +222,8 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
                                        a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j);
     }
     case Recognized::GemmNN: {
-      // b [B.., K, J] is transposed into a stream-ordered temporary [B.., J, K], then the NT kernel runs
+      // b [B.., K, J]: the direct bf16 kernels read it in place; otherwise it is transposed into a stream-ordered
+      // temporary [B.., J, K] and the NT kernel runs
       const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
       const size_t nb = r.batch_rank;
       size_t bh = 1;
@@ -233,6 +234,13 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       const size_t m = a[nb], k = a[nb + 1], n = b[nb + 1];
       if (b[nb] != k) return "gemm operands disagree on the contracted extent";
       const bool f32 = run.dtype_of(r.a.buffer) == DType::F32;
+      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k)) {
+        // the direct kernels read a row-major right operand themselves
+        void* out = nullptr;
+        if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+        return ihip::launch_gemm_nn_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh, m, n, k,
+                                         run.stream, r.tile_i, r.tile_j);
+      }
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
       if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;

@@ -335,7 +335,7 @@ std::string Recognized::describe() const {
   switch (kind) {
     case Attention: return (has_scale ? "hand-written FlashAttention kernel (scaled scores)" : "hand-written FlashAttention kernel") + tiles;
     case GemmNT: return "hand-written MFMA GEMM (transposed right operand)" + tiles;
-    case GemmNN: return "hand-written MFMA GEMM (right operand transposed on the device first)" + tiles;
+    case GemmNN: return "hand-written MFMA GEMM (row-major right operand: read in place when bf16 with k % 64 == 0 and n % 8 == 0, transposed on the device first otherwise)" + tiles;
     case RowSoftmax: return "hand-written row-softmax kernel";
     case RowMaxShift: return "hand-written row kernel (x - row max)";
     case RowNormalize: return "hand-written row kernel (x / row sum)";

@@ -26,6 +26,10 @@ int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t
   return finish(ihip::launch_gemm_nt_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream));
 }
 
+int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k, void* stream) {
+  return finish(ihip::launch_gemm_nn_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream));
+}
+
 int i_hip_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k, void* stream) {
   return finish(ihip::launch_gemm_nt_f32(a, b, c, bh, m, n, k, (hipStream_t)stream));
 }

@@ -138,6 +138,40 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
 
+// NN product on the direct kernels: whole 64-wide k slabs, 16-byte chunks along n, 32-bit byte offsets inside a slab
+static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n) {
+  if (k == 0 || k % 64 != 0 || n % 8 != 0 || k > (size_t(1) << 22) || n > (size_t(1) << 24) || bh > 65535) return 0;
+  if (!fits_u32(m) || !fits_u32(n)) return 0;
+  const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
+  unsigned tile = t256 >= 128 ? 256 : 128;
+  if (tile_m == 256 && tile_n == 256) tile = 256;
+  if (tile_m == 128 && tile_n == 128) tile = 128;
+  if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
+  return tile;
+}
+
+bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return gemm_nn_tile(bh, m, n, k, 0, 0) != 0; }
+
+Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m, size_t tile_n) {
+  const unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
+  if (tile == 0) return "gemm_nn kernel: needs k % 64 == 0 and n % 8 == 0 (and extents within its offset range)";
+  if (bh == 0 || m == 0 || n == 0) return {};
+  if (!a || !b || !c) return "gemm_nn kernel: null device pointer";
+  GemmParams p{};
+  p.a = a; p.b = b; p.c = c;
+  p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.tiles_m = (uint32_t)((m + tile - 1) / tile);
+  p.tiles_n = (uint32_t)((n + tile - 1) / tile);
+  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs
+  const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+  if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
+  hipFunction_t fn;
+  if (Err e = builtin_function(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct", &fn); !e.empty())
+    return e;
+  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
+}
+
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 32 == 0 && k <= (size_t(1) << 21); }
 
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,

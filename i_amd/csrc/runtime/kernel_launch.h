@@ -28,6 +28,12 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
                         hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
 bool gemm_nt_bf16_supported(size_t k);
 
+// c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
+// Needs k % 64 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
+Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
+bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
+
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 32 == 0
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
                        hipStream_t stream);
@@ -37,7 +43,7 @@ bool gemm_nt_f32_supported(size_t k);
 // mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize); 3: y = exp(x)
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0);
 
-// dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  The NN product runs as transpose + NT kernel.
+// dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  An NN product that the direct kernels cannot read runs as transpose + NT kernel.
 Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,
                      hipStream_t stream);
 

@@ -131,11 +131,11 @@ class _OwnedOutputs:
     def __init__(self, outputs):
         self.outputs = outputs
 
-    def __del__(self):
+    def __del__(self, _core=core):
         outputs = getattr(self, "outputs", None)
         if outputs is not None:
             self.outputs = None
-            core.i_outputs_free(outputs)
+            _core.i_outputs_free(outputs)
 
 
 def _is_torch(x):
@@ -228,13 +228,13 @@ class Component:
         self._ptr = _check_ptr(_ptr)
         self._program = None
 
-    def __del__(self):
+    def __del__(self, _core=core):  # bound at definition: module globals may be gone at interpreter shutdown
         program, ptr = getattr(self, "_program", None), getattr(self, "_ptr", None)
         if program:
-            core.i_program_free(program)
+            _core.i_program_free(program)
             self._program = None
         if ptr:
-            core.i_component_free(ptr)
+            _core.i_component_free(ptr)
             self._ptr = None
 
     def _bin(self, other, fn):

@@ -74,6 +74,15 @@ int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c,
                        size_t bh, size_t m, size_t n, size_t k, void* stream);
 
 /*
+ * The product with a row-major right operand,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,k,n]  (bf16 a, b, f32 c):
+ * the fused kernel for  i("ik*kj~ijk") >> i("+ijk~ij ...")  (ilang-python/test.py:52-56) and for the demo's
+ * standalone mm,  i("ij*jk~ikj") >> i("+ikj~ik ...")  (ilang-python/flash-attn.py:51).  Requires k % 64 == 0
+ * and n % 8 == 0; other shapes go through a transpose and i_hip_gemm_nt_bf16.
+ */
+int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c,
+                       size_t bh, size_t m, size_t n, size_t k, void* stream);
+
+/*
  * The same mm_t with f32 a, b, c and f32 products and sums (f32 MFMA), the reference's own
  * arithmetic type: what the host f32 ABI of i.h dispatches to.  Requires k % 32 == 0.
  */

@@ -207,7 +207,7 @@ def test_config3_mm_t_through_the_host_f32_abi(torch):
     close(c[:, cols], oracle.mm_t(a, b[cols]), RTOL_F32)
 
 
-# ------------------------------------------------------------------ NN products: right operand transposed on the device, then the NT kernel
+# ------------------------------------------------------------------ NN products: row-major right operand (read in place, or transposed on the device first)
 MATMUL = "ik*kj~ijk|i:16,k:16|ii'jkk'", "+ijk~ij|i:16,k:16|ii'j!kk'0"  # test.py's matmul with larger splits
 
 
@@ -215,7 +215,7 @@ MATMUL = "ik*kj~ijk|i:16,k:16|ii'jkk'", "+ijk~ij|i:16,k:16|ii'j!kk'0"  # test.py
 def test_matmul_nn_f32_vs_emitted_c(torch, m, k, n):
     a, b = rnd((m, k), 1), rnd((k, n), 2)
     comp = i(MATMUL[0]) >> i(MATMUL[1])
-    assert "right operand transposed" in comp._code()
+    assert "row-major right operand" in comp._code()
     close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
 
 
@@ -234,7 +234,7 @@ def test_matmul_nn_bf16_device_vs_torch(torch, m, k, n):
 def test_matmul_nn_batched_and_the_demo_mm(torch):
     a, b = rnd((2, 3, 40, 64), 1), rnd((2, 3, 64, 50), 2)
     batched = i("bhik*bhkj~bhijk | i:16,k:16 | bhkii'jk'") >> i("+bhijk~bhij | i:16,k:16 | bhkii'jk'0")
-    assert "right operand transposed" in batched._code()
+    assert "row-major right operand" in batched._code()
     close(batched.exec_numpy(a, b), np.einsum("bhik,bhkj->bhij", a.astype(np.float64), b.astype(np.float64)), RTOL_F32)
     p_, v_ = rnd((48, 96), 3), rnd((96, 64), 4)
     mm = i("ij*jk~ikj | i:16,j:16 | jii'kj'") >> i("+ikj~ik | i:16,j:16 | jii'kj'0")
@@ -265,7 +265,7 @@ def test_naive_attention_uses_both_gemm_forms(torch):
     q, k, v = rnd((96, 64), 1), rnd((96, 64), 2), rnd((96, 64), 3)
     comp = naive()
     code = comp._code()
-    assert "transposed right operand" in code and "right operand transposed on the device first" in code
+    assert "transposed right operand" in code and "row-major right operand" in code
     assert np.allclose(comp.exec_numpy(q, k, v), oracle.np_attention64(q, k, v), rtol=3e-4, atol=5e-5)
 
 

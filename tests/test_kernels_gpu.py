@@ -318,6 +318,32 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, dire
     assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 264, 128), (2, 600, 520, 192), (1, 1, 8, 256),
+                                      (3, 257, 248, 320), (1, 130, 1000, 64)])
+@pytest.mark.parametrize("direct", ["256", "128"])
+def test_gemm_nn_bf16_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
+    """Row-major right operand (c = a b, b [k, n]) on the direct kernels: 1 to 5 k-slabs, edge tiles on both
+    axes (n a multiple of 8 only), several batches, both workgroup tiles."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
+    t = env.torch
+    a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((bh, k, n), 2, "uniform"))
+    ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+    cd = t.full((bh, m, n), float("nan"), device="cuda")
+    env.nat.check(env.nat.core.i_hip_gemm_nn_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+    t.cuda.synchronize()
+    assert_close(cd.cpu().numpy(), oracle.mm_t(a, np.ascontiguousarray(b.transpose(0, 2, 1))), RTOL_BF16)
+
+
+def test_gemm_nn_bf16_rejects_what_the_direct_kernels_cannot_read(env):
+    t = env.torch
+    x = t.zeros(64 * 72, device="cuda", dtype=t.bfloat16)
+    c = t.zeros(64 * 72, device="cuda")
+    for m, n, k in ((64, 60, 64), (64, 64, 40)):
+        rc = env.nat.core.i_hip_gemm_nn_bf16(x.data_ptr(), x.data_ptr(), c.data_ptr(), 1, m, n, k, env.stream())
+        assert rc == -1 and "gemm_nn" in env.nat.last_error()
+
+
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 32), (1, 300, 260, 96), (2, 600, 520, 160), (1, 1, 1, 64),
                                       (3, 257, 255, 320), (1, 100, 70, 64)])
 @pytest.mark.parametrize("tile", ["256", "128"])
