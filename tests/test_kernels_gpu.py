@@ -204,6 +204,25 @@ def test_attention_bf16_scores_far_from_zero(env, monkeypatch, waves, d, offset)
     assert_close(gpu_attention(env, q, k, v, 1.0, bf16=True), ref, RTOL_BF16)
 
 
+@pytest.mark.parametrize("d,waves", [(128, "8"), (64, "8"), (64, "64")])
+def test_attention_bf16_large_scores_error_growth(env, monkeypatch, d, waves):
+    """The direct kernels fold scale * log2(e) into Q, rounded to bf16 once more: a perturbation of the scores that
+    grows with their magnitude.  Inputs x 1, x 2 (the recipe of the long-sequence configuration) and x 3 (scores of
+    +-35 nats, far more peaked than attention): the error against the f64 closed form stays below 1e-2, 1.5e-2
+    and 3e-2 of max |reference|; the last is looser than the 2e-2 bar of the other tests and states where it ends."""
+    monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+    bh, nq, nk = 2, 200, 1100
+    for amp, bound in ((1.0, 1e-2), (2.0, 1.5e-2), (3.0, 3e-2)):
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s) * np.float32(amp)) for s, n in ((1, nq), (2, nk), (3, nk)))
+        scale = float(np.float32(1.0 / np.sqrt(d)))
+        s = np.einsum("bik,bjk->bij", q.astype(np.float64), k.astype(np.float64)) * scale
+        p = np.exp(s - s.max(axis=-1, keepdims=True))
+        ref = np.einsum("bij,bjk->bik", p / p.sum(axis=-1, keepdims=True), v.astype(np.float64))
+        got = gpu_attention(env, q, k, v, scale, bf16=True)
+        err = np.abs(got - ref).max() / np.abs(ref).max()
+        assert err <= bound, f"inputs x {amp}: error {err} > {bound}"
+
+
 @pytest.mark.parametrize("q64", [False, True])
 def test_attention_bf16_direct_negative_and_zero_scale(env, monkeypatch, q64):
     if q64:
