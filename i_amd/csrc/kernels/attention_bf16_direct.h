@@ -31,13 +31,18 @@
 // vector pipe, the scores of tile j+1 are computed on the matrix pipe, so K is consumed
 // one trip before V.  K(j+2) and V(j+1) are requested early in trip j, into the buffer
 // of K(j) and of V(j-1) (both last read before the barrier that opens the trip), and are
-// awaited (vmcnt(0) + barrier) at the end of the trip.  One barrier per tile.
+// awaited (vmcnt(0) + barrier) at the end of the trip.  One barrier per tile, and one after the
+// first score tile (K(2) goes into the buffer of K(0)).
 //
 // Other differences from attention_bf16.h:
-//   * in the steady state no row max is taken at all: probabilities are computed against the
-//     reference the row already has and the reference is only moved (with the exp-shift
+//   * in the steady state no row max is taken at all.  d = 64: probabilities are computed against
+//     the reference the row already has and the reference is only moved (with the exp-shift
 //     correction of O and l) when a tile's row sum reaches 2^40, checked before that tile's
-//     PV product; the remaining tiles move it when the tile max exceeds it by 2^8;
+//     PV product.  d = 128: no reference either (P = exp2 of the score as it is); a workgroup
+//     whose rows leave the floating-point range computes its item a second time with the
+//     running max.  The remaining tiles move the reference when the tile max exceeds it by 2^8;
+//   * scale * log2(e) is folded into Q when it is loaded (one more bf16 rounding), so a score is
+//     the argument of its exp2;
 //   * the row sum is taken over the bf16-rounded probabilities with v_dot2c_f32_bf16
 //     (two terms per instruction), i.e. over exactly the weights the PV product uses.
 #pragma once
