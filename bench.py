@@ -150,7 +150,10 @@ def main():
         turn[0] += 1
         sm.into(ys[k_], xs[k_])
 
-    _, sm_ms = time_steps(torch, softmax_step, max(args.steps, 20), max(args.warmup, 4))
+    # ~0.1 ms kernels: enough launches for a timed window of tens of milliseconds, after as long a warm-up
+    # (short runs, as the profiler's counter passes use them, stay short)
+    short_steps, short_warmup = (max(args.steps, 200), max(args.warmup, 100)) if args.steps >= 20 else (args.steps, args.warmup)
+    _, sm_ms = time_steps(torch, softmax_step, short_steps, short_warmup)
     sm.into(y, x)  # the parity check below reads y
     del xs, ys
     sm_bytes = 2.0 * rows * cols * 4
@@ -162,7 +165,7 @@ def main():
     c = torch.empty(M, M, device=dev)
     mm = mm_t_component(i)
     mm.into(c, a, b)
-    _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), max(args.steps, 20), args.warmup)
+    _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), short_steps, short_warmup)
     mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
 
     # long-sequence attention (heavy running-max movement): B1 H16 N32768 d64, inputs x 2.0
