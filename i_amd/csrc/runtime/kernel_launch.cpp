@@ -36,7 +36,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   // Kernel choice for bf16:
   //   d == dv in {64, 128}: direct-to-LDS kernel; a 256-query workgroup (8 waves) halves the
   //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
-  //     larger workgroup is used when it still leaves at least two workgroups per CU
+  //     larger workgroup is used when it still leaves at least two workgroups per CU and does not pad nq by much
   //   otherwise: register-staged kernel with guarded columns
   //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512): the
   //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs
@@ -50,8 +50,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct) {
     if (query_tile == 128 || query_tile == 256) bm = (unsigned)query_tile;  // the schedule's i split
-    else if (d == 64 && (query_tile == 512 || (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256))) q64 = true;
-    else if (bh * ((nq + 255) / 256) >= 2 * 256) bm = 256;
+    else if (d == 64 && (query_tile == 512 || (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256 &&
+                                               10 * ((nq + 511) / 512 * 512) <= 11 * ((nq + 127) / 128 * 128))))
+      q64 = true;
+    else if (bh * ((nq + 255) / 256) >= 2 * 256 && 10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128))
+      bm = 256;  // ... unless rounding nq up to 256 instead of 128 adds more than 10 % of idle query rows
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
       const int waves = std::atoi(w);
       q64 = waves == 64 && d == 64;
