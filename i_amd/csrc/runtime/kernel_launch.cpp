@@ -53,8 +53,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     else if (d == 64 && (query_tile == 512 || (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256 &&
                                                10 * ((nq + 511) / 512 * 512) <= 11 * ((nq + 127) / 128 * 128))))
       q64 = true;
-    else if (bh * ((nq + 255) / 256) >= 2 * 256 && 10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128))
-      bm = 256;  // ... unless rounding nq up to 256 instead of 128 adds more than 10 % of idle query rows
+    else if (bh * ((nq + 255) / 256) >= 2 * 256 && nk >= 2560 &&
+             10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128))
+      bm = 256;  // ... on long key loops (two resident 4-wave workgroups hide each other's prologue and epilogue,
+                 // which wins up to about 2048 keys), and unless rounding nq up to 256 instead of 128 adds more
+                 // than 10 % of idle query rows
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
       const int waves = std::atoi(w);
       q64 = waves == 64 && d == 64;
