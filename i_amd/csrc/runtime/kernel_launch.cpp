@@ -36,7 +36,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   // Kernel choice for bf16:
   //   d == dv in {64, 128}: direct-to-LDS kernel; a 256-query workgroup (8 waves) halves the
   //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
-  //     larger workgroup is used when it still leaves at least two workgroups per CU and does not pad nq by much
+  //     larger workgroup is used on long key loops when it still leaves at least two workgroups per CU and does
+  //     not pad nq by much
   //   otherwise: register-staged kernel with guarded columns
   //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512): the
   //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs
