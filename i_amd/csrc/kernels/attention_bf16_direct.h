@@ -59,6 +59,9 @@
 #ifndef ATTN_NOREF
 #define ATTN_NOREF 1
 #endif
+#ifndef ATTN_STAGED_STORE
+#define ATTN_STAGED_STORE 1
+#endif
 
 template <int DPAD, int BN, int NWAVES>
 __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
@@ -112,6 +115,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr bool PRESCALE = DPAD == 64;
   constexpr bool NOREF = DPAD == 128 && ATTN_NOREF;
   constexpr bool QSCALE = PRESCALE || NOREF;
+  constexpr bool STAGED_STORE = DPAD == 128 && ATTN_STAGED_STORE;  // f32 output written through LDS (see the epilogue)
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
   const float scale_log2 = QSCALE ? 1.0f : fabsf(scale_raw) * I_LOG2_E32;
@@ -621,8 +625,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       int redo = 0;
 #pragma unroll
       for (int w = 0; w < NWAVES; ++w) redo |= wave_flags[w];
+      __syncthreads();  // every wave has read the flags before tile requests or the epilogue overwrite them
       if (redo != 0) {
-        __syncthreads();  // every wave has read the flags before the tile requests overwrite them
         // throw the pass away and compute the item again, every tile through the general loop
 #pragma unroll
         for (int t = 0; t < DT; ++t)
@@ -650,7 +654,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(o[t][4 * g + e] * inv);
           *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
-    } else {
+    } else if constexpr (!STAGED_STORE) {
       float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * d;
 #pragma unroll
       for (int t = 0; t < DT; ++t)
@@ -661,6 +665,46 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
           *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
+    }
+  }
+  if constexpr (STAGED_STORE) {
+    // f32 output through LDS.  In the accumulator layout a lane owns a query row, so a store instruction would
+    // touch 32 rows with 32 bytes each (32 cache lines); staged through the tile memory, which nobody reads any
+    // more, an instruction writes 4 rows x 256 contiguous bytes (8 lines).  Each wave stages its own 32 rows x
+    // 64 columns at a time in 8 KiB of its own: no workgroup barrier, LDS instructions of a wave execute in order.
+    // The 16-byte chunk index of a row is XOR-ed with row % 16, which spreads both the row-per-lane writes and
+    // the 4-rows-per-instruction reads over the banks.
+    if (!p.out_bf16) {
+      // lane coordinates taken afresh (behind an opaque copy), so that nothing computed here is kept in
+      // registers through the main loop
+      uint32_t tid2 = threadIdx.x;
+      asm volatile("" : "+v"(tid2));
+      const uint32_t lane = tid2 & 63, c = tid2 & 31, h = (tid2 >> 5) & 1;
+      const uint32_t wave = __builtin_amdgcn_readfirstlane(tid2 >> 6);
+      char* stage = &smem[0][0][0] + wave * 8192;
+      const uint32_t row0 = qt * BM + wave * 32;  // first query row of this wave
+      const uint32_t rows_valid = row0 < p.nq ? (p.nq - row0 < 32u ? p.nq - row0 : 32u) : 0u;
+      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + row0) * d;
+#pragma unroll
+      for (int half = 0; half < DT / 2; ++half) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = o[2 * half + tt][4 * g + e] * inv;
+            *reinterpret_cast<f32x4*>(stage + c * 256 + 16 * ((8 * tt + 2 * g + h) ^ (c & 15))) = w;
+          }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const uint32_t r = 4 * it + (lane >> 4), q = lane & 15;
+          const f32x4 w = *reinterpret_cast<const f32x4*>(stage + r * 256 + 16 * (q ^ (r & 15)));
+          if (r < rows_valid) *reinterpret_cast<f32x4*>(O + (size_t)r * d + 64 * half + 4 * q) = w;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
     }
   }
 }
