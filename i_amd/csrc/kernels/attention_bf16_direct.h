@@ -115,7 +115,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr bool PRESCALE = DPAD == 64;
   constexpr bool NOREF = DPAD == 128 && ATTN_NOREF;
   constexpr bool QSCALE = PRESCALE || NOREF;
-  constexpr bool STAGED_STORE = DPAD == 128 && ATTN_STAGED_STORE;  // f32 output written through LDS (see the epilogue)
+  // f32 output written through LDS (see the epilogue): 8 KiB of tile memory per wave
+  constexpr bool STAGED_STORE = ATTN_STAGED_STORE && NWAVES * 8192 <= 4 * TILE_BYTES;
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const uint32_t sign_flip = scale_raw < 0.0f ? 0x80008000u : 0u;
   const float scale_log2 = QSCALE ? 1.0f : fabsf(scale_raw) * I_LOG2_E32;
