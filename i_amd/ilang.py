@@ -1,23 +1,29 @@
 """Python frontend of the 𝚒 gfx950 backend.
 
-Same surface as the reference frontend (ilang-python/ilang.py:147-394):
-``Component`` / ``i(src)`` with the operators ``>> << & | ~``, the identity
-``I``, ``Tensor`` for plain Python data, ``exec``, ``exec_numpy``,
-``exec_torch``, ``into``, ``output_shapes`` and ``_code``; errors surface as
-``RuntimeError(i_error())``.  Host data takes the reference's f32 path through
-``i_exec_into`` / ``i_exec``.  In addition, ROCm torch tensors (float32 or
-bfloat16) are passed by device pointer to ``i_exec_into_device`` and never
-leave the GPU.
+The public surface is the reference frontend's (ilang-python/ilang.py:147-394): ``Component`` / ``i(src)``
+with the operators ``>> << & | ~``, the identity ``I``, ``Tensor`` for plain Python data, and the methods
+``exec``, ``exec_numpy``, ``exec_torch``, ``into``, ``output_shapes``, ``_code``; failures of the library
+surface as ``RuntimeError(i_error())``.
+
+Underneath, every operand of a call (a ``Tensor``, a NumPy array, a CPU or ROCm torch tensor, a Python number
+or nested list) is first reduced to one record, ``_Operand``: address, extents, element type, and whether
+the address is host or device memory.  A call is then routed by where its operands live: host operands take
+the reference's f32 path (``i_exec_into`` / ``i_exec``), ROCm tensors (float32 or bfloat16) are passed by
+device pointer to ``i_exec_into_device`` and never leave the GPU.
 """
+import array
 import ctypes
+import numbers
 
 from . import _native as nat
 
 core = nat.core
 _sz = ctypes.c_size_t
 _f32p = ctypes.POINTER(ctypes.c_float)
+_vp = ctypes.c_void_p
 
 
+# ---------------------------------------------------------------- the structs and prototypes of i.h / i_hip.h
 class _CTensor(ctypes.Structure):
     _fields_ = [("data", _f32p), ("shape", ctypes.POINTER(_sz)), ("rank", _sz)]
 
@@ -31,318 +37,340 @@ class _COutputs(ctypes.Structure):
 
 
 class _CDeviceTensor(ctypes.Structure):
-    _fields_ = [("data", ctypes.c_void_p), ("shape", ctypes.POINTER(_sz)), ("rank", _sz), ("dtype", ctypes.c_int)]
+    _fields_ = [("data", _vp), ("shape", ctypes.POINTER(_sz)), ("rank", _sz), ("dtype", ctypes.c_int)]
 
 
-_vp = ctypes.c_void_p
-core.i_parse.argtypes = [ctypes.c_char_p]
-core.i_parse.restype = _vp
-core.i_identity.argtypes = []
-core.i_identity.restype = _vp
-for _name in ("i_chain", "i_compose", "i_fanout", "i_pair"):
-    getattr(core, _name).argtypes = [_vp, _vp]
-    getattr(core, _name).restype = _vp
-core.i_swap.argtypes = [_vp]
-core.i_swap.restype = _vp
-core.i_code.argtypes = [_vp]
-core.i_code.restype = _vp
-core.i_compile.argtypes = [_vp]
-core.i_compile.restype = _vp
-core.i_output_count.argtypes = [_vp]
-core.i_output_count.restype = _sz
-core.i_output_ranks.argtypes = [_vp, ctypes.POINTER(_sz)]
-core.i_output_ranks.restype = ctypes.c_int
-core.i_output_shapes.argtypes = [_vp, ctypes.POINTER(_CTensor), _sz, ctypes.POINTER(ctypes.POINTER(_sz))]
-core.i_output_shapes.restype = ctypes.c_int
-core.i_exec_into.argtypes = [_vp, ctypes.POINTER(_CTensor), _sz, ctypes.POINTER(_CTensor), _sz]
-core.i_exec_into.restype = ctypes.c_int
-core.i_exec.argtypes = [_vp, ctypes.POINTER(_CTensor), _sz]
-core.i_exec.restype = _COutputs
-core.i_exec_into_device.argtypes = [_vp, ctypes.POINTER(_CDeviceTensor), _sz, ctypes.POINTER(_CDeviceTensor), _sz, _vp]
-core.i_exec_into_device.restype = ctypes.c_int
-core.i_component_free.argtypes = [_vp]
-core.i_program_free.argtypes = [_vp]
-core.i_outputs_free.argtypes = [_COutputs]
-core.i_string_free.argtypes = [_vp]
-
-_check, _check_ptr = nat.check, nat.check_ptr
+_PROTOTYPES = {
+    "i_parse": ([ctypes.c_char_p], _vp),
+    "i_identity": ([], _vp),
+    "i_chain": ([_vp, _vp], _vp),
+    "i_compose": ([_vp, _vp], _vp),
+    "i_fanout": ([_vp, _vp], _vp),
+    "i_pair": ([_vp, _vp], _vp),
+    "i_swap": ([_vp], _vp),
+    "i_code": ([_vp], _vp),
+    "i_compile": ([_vp], _vp),
+    "i_output_count": ([_vp], _sz),
+    "i_output_ranks": ([_vp, ctypes.POINTER(_sz)], ctypes.c_int),
+    "i_output_shapes": ([_vp, ctypes.POINTER(_CTensor), _sz, ctypes.POINTER(ctypes.POINTER(_sz))], ctypes.c_int),
+    "i_exec_into": ([_vp, ctypes.POINTER(_CTensor), _sz, ctypes.POINTER(_CTensor), _sz], ctypes.c_int),
+    "i_exec": ([_vp, ctypes.POINTER(_CTensor), _sz], _COutputs),
+    "i_exec_into_device": ([_vp, ctypes.POINTER(_CDeviceTensor), _sz, ctypes.POINTER(_CDeviceTensor), _sz, _vp], ctypes.c_int),
+    "i_component_free": ([_vp], None),
+    "i_program_free": ([_vp], None),
+    "i_outputs_free": ([_COutputs], None),
+    "i_string_free": ([_vp], None),
+}
+for _name, (_args, _res) in _PROTOTYPES.items():
+    getattr(core, _name).argtypes = _args
+    getattr(core, _name).restype = _res
 
 
-def _shape_array(shape):
-    shape = tuple(int(d) for d in shape)
-    return shape, (_sz * max(len(shape), 1))(*shape)
+# ---------------------------------------------------------------- operands
+class _Operand:
+    """One operand of a call, whatever object it came from."""
+
+    __slots__ = ("address", "extents", "dtype", "device", "anchor")
+
+    def __init__(self, address, extents, dtype, device, anchor):
+        self.address = address              # integer address of the first element (0 for an empty operand is fine)
+        self.extents = tuple(int(n) for n in extents)
+        self.dtype = dtype                  # nat.F32 or nat.BF16
+        self.device = device                # None: host memory; otherwise the torch device the address belongs to
+        self.anchor = anchor                # whatever must stay alive while the address is in use
 
 
-def _flatten(x):
-    if isinstance(x, (int, float)):
-        return (), [float(x)]
-    if not isinstance(x, (list, tuple)):
-        raise TypeError("Tensor expects a scalar or nested Python lists")
-    if not x:
-        return (0,), []
-    child_shape, _ = _flatten(x[0])
-    data = []
-    for item in x:
-        item_shape, item_data = _flatten(item)
-        if item_shape != child_shape:
-            raise ValueError("ragged Tensor input")
-        data.extend(item_data)
-    return (len(x),) + child_shape, data
+def _torch_like(x):
+    return all(hasattr(x, name) for name in ("data_ptr", "device", "is_contiguous", "dtype"))
 
 
-class Tensor:
-    """Host tensor built from a scalar or nested lists (ilang-python/ilang.py:147-199)."""
-
-    def __init__(self, x, shape=None):
-        if shape is None:
-            shape, data = _flatten(x)
-        else:
-            shape = tuple(int(d) for d in shape)
-            data = [float(v) for v in x]
-        self.shape = tuple(shape)
-        self._len = len(data)
-        self._data = (ctypes.c_float * max(self._len, 1))(*data)
-        self._shape, self._shape_buf = _shape_array(self.shape)
-        self._owner = None
-
-    @classmethod
-    def _from_owned(cls, owner, index):
-        raw = owner.outputs.tensors[index]
-        self = cls.__new__(cls)
-        self.shape = tuple(raw.shape[i] for i in range(raw.rank))
-        self._len = raw.len
-        self._data = raw.data
-        self._shape, self._shape_buf = _shape_array(self.shape)
-        self._owner = owner
-        return self
-
-    @property
-    def data(self):
-        return [self._data[i] for i in range(self._len)]
-
-    def _view(self):
-        return _CTensor(ctypes.cast(self._data, _f32p), self._shape_buf, len(self.shape))
-
-    def __repr__(self):
-        return f"Tensor(shape={self.shape}, data={self.data})"
+def _on_gpu(x):
+    return _torch_like(x) and x.device.type != "cpu"
 
 
-class _OwnedOutputs:
-    def __init__(self, outputs):
-        self.outputs = outputs
+def _from_numpy(x, role):
+    import numpy as np
 
-    def __del__(self, _core=core):
-        outputs = getattr(self, "outputs", None)
-        if outputs is not None:
-            self.outputs = None
-            _core.i_outputs_free(outputs)
-
-
-def _is_torch(x):
-    return hasattr(x, "data_ptr") and hasattr(x, "shape") and hasattr(x, "device")
-
-
-def _is_device_tensor(x):
-    return _is_torch(x) and str(x.device) != "cpu"
-
-
-def _input(x):
-    """(ctypes view, keepalive) for one host operand; non-f32 / non-contiguous data is copied to f32."""
-    if isinstance(x, Tensor):
-        return x._view(), x
-    try:
-        import numpy as np
-
-        if isinstance(x, np.ndarray):
-            arr = x
-            if arr.dtype != np.float32 or not arr.flags.c_contiguous:
-                arr = np.ascontiguousarray(arr, dtype=np.float32)
-            shape, shape_buf = _shape_array(arr.shape)
-            return _CTensor(arr.ctypes.data_as(_f32p), shape_buf, len(shape)), (arr, shape_buf)
-    except ImportError:
-        pass
-    if _is_torch(x):
-        if str(x.device) != "cpu":
-            raise TypeError("mixing host and device operands is not supported; move all tensors to the GPU")
-        if str(x.dtype) != "torch.float32":
-            raise TypeError("Torch tensors must be float32")
-        if not x.is_contiguous():
-            x = x.contiguous()
-        shape, shape_buf = _shape_array(tuple(x.shape))
-        return _CTensor(ctypes.cast(x.data_ptr(), _f32p), shape_buf, len(shape)), (x, shape_buf)
-    return _input(Tensor(x))
-
-
-def _inputs(xs):
-    views = [_input(x) for x in xs]
-    return (_CTensor * max(len(views), 1))(*(v[0] for v in views)), views
-
-
-def _output(x):
-    try:
-        import numpy as np
-
-        if isinstance(x, np.ndarray):
-            if x.dtype != np.float32 or not x.flags.c_contiguous:
-                raise TypeError("NumPy outputs must be float32 and C-contiguous")
-            shape, shape_buf = _shape_array(x.shape)
-            return _CTensor(x.ctypes.data_as(_f32p), shape_buf, len(shape)), (x, shape_buf)
-    except ImportError:
-        pass
-    if _is_torch(x):
-        if str(x.device) != "cpu":
-            raise TypeError("Torch outputs for host inputs must be on CPU")
-        if str(x.dtype) != "torch.float32":
-            raise TypeError("Torch outputs must be float32")
-        if not x.is_contiguous():
-            raise TypeError("Torch outputs must be contiguous")
-        shape, shape_buf = _shape_array(tuple(x.shape))
-        return _CTensor(ctypes.cast(x.data_ptr(), _f32p), shape_buf, len(shape)), (x, shape_buf)
-    raise TypeError("outputs must be NumPy arrays or Torch tensors")
+    if role == "output":
+        if x.dtype != np.float32 or not x.flags.c_contiguous:
+            raise TypeError("a NumPy output has to be a C-contiguous float32 array (it is written in place)")
+        if not x.flags.writeable:
+            raise TypeError("a NumPy output has to be writeable")
+    elif x.dtype != np.float32 or not x.flags.c_contiguous:
+        x = np.ascontiguousarray(x, dtype=np.float32)  # the host ABI carries f32 only: other inputs are copied
+    return _Operand(x.ctypes.data, x.shape, nat.F32, None, x)
 
 
 _TORCH_DTYPES = {"torch.float32": nat.F32, "torch.bfloat16": nat.BF16}
 
 
-def _device_views(tensors, what):
-    views, keep = [], []
-    for t in tensors:
-        if not _is_device_tensor(t):
-            raise TypeError(f"{what} must all be GPU tensors")
-        if str(t.dtype) not in _TORCH_DTYPES:
-            raise TypeError(f"{what} must be float32 or bfloat16")
-        if not t.is_contiguous():
-            raise TypeError(f"{what} must be contiguous")
-        shape, shape_buf = _shape_array(tuple(t.shape))
-        views.append(_CDeviceTensor(t.data_ptr(), shape_buf, len(shape), _TORCH_DTYPES[str(t.dtype)]))
-        keep.append((t, shape_buf))
-    return (_CDeviceTensor * max(len(views), 1))(*views), keep
+def _from_torch(x, role):
+    dtype = _TORCH_DTYPES.get(str(x.dtype))
+    if x.device.type == "cpu":
+        if dtype != nat.F32:
+            raise TypeError(f"a CPU torch {role} has to be float32, got {x.dtype}")
+        if not x.is_contiguous():
+            if role == "output":
+                raise TypeError("a torch output has to be contiguous (it is written in place)")
+            x = x.contiguous()
+        return _Operand(x.data_ptr(), x.shape, nat.F32, None, x)
+    if dtype is None:
+        raise TypeError(f"a GPU {role} has to be float32 or bfloat16, got {x.dtype}")
+    if not x.is_contiguous():
+        raise TypeError(f"a GPU {role} has to be contiguous")
+    return _Operand(x.data_ptr(), x.shape, dtype, x.device, x)
 
 
+def _operand(x, role):
+    if isinstance(x, Tensor):
+        return x._operand()
+    if _torch_like(x):
+        return _from_torch(x, role)
+    if type(x).__module__.split(".")[0] == "numpy" and hasattr(x, "ctypes"):
+        return _from_numpy(x, role)
+    if role == "output":
+        raise TypeError(f"an output has to be a NumPy array or a torch tensor, got {type(x).__name__}")
+    return Tensor(x)._operand()
+
+
+def _extent_buffer(extents):
+    return (_sz * max(len(extents), 1))(*extents)
+
+
+def _pack(operands, on_device):
+    """The C array for a list of operands, plus the objects that must outlive the call."""
+    keep = [op.anchor for op in operands]
+    records = []
+    for op in operands:
+        dims = _extent_buffer(op.extents)
+        keep.append(dims)
+        if on_device:
+            records.append(_CDeviceTensor(op.address, dims, len(op.extents), op.dtype))
+        else:
+            records.append(_CTensor(ctypes.cast(op.address, _f32p), dims, len(op.extents)))
+    kind = _CDeviceTensor if on_device else _CTensor
+    return (kind * max(len(records), 1))(*records), keep
+
+
+def _placement(operands, what):
+    """None when every operand is host memory, the torch device when every operand is on one GPU."""
+    devices = {op.device for op in operands}
+    if len(devices) > 1:
+        raise TypeError(f"{what} live in different places ({', '.join(sorted(str(d or 'host') for d in devices))}); "
+                        "move them all to one GPU or all to the host")
+    return devices.pop() if devices else None
+
+
+# ---------------------------------------------------------------- Tensor
+def _measure(x):
+    """Extents of a number or of rectangular nested sequences, judged along the first element of each level."""
+    extents = []
+    while isinstance(x, (list, tuple)):
+        extents.append(len(x))
+        if not x:
+            break
+        x = x[0]
+    else:
+        if not isinstance(x, numbers.Real):
+            raise TypeError(f"Tensor data has to be a number or nested lists of numbers, found {type(x).__name__}")
+    return tuple(extents)
+
+
+def _pour(x, extents, level, out):
+    if level == len(extents):
+        if not isinstance(x, numbers.Real):
+            raise TypeError(f"Tensor data has to be a number or nested lists of numbers, found {type(x).__name__}")
+        out.append(float(x))
+        return
+    if not isinstance(x, (list, tuple)) or len(x) != extents[level]:
+        raise ValueError(f"Tensor data is not rectangular: expected {extents[level]} items at depth {level}")
+    for item in x:
+        _pour(item, extents, level + 1, out)
+
+
+class Tensor:
+    """A host f32 tensor made from a Python number or nested lists (reference: ilang-python/ilang.py:147-199).
+    ``Tensor(values, shape)`` takes flat values.  ``.shape`` is a tuple, ``.data`` the flat list of values."""
+
+    def __init__(self, x, shape=None):
+        values = array.array("f")
+        if shape is None:
+            self.shape = _measure(x)
+            _pour(x, self.shape, 0, values)
+        else:
+            self.shape = tuple(int(n) for n in shape)
+            values.extend(float(v) for v in x)
+            count = 1
+            for n in self.shape:
+                count *= n
+            if len(values) != count:
+                raise ValueError(f"shape {self.shape} holds {count} values, got {len(values)}")
+        self._values = values
+
+    @classmethod
+    def _take(cls, owned):
+        """Copies one library-owned output record (i_owned_tensor) into a Tensor."""
+        self = cls.__new__(cls)
+        self.shape = tuple(owned.shape[d] for d in range(owned.rank))
+        self._values = array.array("f", bytes(ctypes.string_at(owned.data, owned.len * 4)) if owned.len else b"")
+        return self
+
+    @property
+    def data(self):
+        return self._values.tolist()
+
+    def _operand(self):
+        address, _ = self._values.buffer_info()
+        return _Operand(address, self.shape, nat.F32, None, self._values)
+
+    def __repr__(self):
+        return f"Tensor(shape={self.shape}, data={self.data})"
+
+
+# ---------------------------------------------------------------- Component
 class Component:
-    def __init__(self, src=None, _ptr=None):
-        if _ptr is None:
-            if src is None:
-                raise TypeError("Component needs source")
-            _ptr = core.i_parse(src.encode())
-        self._ptr = _check_ptr(_ptr)
+    """An 𝚒 component: an expression ``i("ik*jk~ijk | i:16 | ii'jk")`` or a combination of components."""
+
+    def __init__(self, src=None, *, _handle=None):
+        self._ptr = None
         self._program = None
+        if _handle is None:
+            if not isinstance(src, str):
+                raise TypeError("Component takes the source text of one expression")
+            _handle = core.i_parse(src.encode())
+        self._ptr = nat.check_ptr(_handle)
 
     def __del__(self, _core=core):  # bound at definition: module globals may be gone at interpreter shutdown
-        program, ptr = getattr(self, "_program", None), getattr(self, "_ptr", None)
-        if program:
-            _core.i_program_free(program)
-            self._program = None
-        if ptr:
-            _core.i_component_free(ptr)
-            self._ptr = None
+        if getattr(self, "_program", None):
+            _core.i_program_free(self._program)
+        if getattr(self, "_ptr", None):
+            _core.i_component_free(self._ptr)
+        self._program = self._ptr = None
 
-    def _bin(self, other, fn):
-        if not isinstance(other, Component):
+    @property
+    def handle(self):
+        """The ``i_component*`` behind this object (owned by it)."""
+        return self._ptr
+
+    # combinators: each returns a new component; the operands stay valid (the library clones them)
+    def _with(self, other, combine):
+        if isinstance(other, str):
             other = Component(other)
-        return Component(_ptr=_check_ptr(fn(self._ptr, other._ptr)))
+        if not isinstance(other, Component):
+            return NotImplemented
+        return Component(_handle=combine(self._ptr, other._ptr))
 
     def chain(self, other):
-        return self._bin(other, core.i_chain)
+        return self._with(other, core.i_chain)
 
     def compose(self, other):
-        return self._bin(other, core.i_compose)
+        return self._with(other, core.i_compose)
 
     def fanout(self, other):
-        return self._bin(other, core.i_fanout)
+        return self._with(other, core.i_fanout)
 
     def pair(self, other):
-        return self._bin(other, core.i_pair)
+        return self._with(other, core.i_pair)
 
     def swap(self):
-        return Component(_ptr=_check_ptr(core.i_swap(self._ptr)))
+        return Component(_handle=core.i_swap(self._ptr))
 
     __rshift__ = chain
     __lshift__ = compose
     __and__ = fanout
     __or__ = pair
-
-    def __invert__(self):
-        return self.swap()
+    __invert__ = swap
 
     def _compile(self):
-        if self._program is None:
-            self._program = _check_ptr(core.i_compile(self._ptr))
+        """The compiled program, built on first use and kept for the life of the component."""
+        if not self._program:
+            self._program = nat.check_ptr(core.i_compile(self._ptr))
         return self._program
 
     def _code(self):
-        s = _check_ptr(core.i_code(self._ptr))
+        """The backend's source for this component: the kernel plan and the generated HIP."""
+        text = nat.check_ptr(core.i_code(self._ptr))
         try:
-            return ctypes.cast(s, ctypes.c_char_p).value.decode()
+            return ctypes.string_at(text).decode()
         finally:
-            core.i_string_free(s)
+            core.i_string_free(text)
 
-    def output_shapes(self, *inputs):
-        program = self._compile()
-        if inputs and all(_is_device_tensor(x) for x in inputs):
-            views = [(_CTensor(None, _shape_array(tuple(x.shape))[1], len(x.shape)), None) for x in inputs]
-            input_arr = (_CTensor * len(views))(*(v[0] for v in views))
-        else:
-            input_arr, views = _inputs(inputs)
+    def _result_extents(self, program, operands):
         count = core.i_output_count(program)
         ranks = (_sz * max(count, 1))()
-        _check(core.i_output_ranks(program, ranks))
-        shape_bufs = [(_sz * max(ranks[i], 1))() for i in range(count)]
-        shape_ptrs = (ctypes.POINTER(_sz) * max(count, 1))(*(ctypes.cast(b, ctypes.POINTER(_sz)) for b in shape_bufs))
-        _check(core.i_output_shapes(program, input_arr, len(inputs), shape_ptrs))
-        return [tuple(buf[j] for j in range(ranks[i])) for i, buf in enumerate(shape_bufs)]
+        nat.check(core.i_output_ranks(program, ranks))
+        rows = [_extent_buffer([0] * ranks[o]) for o in range(count)]
+        table = (ctypes.POINTER(_sz) * max(count, 1))(*(ctypes.cast(r, ctypes.POINTER(_sz)) for r in rows))
+        # only the extents of the inputs are read here, so device operands are described without their data
+        described = [_Operand(0, op.extents, nat.F32, None, None) for op in operands]
+        records, keep = _pack(described, on_device=False)
+        nat.check(core.i_output_shapes(program, records, len(operands), table))
+        del keep
+        return [tuple(rows[o][d] for d in range(ranks[o])) for o in range(count)]
+
+    def output_shapes(self, *inputs):
+        return self._result_extents(self._compile(), [_operand(x, "input") for x in inputs])
 
     def exec(self, *inputs):
+        """Runs on host data; the library allocates the outputs, which come back as ``Tensor``s."""
         program = self._compile()
-        input_arr, keepalive = _inputs(inputs)
-        outputs = core.i_exec(program, input_arr, len(inputs))
-        if outputs.count == 0:
-            _check(-1)
-        owner = _OwnedOutputs(outputs)
-        tensors = [Tensor._from_owned(owner, i) for i in range(outputs.count)]
-        return tensors[0] if len(tensors) == 1 else tuple(tensors)
+        records, keep = _pack([_operand(x, "input") for x in inputs], on_device=False)
+        produced = core.i_exec(program, records, len(inputs))
+        del keep
+        if not produced.tensors:
+            raise RuntimeError(nat.last_error())
+        try:
+            results = [Tensor._take(produced.tensors[o]) for o in range(produced.count)]
+        finally:
+            core.i_outputs_free(produced)
+        return results[0] if len(results) == 1 else tuple(results)
 
     def exec_numpy(self, *inputs):
         import numpy as np
 
-        outs = [np.empty(shape, dtype=np.float32) for shape in self.output_shapes(*inputs)]
-        self.into(outs if len(outs) != 1 else outs[0], *inputs)
-        return outs[0] if len(outs) == 1 else tuple(outs)
+        operands = [_operand(x, "input") for x in inputs]
+        results = [np.empty(extents, dtype=np.float32) for extents in self._result_extents(self._compile(), operands)]
+        self._run(operands, [_operand(r, "output") for r in results])
+        return results[0] if len(results) == 1 else tuple(results)
 
     def exec_torch(self, *inputs, out_dtype=None):
-        """Host tensors: as the reference (CPU float32).  GPU tensors: runs on their device
-        and stream; outputs are float32 unless ``out_dtype`` says otherwise."""
+        """Host tensors: as the reference (CPU float32 results).  ROCm tensors: runs on their device and on the
+        current stream; results are float32 unless ``out_dtype`` says bfloat16."""
         import torch
 
-        shapes = self.output_shapes(*inputs)
-        if inputs and all(_is_device_tensor(x) for x in inputs):
-            outs = [torch.empty(shape, dtype=out_dtype or torch.float32, device=inputs[0].device) for shape in shapes]
+        operands = [_operand(x, "input") for x in inputs]
+        device = _placement(operands, "inputs")
+        extents = self._result_extents(self._compile(), operands)
+        if device is None:
+            results = [torch.empty(e, dtype=torch.float32) for e in extents]
         else:
-            outs = [torch.empty(shape, dtype=torch.float32, device="cpu") for shape in shapes]
-        self.into(outs if len(outs) != 1 else outs[0], *inputs)
-        return outs[0] if len(outs) == 1 else tuple(outs)
+            results = [torch.empty(e, dtype=out_dtype or torch.float32, device=device) for e in extents]
+        self._run(operands, [_operand(r, "output") for r in results])
+        return results[0] if len(results) == 1 else tuple(results)
 
     def into(self, outputs, *inputs):
+        """Runs into caller-provided outputs (one object or a sequence of them) and returns them."""
+        targets = list(outputs) if isinstance(outputs, (tuple, list)) else [outputs]
+        self._run([_operand(x, "input") for x in inputs], [_operand(t, "output") for t in targets])
+        return targets[0] if len(targets) == 1 else tuple(targets)
+
+    def _run(self, operands, targets):
         program = self._compile()
-        if not isinstance(outputs, (tuple, list)):
-            outputs = (outputs,)
-        if inputs and all(_is_device_tensor(x) for x in inputs):
+        device = _placement(operands + targets, "inputs and outputs")
+        in_records, keep_in = _pack(operands, device is not None)
+        out_records, keep_out = _pack(targets, device is not None)
+        if device is None:
+            nat.check(core.i_exec_into(program, in_records, len(operands), out_records, len(targets)))
+        else:
             import torch
 
-            in_arr, keep_in = _device_views(inputs, "inputs")
-            out_arr, keep_out = _device_views(outputs, "outputs")
-            with torch.cuda.device(inputs[0].device):
+            with torch.cuda.device(device):
                 stream = torch.cuda.current_stream().cuda_stream
-                _check(core.i_exec_into_device(program, in_arr, len(inputs), out_arr, len(outputs), stream))
-        else:
-            input_arr, keepalive = _inputs(inputs)
-            out_views = [_output(out) for out in outputs]
-            output_arr = (_CTensor * max(len(out_views), 1))(*(v[0] for v in out_views))
-            _check(core.i_exec_into(program, input_arr, len(inputs), output_arr, len(out_views)))
-        return outputs[0] if len(outputs) == 1 else tuple(outputs)
+                nat.check(core.i_exec_into_device(program, in_records, len(operands), out_records, len(targets), stream))
+        del keep_in, keep_out
 
 
-I = Component(_ptr=core.i_identity())
+I = Component(_handle=core.i_identity())
 
 
 def i(src):

@@ -15,8 +15,8 @@ core = nat.core
 
 
 def test_null_handles_report_reference_errors():
-    assert not core.i_chain(None, I._ptr) and nat.last_error() == "null left component"
-    assert not core.i_chain(I._ptr, None) and nat.last_error() == "null right component"
+    assert not core.i_chain(None, I.handle) and nat.last_error() == "null left component"
+    assert not core.i_chain(I.handle, None) and nat.last_error() == "null right component"
     assert not core.i_swap(None) and nat.last_error() == "null component"
     assert not core.i_code(None) and nat.last_error() == "null component"
     assert not core.i_compile(None) and nat.last_error() == "null component"
@@ -35,7 +35,7 @@ def test_null_handles_report_reference_errors():
 def test_error_is_thread_local_and_sticky():
     assert not core.i_swap(None)
     assert nat.last_error() == "null component"
-    assert i("ij~ij")._ptr  # success does not clear the slot
+    assert i("ij~ij").handle  # success does not clear the slot
     assert nat.last_error() == "null component"
     seen = {}
 
@@ -82,7 +82,7 @@ def test_exec_into_checks_output_count_before_touching_the_device():
     prog = i("+ij~i")
     program = prog._compile()
     x = np.zeros((4, 9), np.float32)
-    arr, keep = ilang._inputs([x])
+    arr, keep = ilang._pack([ilang._operand(x, "input")], on_device=False)
     assert core.i_exec_into(program, arr, 1, None, 0) == -1
     assert nat.last_error() == "wrong output count"
     assert core.i_exec_into(program, None, 1, None, 1) == -1
@@ -115,3 +115,29 @@ def test_generated_source_builds_for_gfx950_without_a_gpu():
     # i_compile runs hipcc for kernels that have no hand-written form
     prog = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")
     assert prog._compile()
+
+
+def test_tensor_from_python_data():
+    from i_amd import Tensor
+
+    t = Tensor([[1, 2, 3], [4, 5, 6]])
+    assert t.shape == (2, 3) and t.data == [1.0, 2.0, 3.0, 4.0, 5.0, 6.0]
+    assert Tensor(2.5).shape == () and Tensor(2.5).data == [2.5]
+    assert Tensor([]).shape == (0,) and Tensor([[], []]).shape == (2, 0)
+    assert Tensor([1, 2, 3, 4], shape=(2, 2)).shape == (2, 2)
+    assert "shape=(2, 3)" in repr(t)
+    with pytest.raises(ValueError):
+        Tensor([[1, 2], [3]])
+    with pytest.raises(ValueError):
+        Tensor([1, 2, 3], shape=(2, 2))
+    with pytest.raises(TypeError):
+        Tensor([["a"]])
+
+
+def test_operands_must_share_a_place_and_outputs_are_written_in_place():
+    prog = i("+ij~i")
+    x = np.ones((4, 9), np.float32)
+    with pytest.raises(TypeError):
+        prog.into(np.zeros((4,), np.float64), x)           # an output is never converted
+    with pytest.raises(TypeError):
+        prog.into([1.0, 2.0, 3.0, 4.0], x)                 # a list cannot be written in place

@@ -25,11 +25,11 @@ ROOT = Path(__file__).resolve().parents[1]
 
 
 def c_of(component):
-    return oracle.emit_c(component._ptr)
+    return oracle.emit_c(component.handle)
 
 
 def run_c(component, *inputs):
-    return oracle.compile_component(component._ptr).run(*inputs)
+    return oracle.compile_component(component.handle).run(*inputs)
 
 
 def rnd(shape, seed):
@@ -88,7 +88,7 @@ def test_flash_attention_emission_structure():
     "+ijk~ij|i:2,k:4|", "  ij + i ~ ij |  | i j 1 ", "ij/i~ij|i:2,j:2|iji'j'01", "ij~ij",
 ])
 def test_parser_accepts(src):
-    assert i(src)._ptr
+    assert i(src).handle
 
 
 @pytest.mark.parametrize("src,offset,message", [

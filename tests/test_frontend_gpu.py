@@ -125,7 +125,7 @@ def test_reference_demo_flash_and_naive_attention(torch):
 def test_config1_demo_attention_f32_vs_emitted_c(torch, split):
     q, k, v = (np.random.default_rng(s).uniform(-1, 1, (512, 64)).astype(np.float32) for s in (1, 2, 3))
     comp = flash(split)
-    ref = oracle.compile_component(comp._ptr).run(q, k, v)  # the C the reference backend would emit for these strings
+    ref = oracle.compile_component(comp.handle).run(q, k, v)  # the C the reference backend would emit for these strings
     close(comp.exec_numpy(q, k, v), ref, RTOL_F32)
     close(comp.exec_torch(*(torch.from_numpy(a) for a in (q, k, v))).numpy(), ref, RTOL_F32)
 
@@ -161,7 +161,7 @@ def test_generated_and_hand_written_forms_agree(torch):
 def test_config2_row_softmax_small_vs_emitted_c(torch, comp_fn):
     x = rnd((50, 70), 1)
     comp = comp_fn()
-    close(comp.exec_numpy(x), oracle.compile_component(comp._ptr).run(x), RTOL_F32)
+    close(comp.exec_numpy(x), oracle.compile_component(comp.handle).run(x), RTOL_F32)
 
 
 def test_config2_row_softmax_full_size_device(torch):
@@ -190,7 +190,7 @@ def test_config3_mm_t_bf16_device(torch):
 def test_mm_t_f32_small_vs_emitted_c(torch, k):
     a, b = rnd((100, k), 1), rnd((70, k), 2)
     comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
-    close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
+    close(comp.exec_numpy(a, b), oracle.compile_component(comp.handle).run(a, b), RTOL_F32)
 
 
 def test_config3_mm_t_through_the_host_f32_abi(torch):
@@ -216,7 +216,7 @@ def test_matmul_nn_f32_vs_emitted_c(torch, m, k, n):
     a, b = rnd((m, k), 1), rnd((k, n), 2)
     comp = i(MATMUL[0]) >> i(MATMUL[1])
     assert "row-major right operand" in comp._code()
-    close(comp.exec_numpy(a, b), oracle.compile_component(comp._ptr).run(a, b), RTOL_F32)
+    close(comp.exec_numpy(a, b), oracle.compile_component(comp.handle).run(a, b), RTOL_F32)
 
 
 @pytest.mark.parametrize("m,k,n", [(300, 256, 200), (128, 64, 128), (77, 1024, 513)])
@@ -238,7 +238,7 @@ def test_matmul_nn_batched_and_the_demo_mm(torch):
     close(batched.exec_numpy(a, b), np.einsum("bhik,bhkj->bhij", a.astype(np.float64), b.astype(np.float64)), RTOL_F32)
     p_, v_ = rnd((48, 96), 3), rnd((96, 64), 4)
     mm = i("ij*jk~ikj | i:16,j:16 | jii'kj'") >> i("+ikj~ik | i:16,j:16 | jii'kj'0")
-    close(mm.exec_numpy(p_, v_), oracle.compile_component(mm._ptr).run(p_, v_), RTOL_F32)
+    close(mm.exec_numpy(p_, v_), oracle.compile_component(mm.handle).run(p_, v_), RTOL_F32)
 
 
 @pytest.mark.parametrize("rows,cols", [(37, 100), (64, 4096), (5, 9000), (300, 33)])
@@ -255,7 +255,7 @@ def test_row_max_shift_and_row_normalize_kernels(torch, rows, cols):
     ex = i("^ij~ij|i:16,j:16|jii'j'")
     assert "exp x" in ex._code()
     small = np.clip(x, -20.0, 5.0)
-    close(ex.exec_numpy(small), oracle.compile_component(ex._ptr).run(small), RTOL_F32)
+    close(ex.exec_numpy(small), oracle.compile_component(ex.handle).run(small), RTOL_F32)
     # the three-kernel naive softmax of the reference's demo runs on them
     close(softmax_naive().exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
 
