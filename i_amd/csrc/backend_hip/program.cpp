@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <set>
 #include <sstream>
 
@@ -364,6 +365,40 @@ const Step* find_dispatch(const ExecPlan& plan, size_t k) {
   return nullptr;
 }
 
+// Which dimensions of which program inputs every index symbol of every expression stands for.  An operand of a
+// node is a program input or another node's result; a result dimension stands for whatever its output symbol
+// stands for, so the groups carry through chains of expressions.
+std::vector<std::vector<std::pair<size_t, size_t>>> tied_extents(const Graph<Node>& graph) {
+  using Dims = std::set<std::pair<size_t, size_t>>;
+  std::vector<std::vector<Dims>> result_dims(graph.nodes.size());
+  std::vector<char> state(graph.nodes.size(), 0);  // 0 not visited, 1 in progress, 2 done
+  std::set<std::vector<std::pair<size_t, size_t>>> groups;
+  std::function<void(size_t)> visit = [&](size_t n) {
+    if (state[n] != 0) return;  // done, or a cycle (which lowering has rejected)
+    state[n] = 1;
+    const GNode<Node>& g = graph.nodes[n];
+    const Node& node = g.inner;
+    std::vector<Dims> of_symbol(node.rank);
+    for (size_t o = 0; o < node.inputs.size() && o < g.inputs.size(); ++o) {
+      const Source& src = g.inputs[o];
+      if (!src.is_input && src.id < graph.nodes.size()) visit(src.id);
+      for (size_t pos = 0; pos < node.inputs[o].size(); ++pos) {
+        const size_t symbol = node.inputs[o][pos];
+        if (symbol >= of_symbol.size()) continue;
+        if (src.is_input) of_symbol[symbol].insert({src.id, pos});
+        else if (src.id < graph.nodes.size() && pos < result_dims[src.id].size())
+          of_symbol[symbol].insert(result_dims[src.id][pos].begin(), result_dims[src.id][pos].end());
+      }
+    }
+    for (const Dims& d : of_symbol)
+      if (d.size() > 1) groups.insert(std::vector<std::pair<size_t, size_t>>(d.begin(), d.end()));
+    for (size_t symbol : node.output) result_dims[n].push_back(symbol < of_symbol.size() ? of_symbol[symbol] : Dims{});
+    state[n] = 2;
+  };
+  for (size_t n = 0; n < graph.nodes.size(); ++n) visit(n);
+  return {groups.begin(), groups.end()};
+}
+
 }  // namespace
 
 Program::~Program() {
@@ -375,6 +410,7 @@ std::string compile_program(const Component& component, Program** out) {
   p->low = lower_component(component);
   p->module = lower_exec_plan_to_module(p->low.plan);
   p->recognized = recognize_kernels(p->low);
+  p->same_extent = tied_extents(p->low.graph);
   if (p->recognized.size() != p->low.plan.kernels.size()) lower_error("kernel recognition lost track of the kernel list");
   std::vector<bool> emit(p->low.plan.kernels.size(), true);
   p->generic = emit_generic_hip(p->low.plan, p->module, emit);
@@ -460,6 +496,17 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
       return "input " + std::to_string(i) + " has rank " + std::to_string(inputs[i].shape.size()) + ", program expects rank " +
              std::to_string(plan.inputs[i].shape.size());
     if (!inputs[i].data && product(inputs[i].shape) != 0) return "input " + std::to_string(i) + " has no data";
+  }
+  // operands that share an index must agree on its extent: a kernel takes each loop bound from one of them
+  for (const auto& group : p.same_extent) {
+    const auto& first = group.front();
+    for (const auto& other : group)
+      if (inputs.at(other.first).shape.at(other.second) != inputs.at(first.first).shape.at(first.second))
+        return "inputs " + std::to_string(first.first) + " and " + std::to_string(other.first) +
+               " disagree on an index they share: dimension " + std::to_string(first.second) + " of input " +
+               std::to_string(first.first) + " is " + std::to_string(inputs[first.first].shape[first.second]) +
+               ", dimension " + std::to_string(other.second) + " of input " + std::to_string(other.first) + " is " +
+               std::to_string(inputs[other.first].shape[other.second]);
   }
   if (outputs.size() != plan.count) return "wrong output count";
   Run run{p, plan, inputs, outputs, stream, {}, std::vector<void*>(plan.intermediates.size(), nullptr), {}, {}};

@@ -30,6 +30,9 @@ struct Program {
   ic::Lowered low;
   ic::Module module;
   std::vector<Recognized> recognized;  // per plan kernel
+  // Groups of (input, dimension) pairs that one index symbol ties together, directly or through intermediate
+  // results: their extents must agree, or some kernel would index an operand out of bounds.
+  std::vector<std::vector<std::pair<size_t, size_t>>> same_extent;
   GenericModule generic;               // source for every kernel (hand-written ones keep a generated twin)
   std::vector<char> image;             // built lazily unless some kernel can only run generated
   bool image_built = false;

@@ -51,6 +51,34 @@ def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
 
 
+def test_operands_that_disagree_on_a_shared_index_are_refused_before_any_launch(shim_lib):
+    """A kernel takes each loop bound from one operand; another operand with a smaller extent for the same index
+    would be read out of bounds (a GPU memory fault on the device, a guard-page hit here)."""
+    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"), ILANG_HIP_GENERATED_ONLY="1",
+               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
+    code = """
+import numpy as np
+from i_amd import Component as i
+ones = lambda *s: np.ones(s, np.float32)
+cases = [
+    (i('ij+ij~ij'), [ones(64, 64), ones(2, 2)], 'inputs 0 and 1 disagree'),
+    (i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0"), [ones(8, 4), ones(8, 5)], 'inputs 0 and 1 disagree'),
+    (i('ij+ij~ij') >> i('ij*ij~ij'), [ones(8, 4), ones(8, 4), ones(8, 5)], 'disagree'),   # tied through an intermediate result
+    (i('ik*kj~ijk') >> i('+ijk~ij'), [ones(8, 4), ones(5, 3)], 'dimension 1 of input 0 is 4, dimension 0 of input 1 is 5'),
+]
+for comp, operands, text in cases:
+    try:
+        comp.exec_numpy(*operands)
+        print('NOT REFUSED')
+    except RuntimeError as e:
+        print('ok' if text in str(e) else 'WRONG TEXT: ' + str(e))
+print(i('ij+ij~ij').exec_numpy(ones(3, 2), ones(3, 2)).sum())
+"""
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.split() == ["ok"] * 4 + ["12.0"], r.stdout
+
+
 def test_phase_plan_is_reported(shim_lib):
     env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_NO_TORCH="1")
     code = ("from i_amd import Component as i, I\n"
