@@ -34,10 +34,20 @@ def build_kernels():
     _run([ROCM / "bin" / "hipcc", "--genco", *HIPCC_FLAGS, CSRC / "kernels" / "kernels.hip", "-o", HSACO])
 
 
+def build_static_scratch():
+    """The one host + device source: the fixed device workspace (a file-scope __device__ array) and its lookup."""
+    obj = CSRC / "runtime" / "static_scratch.o"
+    _run([ROCM / "bin" / "hipcc", "-c", "-fPIC", "-O2", "-std=c++17", "--offload-arch=gfx950",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          CSRC / "runtime" / "static_scratch.hip", "-o", obj])
+    return obj
+
+
 def build_host():
+    scratch_obj = build_static_scratch()
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-fvisibility=hidden", "-Wno-unused-function",
           "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{PKG.parent / 'include'}",
-          *host_sources(), "-o", LIB,
+          *host_sources(), scratch_obj, "-o", LIB,
           f"-L{ROCM / 'lib'}", "-lamdhip64", f"-Wl,-rpath,{ROCM / 'lib'}", "-ldl", "-lpthread"])
 
 

@@ -1,6 +1,7 @@
 #include "program.h"
 
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
@@ -40,6 +41,7 @@ struct Run {
   std::vector<void*> intermediates;          // device pointers (f32), null when not needed
   std::map<size_t, void*> input_f32;         // bf16 inputs widened for f32 kernels
   std::map<size_t, void*> output_f32;        // f32 staging for bf16 outputs
+  Workspace* workspace = nullptr;            // when set, temporaries are carved out of it and nothing is allocated
 
   size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
   size_t extent(const Extent<size_t>& e) const {
@@ -77,6 +79,14 @@ struct Run {
 
   ihip::Err alloc(void** ptr, size_t bytes) {
     if (bytes == 0) bytes = 4;
+    if (workspace) {
+      // bump allocation in 256-byte steps; the sizing pass has no limit and only adds up
+      const size_t step = (bytes + 255) / 256 * 256;
+      if (workspace->limit && step > workspace->limit - workspace->used) return "workspace exhausted";
+      *ptr = static_cast<char*>(workspace->base) + workspace->used;
+      workspace->used += step;
+      return {};
+    }
     if (ihip::Err e = ihip::check(hipMallocAsync(ptr, bytes, stream), "hipMallocAsync"); !e.empty()) return e;
     temps.push_back(*ptr);
     return {};
@@ -487,7 +497,7 @@ std::string output_shapes(const Program& p, const std::vector<std::vector<size_t
 }
 
 std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
-                    hipStream_t stream) {
+                    hipStream_t stream, Workspace* workspace) {
   const ExecPlan& plan = p.low.plan;
   if (inputs.size() < plan.inputs.size())
     return "program takes " + std::to_string(plan.inputs.size()) + " inputs, got " + std::to_string(inputs.size());
@@ -509,7 +519,7 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
                std::to_string(inputs[other.first].shape[other.second]);
   }
   if (outputs.size() != plan.count) return "wrong output count";
-  Run run{p, plan, inputs, outputs, stream, {}, std::vector<void*>(plan.intermediates.size(), nullptr), {}, {}};
+  Run run{p, plan, inputs, outputs, stream, {}, std::vector<void*>(plan.intermediates.size(), nullptr), {}, {}, workspace};
   for (size_t o = 0; o < outputs.size(); ++o) {
     const auto want = run.shape_of({BufferRef::Output, o});
     if (!outputs[o].shape.empty() && outputs[o].shape != want) return "output " + std::to_string(o) + " has the wrong shape";
@@ -554,6 +564,16 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
     if (ihip::Err e = ihip::launch_convert(tmp, outputs[o].data, ihip::F32, ihip::BF16, n, stream); !e.empty()) return finish(e);
   }
   return finish({});
+}
+
+std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
+                            size_t* bytes) {
+  ihip::DryRun nothing_is_launched;
+  Workspace sizing;
+  sizing.base = reinterpret_cast<void*>(uintptr_t(256));  // never dereferenced: only has to be non-null
+  const std::string err = execute(p, inputs, outputs, nullptr, &sizing);
+  *bytes = sizing.used;
+  return err;
 }
 
 }  // namespace ihipc

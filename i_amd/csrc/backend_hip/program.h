@@ -57,10 +57,24 @@ std::string output_shapes(const Program& p, const std::vector<std::vector<size_t
 size_t input_count(const Program& p);
 size_t input_rank(const Program& p, size_t input);
 
+// Caller-provided device memory for a program's temporaries (intermediates of multi-kernel plans, dtype
+// staging, transposed operands, per-work-item slices of generated kernels).  `used` counts what one
+// execution took; limit == 0 means "only add up" (a sizing pass).
+struct Workspace {
+  void* base = nullptr;
+  size_t limit = 0;
+  size_t used = 0;
+};
+
 // Enqueue the program on `stream`.  All tensors live in device memory.
 // Temporary buffers are stream-ordered allocations, so the call does not wait
-// for the GPU.  Returns "" on success.
+// for the GPU; with a workspace they are carved out of it instead and the
+// call allocates and frees no device memory.  Returns "" on success.
 std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
-                    hipStream_t stream);
+                    hipStream_t stream, Workspace* workspace = nullptr);
+
+// What execute() with a workspace would take from it for these operands, in bytes.  Launches nothing.
+std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
+                            size_t* bytes);
 
 }  // namespace ihipc

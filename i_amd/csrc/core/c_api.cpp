@@ -11,6 +11,7 @@
 #include "../../../include/i_hip.h"
 #include "../backend_hip/program.h"
 #include "../runtime/hip_rt.h"
+#include "../runtime/static_scratch.h"
 #include "error.h"
 #include "handles.h"
 
@@ -126,6 +127,31 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
   if (err.empty()) err = sync_err;
   cleanup();
   return err;
+}
+
+// Argument checks shared by the device entry points; fills `in` / `out` and returns true, or sets the error.
+bool device_call_ok(const i_program* program, const i_device_tensor* inputs, size_t input_count,
+                    const i_device_tensor* outputs, size_t output_count, std::vector<ihipc::DeviceTensor>* in,
+                    std::vector<ihipc::DeviceTensor>* out) {
+  if (!program) return fail("null program"), false;
+  if (input_count > 0 && !inputs) return fail("null inputs"), false;
+  if (output_count != ihipc::output_count(*program->inner)) return fail("wrong output count"), false;
+  if (output_count > 0 && !outputs) return fail("null outputs"), false;
+  auto convert = [](const i_device_tensor* t, size_t n, std::vector<ihipc::DeviceTensor>* dst) -> bool {
+    for (size_t i = 0; i < n; ++i) {
+      if (t[i].dtype != I_DTYPE_F32 && t[i].dtype != I_DTYPE_BF16) return false;
+      ihipc::DeviceTensor d;
+      d.data = t[i].data;
+      d.dtype = t[i].dtype == I_DTYPE_BF16 ? ihipc::DType::BF16 : ihipc::DType::F32;
+      if (t[i].rank > 0 && !t[i].shape) return false;
+      d.shape.assign(t[i].shape, t[i].shape + t[i].rank);
+      dst->push_back(std::move(d));
+    }
+    return true;
+  };
+  if (!convert(inputs, input_count, in) || !convert(outputs, output_count, out))
+    return fail("bad device tensor (dtype or shape)"), false;
+  return true;
 }
 
 }  // namespace
@@ -301,26 +327,32 @@ i_outputs i_exec(const i_program* program, const i_tensor* inputs, size_t input_
 
 int i_exec_into_device(const i_program* program, const i_device_tensor* inputs, size_t input_count,
                        const i_device_tensor* outputs, size_t output_count, void* stream) {
-  if (!program) return fail("null program");
-  if (input_count > 0 && !inputs) return fail("null inputs");
-  if (output_count != ihipc::output_count(*program->inner)) return fail("wrong output count");
-  if (output_count > 0 && !outputs) return fail("null outputs");
-  auto convert = [](const i_device_tensor* t, size_t n, std::vector<ihipc::DeviceTensor>* out) -> bool {
-    for (size_t i = 0; i < n; ++i) {
-      if (t[i].dtype != I_DTYPE_F32 && t[i].dtype != I_DTYPE_BF16) return false;
-      ihipc::DeviceTensor d;
-      d.data = t[i].data;
-      d.dtype = t[i].dtype == I_DTYPE_BF16 ? ihipc::DType::BF16 : ihipc::DType::F32;
-      if (t[i].rank > 0 && !t[i].shape) return false;
-      d.shape.assign(t[i].shape, t[i].shape + t[i].rank);
-      out->push_back(std::move(d));
-    }
-    return true;
-  };
   std::vector<ihipc::DeviceTensor> in, out;
-  if (!convert(inputs, input_count, &in) || !convert(outputs, output_count, &out)) return fail("bad device tensor (dtype or shape)");
+  if (!device_call_ok(program, inputs, input_count, outputs, output_count, &in, &out)) return -1;
   try {
     const std::string err = ihipc::execute(*program->inner, in, out, static_cast<hipStream_t>(stream));
+    return err.empty() ? 0 : fail(err);
+  } catch (const std::exception& e) {
+    return fail(e.what());
+  }
+}
+
+int i_exec_into_device_noalloc(const i_program* program, const i_device_tensor* inputs, size_t input_count,
+                               const i_device_tensor* outputs, size_t output_count, void* stream) {
+  std::vector<ihipc::DeviceTensor> in, out;
+  if (!device_call_ok(program, inputs, input_count, outputs, output_count, &in, &out)) return -1;
+  try {
+    // set-up, once per device: the address of this device's copy of the static workspace
+    void* base = nullptr;
+    if (ihip::Err e = ihip::static_scratch(&base); !e.empty()) return fail(e);
+    // size the temporaries first, so that a program that does not fit is refused before anything is enqueued
+    size_t need = 0;
+    if (std::string e = ihipc::workspace_bytes(*program->inner, in, out, &need); !e.empty()) return fail(e);
+    if (need > ihip::kStaticScratchBytes)
+      return fail("program needs " + std::to_string(need) + " bytes of temporaries for these operands, the static workspace holds " +
+                  std::to_string(ihip::kStaticScratchBytes) + " (use i_exec_into_device)");
+    ihipc::Workspace ws{base, ihip::kStaticScratchBytes, 0};
+    const std::string err = ihipc::execute(*program->inner, in, out, static_cast<hipStream_t>(stream), &ws);
     return err.empty() ? 0 : fail(err);
   } catch (const std::exception& e) {
     return fail(e.what());

@@ -26,6 +26,7 @@ struct DeviceModule {
   std::map<std::string, hipFunction_t> fns;
 };
 
+thread_local int g_dry_run = 0;
 std::mutex g_mu;
 std::map<int, DeviceModule> g_builtin;  // keyed by device ordinal
 std::vector<char> g_image;
@@ -91,12 +92,15 @@ void unload_module(hipModule_t mod) {
 
 Err launch(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, const void* params,
            size_t params_size, hipStream_t stream) {
-  if (gx == 0 || gy == 0 || gz == 0) return {};
+  if (gx == 0 || gy == 0 || gz == 0 || g_dry_run) return {};
   size_t size = params_size;
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(params), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};
   return check(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, 0, stream, nullptr, config), "hipModuleLaunchKernel");
 }
+
+DryRun::DryRun() { ++g_dry_run; }
+DryRun::~DryRun() { --g_dry_run; }
 
 Err dev_alloc(void** p, size_t bytes) {
   *p = nullptr;

@@ -28,6 +28,15 @@ void unload_module(hipModule_t mod);
 Err launch(hipFunction_t fn, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned block_x,
            const void* params, size_t params_size, hipStream_t stream);
 
+// While one of these lives on a thread, launch() on that thread checks nothing in and enqueues nothing: the
+// executor walks a program once this way to add up the temporaries it would need.
+struct DryRun {
+  DryRun();
+  ~DryRun();
+  DryRun(const DryRun&) = delete;
+  DryRun& operator=(const DryRun&) = delete;
+};
+
 Err dev_alloc(void** p, size_t bytes);
 void dev_free(void* p);
 Err h2d(void* dst, const void* src, size_t bytes, hipStream_t stream);

@@ -56,6 +56,7 @@ _PROTOTYPES = {
     "i_exec_into": ([_vp, ctypes.POINTER(_CTensor), _sz, ctypes.POINTER(_CTensor), _sz], ctypes.c_int),
     "i_exec": ([_vp, ctypes.POINTER(_CTensor), _sz], _COutputs),
     "i_exec_into_device": ([_vp, ctypes.POINTER(_CDeviceTensor), _sz, ctypes.POINTER(_CDeviceTensor), _sz, _vp], ctypes.c_int),
+    "i_exec_into_device_noalloc": ([_vp, ctypes.POINTER(_CDeviceTensor), _sz, ctypes.POINTER(_CDeviceTensor), _sz, _vp], ctypes.c_int),
     "i_component_free": ([_vp], None),
     "i_program_free": ([_vp], None),
     "i_outputs_free": ([_COutputs], None),
@@ -330,12 +331,13 @@ class Component:
 
         operands = [_operand(x, "input") for x in inputs]
         results = [np.empty(extents, dtype=np.float32) for extents in self._result_extents(self._compile(), operands)]
-        self._run(operands, [_operand(r, "output") for r in results])
+        self._run(operands, [_operand(r, "output") for r in results], False)
         return results[0] if len(results) == 1 else tuple(results)
 
-    def exec_torch(self, *inputs, out_dtype=None):
+    def exec_torch(self, *inputs, out_dtype=None, static_workspace=False):
         """Host tensors: as the reference (CPU float32 results).  ROCm tensors: runs on their device and on the
-        current stream; results are float32 unless ``out_dtype`` says bfloat16."""
+        current stream; results are float32 unless ``out_dtype`` says bfloat16.  ``static_workspace`` (ROCm
+        tensors only) runs through ``i_exec_into_device_noalloc``: no device memory is allocated."""
         import torch
 
         operands = [_operand(x, "input") for x in inputs]
@@ -345,28 +347,31 @@ class Component:
             results = [torch.empty(e, dtype=torch.float32) for e in extents]
         else:
             results = [torch.empty(e, dtype=out_dtype or torch.float32, device=device) for e in extents]
-        self._run(operands, [_operand(r, "output") for r in results])
+        self._run(operands, [_operand(r, "output") for r in results], static_workspace)
         return results[0] if len(results) == 1 else tuple(results)
 
-    def into(self, outputs, *inputs):
+    def into(self, outputs, *inputs, static_workspace=False):
         """Runs into caller-provided outputs (one object or a sequence of them) and returns them."""
         targets = list(outputs) if isinstance(outputs, (tuple, list)) else [outputs]
-        self._run([_operand(x, "input") for x in inputs], [_operand(t, "output") for t in targets])
+        self._run([_operand(x, "input") for x in inputs], [_operand(t, "output") for t in targets], static_workspace)
         return targets[0] if len(targets) == 1 else tuple(targets)
 
-    def _run(self, operands, targets):
+    def _run(self, operands, targets, static_workspace):
         program = self._compile()
         device = _placement(operands + targets, "inputs and outputs")
         in_records, keep_in = _pack(operands, device is not None)
         out_records, keep_out = _pack(targets, device is not None)
         if device is None:
+            if static_workspace:
+                raise TypeError("static_workspace applies to GPU tensors only")
             nat.check(core.i_exec_into(program, in_records, len(operands), out_records, len(targets)))
         else:
             import torch
 
+            entry = core.i_exec_into_device_noalloc if static_workspace else core.i_exec_into_device
             with torch.cuda.device(device):
                 stream = torch.cuda.current_stream().cuda_stream
-                nat.check(core.i_exec_into_device(program, in_records, len(operands), out_records, len(targets), stream))
+                nat.check(entry(program, in_records, len(operands), out_records, len(targets), stream))
         del keep_in, keep_out
 
 

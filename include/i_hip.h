@@ -53,6 +53,26 @@ int i_exec_into_device(const i_program* program,
                        void* stream);
 
 /*
+ * i_exec_into_device for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose generated
+ * `exec` mallocs its scratch on every call, ilang-python/annotated-flashattn.c:318-386).  Same arguments,
+ * same kernels and same results as i_exec_into_device, but the program's temporaries (intermediates of
+ * multi-kernel plans, f32 staging of bf16 operands, transposed operands, per-work-item slices of generated
+ * kernels) are carved out of one fixed array of I_HIP_STATIC_WORKSPACE_BYTES that the library holds in the
+ * memory of every GPU it runs on until the process ends; the call allocates and frees no device memory.
+ * Operands whose temporaries add up to more are refused (-1, i_error says how much was needed) before
+ * anything is enqueued.  Nothing in the array has to start at zero, and nothing is kept from call to call.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU, from different
+ * streams or threads, race; serialise them (one stream, or events).  The first call of a program on a
+ * device loads its code objects; make that call before capturing a graph.
+ */
+#define I_HIP_STATIC_WORKSPACE_BYTES ((size_t)64 << 20)
+int i_exec_into_device_noalloc(const i_program* program,
+                               const i_device_tensor* inputs, size_t input_count,
+                               const i_device_tensor* outputs, size_t output_count,
+                               void* stream);
+
+/*
  * FlashAttention forward,  o = softmax(scale * q k^T) v  per (batch*head):
  * the fused kernel for  mm_t >> [scale] >> row_max_shift >> exp >> row_normalize >> mm
  * (reference emission of the same component: ilang-python/annotated-flashattn.c:52-310,

@@ -18,6 +18,8 @@
 #include <mutex>
 #include <string>
 
+#include "../../i_amd/csrc/runtime/static_scratch.h"
+
 namespace {
 std::mutex g_mu;
 struct Block {
@@ -59,6 +61,17 @@ struct BigArgs {
   unsigned char bytes[4096];
 };
 }  // namespace
+
+// The product takes its fixed workspace from a file-scope array in device memory (static_scratch.hip, built by
+// hipcc); here it is one guarded host block of the same size, so a temporary carved past its end faults.
+namespace ihip {
+Err static_scratch(void** ptr) {
+  static void* block = nullptr;
+  if (!block && guarded_alloc(&block, kStaticScratchBytes) != hipSuccess) return "shim: no memory for the workspace";
+  *ptr = block;
+  return {};
+}
+}  // namespace ihip
 
 extern "C" {
 hipError_t hipGetDevice(int* dev) {

@@ -141,3 +141,13 @@ def test_operands_must_share_a_place_and_outputs_are_written_in_place():
         prog.into(np.zeros((4,), np.float64), x)           # an output is never converted
     with pytest.raises(TypeError):
         prog.into([1.0, 2.0, 3.0, 4.0], x)                 # a list cannot be written in place
+    with pytest.raises(TypeError):
+        prog.into(np.zeros((4,), np.float32), x, static_workspace=True)  # host operands have no workspace
+
+
+def test_noalloc_entry_checks_arguments_before_touching_the_device():
+    comp = i("+ij~i")  # owns the program
+    program = comp._compile()
+    assert core.i_exec_into_device_noalloc(None, None, 0, None, 0, None) == -1 and nat.last_error() == "null program"
+    assert core.i_exec_into_device_noalloc(program, None, 1, None, 1, None) == -1 and nat.last_error() == "null inputs"
+    assert core.i_exec_into_device_noalloc(program, None, 0, None, 0, None) == -1 and nat.last_error() == "wrong output count"

@@ -51,6 +51,13 @@ def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
 
 
+def test_fixed_workspace_entry_matches_on_the_cpu(shim_lib):
+    """i_exec_into_device_noalloc: every temporary comes out of one fixed block (here a guarded host block of the
+    product's size), in both launch modes; results must equal the emitted C as through the allocating entry."""
+    run_cases(shim_lib, {"ILANG_SHIM_NOALLOC": "1"})
+    run_cases(shim_lib, {"ILANG_SHIM_NOALLOC": "1", "ILANG_HIP_PHASES": "1"})
+
+
 def test_operands_that_disagree_on_a_shared_index_are_refused_before_any_launch(shim_lib):
     """A kernel takes each loop bound from one operand; another operand with a smaller extent for the same index
     would be read out of bounds (a GPU memory fault on the device, a guard-page hit here)."""

@@ -1,0 +1,100 @@
+"""i_exec_into_device_noalloc (the entry point that allocates no device memory) against i_exec_into_device, through
+the C ABI, on programs whose temporaries are real: the two [rows, cols] intermediates of the naive three-kernel
+softmax, the f32 staging of bf16 operands and outputs, the transposed right operand of a ragged f32 product, and
+the [i, j, k] intermediate of an unfused product run on generated kernels.  Both entries launch the same kernels,
+so the results are compared bit for bit; each case runs twice in a row, the second time on a smaller input, because
+every call reuses the same fixed array and finds the previous call's contents in it."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from i_amd import Component as i, I
+from i_amd import _native as nat
+from i_amd import ilang
+
+pytestmark = pytest.mark.gpu
+LIMIT = 64 << 20  # I_HIP_STATIC_WORKSPACE_BYTES
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+
+    assert torch.cuda.is_available()
+    return torch
+
+
+def softmax_naive(s="i:16,j:16"):
+    return (((I & i(f">ij~i|{s}|jii'j'")) >> i(f"ij-i~ij|{s}|1jii'j'")) >> i(f"^ij~ij|{s}|jii'j'")
+            >> ((I & i(f"+ij~i|{s}|jii'j'")) >> i(f"ij/i~ij|{s}|1jii'j'")))
+
+
+def call(entry, comp, inputs, outputs, torch):
+    """One call of a device entry point of the C ABI on torch tensors, on the current stream."""
+    in_records, keep_in = ilang._pack([ilang._operand(x, "input") for x in inputs], on_device=True)
+    out_records, keep_out = ilang._pack([ilang._operand(x, "output") for x in outputs], on_device=True)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = entry(comp._compile(), in_records, len(inputs), out_records, len(outputs), stream)
+    torch.cuda.synchronize()
+    return rc
+
+
+def both(comp, inputs, torch, out_dtype=None):
+    shapes = comp.output_shapes(*inputs)
+    outs_a = [torch.full(s, float("nan"), dtype=out_dtype or torch.float32, device="cuda") for s in shapes]
+    outs_b = [torch.full(s, float("nan"), dtype=out_dtype or torch.float32, device="cuda") for s in shapes]
+    assert call(nat.core.i_exec_into_device, comp, inputs, outs_a, torch) == 0, nat.last_error()
+    assert call(nat.core.i_exec_into_device_noalloc, comp, inputs, outs_b, torch) == 0, nat.last_error()
+    for a, b in zip(outs_a, outs_b):
+        assert torch.isfinite(a.float()).all()
+        assert torch.equal(a, b)
+    return outs_b
+
+
+def randn(torch, shape, seed, dtype=None):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    return x.cuda().to(dtype) if dtype else x.cuda()
+
+
+def test_naive_softmax_twice_second_smaller(torch):
+    comp = softmax_naive()
+    for shape in ((1024, 2000), (100, 37)):  # 2 x 7.8 MiB of intermediates, then a smaller problem in the same array
+        print("case naive softmax", shape, flush=True)
+        (y,) = both(comp, [randn(torch, shape, 1)], torch)
+        ref = torch.softmax(randn(torch, shape, 1).double(), dim=-1)
+        assert float((y.double() - ref).abs().max() / ref.abs().max()) <= 1e-4
+
+
+def test_bf16_operands_and_outputs_are_staged_in_the_workspace(torch):
+    comp = softmax_naive()
+    for shape in ((512, 768), (33, 40)):
+        print("case bf16 staging", shape, flush=True)
+        both(comp, [randn(torch, shape, 2, torch.bfloat16)], torch, out_dtype=torch.bfloat16)
+
+
+def test_transposed_operand_and_generated_kernels(torch):
+    plain = i("ik*kj~ijk|i:16,j:16|jii'j'k") >> i("+ijk~ij|i:16,j:16|jii'j'k0")  # f32, ragged: transpose + NT kernel
+    unfused = i("ik*kj~ijk") >> i("+ijk~ij")                                        # two generated kernels, [i,j,k] between
+    for m, k, n in ((300, 96, 77), (40, 32, 9)):
+        print("case products", (m, k, n), flush=True)
+        a, b = randn(torch, (m, k), 3), randn(torch, (k, n), 4)
+        (c,) = both(plain, [a, b], torch)
+        ref = a.double() @ b.double()
+        assert float((c.double() - ref).abs().max() / ref.abs().max()) <= 1e-4
+        (c2,) = both(unfused, [a, b], torch)
+        assert float((c2.double() - ref).abs().max() / ref.abs().max()) <= 1e-4
+
+
+def test_operands_beyond_the_workspace_are_refused_before_anything_runs(torch):
+    comp = softmax_naive()
+    x = randn(torch, (8192, 4096), 5)  # two 128 MiB intermediates
+    y = torch.full((8192, 4096), 7.0, device="cuda")
+    print("case refusal", flush=True)
+    assert call(nat.core.i_exec_into_device_noalloc, comp, [x], [y], torch) == -1
+    message = nat.last_error()
+    assert str(2 * 8192 * 4096 * 4) in message and str(LIMIT) in message
+    assert bool((y == 7.0).all())  # nothing was enqueued
+    # and the entry point still works afterwards
+    both(comp, [randn(torch, (64, 64), 6)], torch)
