@@ -10,10 +10,17 @@ bf16 inputs, f32 accumulation, f32 output, scores scaled by 1/sqrt(d).
 Prints ONE JSON line.  Besides the headline TFLOP/s it carries
   roofline      achieved vs MI355X dense bf16 MFMA peak for the attention kernel,
                 from HIP events recorded on the launch stream
-  cpu_baseline  the CPU oracle (scalar port of the reference C backend's loop
-                nest) timed on one host core on a bounded sample
-  secondary     row-softmax [16384,4096] f32 (HBM bound), mm_t 4096^3 bf16 and the
-                long-sequence attention B1 H16 N32768 d64 (inputs x 2.0)
+  cpu_baseline  the C the reference backend emits for the benchmark's own
+                component strings, compiled with the reference's command
+                (cc -O3 -shared -fPIC -lm) and timed on one host core on a
+                bounded sample, with the GPU result checked against it
+  secondary     row-softmax [16384,4096] f32 (HBM bound), mm_t 4096^3 bf16, the
+                long-sequence attention B1 H16 N32768 d64 (inputs x 2.0) and the
+                reference's own demo (attention f32 [512,64]), each with its own
+                roofline, cpu_baseline and rel_err
+
+Operands follow the recipe of the reference's scripts (NumPy default_rng(seed),
+seeds 1, 2, 3 for the first, second, third operand; ilang-python/flash-attn.py:33-35).
 
 roofline.traffic is the HBM traffic per launch measured with rocprofv3
 (FETCH_SIZE + WRITE_SIZE passes, scaled by a plain copy of known size); it is read
@@ -31,6 +38,10 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# launches of the headline kernel before the W warm-up steps: the compile-and-first-run call plus 40 more.  The
+# launch time of a fresh process keeps falling over its first two dozen launches (2.2 ms -> 1.8 ms while the
+# clocks settle); this brings the device to that steady state whatever W is.
+PRE_WARMUP_LAUNCHES = 41
 
 
 def flash_component(i, I, split):
@@ -92,6 +103,37 @@ def time_steps(torch, fn, steps, warmup):
     return wall_ms, kernel_ms
 
 
+def host_cpu_model():
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def rel_err(got, ref):
+    import numpy as np
+
+    return float(np.abs(got - ref).max() / max(float(np.abs(ref).max()), 1e-30))
+
+
+def emitted_c_baseline(oracle, component, operands, work, unit, sample, got, repeats=1):
+    """Times the C emitted for `component` (compiled the reference's way) on `operands` (NumPy, f32) on one host
+    core, and compares `got` (the GPU's result for the same operands) with what it computes."""
+    prog = oracle.compile_component(component.handle)
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        ref = prog.run(*operands)
+    seconds = (time.perf_counter() - t0) / repeats
+    err = rel_err(got, ref)
+    return {"value": work / seconds, "unit": unit, "cores": 1, "kind": "port",
+            "form": "emitted-c: the C that the restated reference C backend prints for this line's own component "
+                    "strings, built with cc -O3 -shared -fPIC -lm and run through count/ranks/shapes/exec",
+            "host_cpu": host_cpu_model(), "seconds": seconds, "sample": sample}, err
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -100,6 +142,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="time the emitted C of mm_t on the whole workload instead of a sample (about four minutes)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, a kernel of known traffic for scaling profiler counters")
     args = ap.parse_args()
@@ -113,19 +157,25 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+
+    def normal(shape, seed, amp=1.0):
+        return np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(amp)
+
+    def to_dev_bf16(a):
+        return torch.from_numpy(a).to(dev).bfloat16()
+
+    # ------------------------------------------------------------------ headline: attention B8 H32 N4096 d128
     B, H, N, D = 8, 32, 4096, 128
-    gen = torch.Generator(device=dev).manual_seed(1)
-    q, k, v = (torch.randn(B, H, N, D, device=dev, generator=gen).bfloat16() for _ in range(3))
-    scale = torch.tensor(1.0 / np.sqrt(D), dtype=torch.float32, device=dev)
+    q, k, v = (to_dev_bf16(normal((B, H, N, D), seed)) for seed in (1, 2, 3))
+    scale = torch.tensor(np.float32(1.0 / np.sqrt(D)), dtype=torch.float32, device=dev)
     out = torch.empty(B, H, N, D, dtype=torch.float32, device=dev)
     attn = flash_component(i, I, "i:256,j:64")
     attn.into(out, q, k, scale, v)  # compile + first run outside the timed region
-    # The launch time of a fresh process keeps falling over its first two dozen launches (2.2 ms -> 1.8 ms while
-    # the clocks settle).  Bring the device to that steady state before the W warm-up steps, whatever W is.
-    for _ in range(40):
+    for _ in range(PRE_WARMUP_LAUNCHES - 1):
         attn.into(out, q, k, scale, v)
     torch.cuda.synchronize()
     wall_ms, kernel_ms = time_steps(torch, lambda: attn.into(out, q, k, scale, v), args.steps, args.warmup)
+    attn_kernel = attn.report().split()[1]
     flop = 4.0 * B * H * N * N * D
     tflops = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (kernel_ms * 1e-3) / 1e12
@@ -138,15 +188,16 @@ def main():
     del qc, kc, vc
     attn.into(out, q, k, scale, v)  # leave the seeded result in `out` for the parity check below
 
-    # ---- secondary: row softmax (HBM bound) and mm_t (MFMA bound)
+    # ------------------------------------------------------------------ row softmax [16384, 4096] f32 (HBM bound)
     rows, cols = 16384, 4096
-    x = torch.randn(rows, cols, device=dev, generator=gen)
+    x = torch.from_numpy(normal((rows, cols), 1)).to(dev)
     y = torch.empty_like(x)
     sm = softmax_component(i, I)
     sm.into(y, x)
+    sm_kernel = sm.report().split()[1]
     # The timed calls walk four input/output pairs (2 GiB): one pair alone (512 MiB) would be re-read partly out of
     # the 256 MiB Infinity Cache from one step to the next, and that is not HBM bandwidth.
-    xs = [x] + [torch.randn(rows, cols, device=dev, generator=gen) for _ in range(3)]
+    xs = [x] + [torch.from_numpy(normal((rows, cols), 10 + n)).to(dev) for n in range(3)]
     ys = [y] + [torch.empty_like(x) for _ in range(3)]
     turn = [0]
 
@@ -164,110 +215,132 @@ def main():
     sm_bytes = 2.0 * rows * cols * 4
     sm_gbs = sm_bytes / (sm_ms * 1e-3) / 1e9
 
+    # ------------------------------------------------------------------ mm_t 4096^3 bf16 (MFMA bound)
+    import oracle  # the CPU side of the checks below; never on the timed path
+
     M = 4096
-    a = (torch.rand(M, M, device=dev, generator=gen) * 2 - 1).bfloat16()
-    b = (torch.rand(M, M, device=dev, generator=gen) * 2 - 1).bfloat16()
+    a_host = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (M, M)).astype(np.float32))
+    b_host = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (M, M)).astype(np.float32))
+    a, b = to_dev_bf16(a_host), to_dev_bf16(b_host)
     c = torch.empty(M, M, device=dev)
     mm = mm_t_component(i)
     mm.into(c, a, b)
+    mm_kernel = mm.report().split()[1]
     _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), short_steps, short_warmup)
     mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
 
-    # long-sequence attention (heavy running-max movement): B1 H16 N32768 d64, inputs x 2.0
+    # ------------------------------------------------------------------ long-sequence attention B1 H16 N32768 d64, x 2.0
     B5, H5, N5, D5 = 1, 16, 32768, 64
-    q5, k5, v5 = ((torch.randn(B5, H5, N5, D5, device=dev, generator=gen) * 2.0).bfloat16() for _ in range(3))
-    scale5 = torch.tensor(1.0 / np.sqrt(D5), dtype=torch.float32, device=dev)
+    q5, k5, v5 = (to_dev_bf16(normal((B5, H5, N5, D5), seed, 2.0)) for seed in (1, 2, 3))
+    scale5 = torch.tensor(np.float32(1.0 / np.sqrt(D5)), dtype=torch.float32, device=dev)
     out5 = torch.empty(B5, H5, N5, D5, dtype=torch.float32, device=dev)
     attn5 = flash_component(i, I, "i:512,j:32")  # 512 query rows per workgroup, 32-key LDS tiles: the d = 64 kernel
     attn5.into(out5, q5, k5, scale5, v5)
+    c5_kernel = attn5.report().split()[1]
     _, c5_ms = time_steps(torch, lambda: attn5.into(out5, q5, k5, scale5, v5), max(args.steps // 2, 5), 2)
     c5_tflops = 4.0 * B5 * H5 * N5 * N5 * D5 / (c5_ms * 1e-3) / 1e12
+
+    # ------------------------------------------------------------------ the reference's own demo: attention f32 [512, 64]
+    # (BASELINE configs[0]): no scale, i:16,j:16, through the f32 kernel.  Timed here, with the other GPU work and
+    # before the host legs below: after seconds of CPU-only work the device has clocked down, and a 70 us kernel
+    # timed then reads ten times slower.
+    demo_in = [np.random.default_rng(sd).uniform(-1, 1, (512, 64)).astype(np.float32) for sd in (1, 2, 3)]
+    demo = flash_demo_component(i, I)
+    dq, dk, dv_ = (torch.from_numpy(t).to(dev) for t in demo_in)
+    dout = torch.empty(512, 64, device=dev)
+    demo.into(dout, dq, dk, dv_)
+    c1_kernel = demo.report().split()[1]
+    _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), 200, 50)
+    c1_flop = 4.0 * 512 * 512 * 64
 
     if args.calibrate_copy:
         y.copy_(x)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
 
-    # ---- CPU baseline: the oracle on one host core, one (b, h) slice of the same workload
-    cpu = None
+    # ------------------------------------------------------------------ host legs: emitted C on one core, and the checks
+    cpu = cpu2 = cpu3 = cpu5 = cpu1 = None
+    err4 = err2 = err3 = err5 = err1 = None
     if not args.no_cpu_baseline:
-        import oracle
+        # C4: one (b, h) slice of the workload, 1024 of its 4096 query rows (query tiles and (b, h) pairs are the
+        # outermost independent loops of the emitted nest, so the rate carries over to the whole workload)
+        b0, h0, r4 = 3, 17, 2048
+        ops = [q[b0:b0 + 1, h0:h0 + 1, :r4].float().cpu().numpy(), k[b0:b0 + 1, h0:h0 + 1].float().cpu().numpy(),
+               np.float32(scale.item()), v[b0:b0 + 1, h0:h0 + 1].float().cpu().numpy()]
+        cpu, err4 = emitted_c_baseline(
+            oracle, attn, ops, 4.0 * r4 * N * D / 1e12, "TFLOP/s",
+            f"(b,h) = ({b0},{h0}), query rows 0..{r4 - 1} against all {N} keys: 1/{B * H * N // r4} of the workload "
+            "(independent outer loops: the rate carries over)", out[b0:b0 + 1, h0:h0 + 1, :r4].cpu().numpy())
+        # C2: rows are independent
+        r2 = rows  # the whole workload: a few seconds
+        cpu2, err2 = emitted_c_baseline(
+            oracle, sm, [x[:r2].cpu().numpy()], 2.0 * r2 * cols * 4 / 1e9, "GB/s",
+            f"rows 0..{r2 - 1} of {rows} (algorithmic bytes of those rows)", y[:r2].cpu().numpy())
+        # C3: output tiles are independent; all of k
+        m3 = M if args.cpu_full else 1024
+        cpu3, err3 = emitted_c_baseline(
+            oracle, mm, [a_host[:m3], b_host[:m3]], 2.0 * m3 * m3 * M / 1e12, "TFLOP/s",
+            f"rows 0..{m3 - 1} of A against rows 0..{m3 - 1} of B, all {M} of k: 1/{(M // m3) ** 2} of the workload",
+            c[:m3, :m3].cpu().numpy())
+        # C5: one head, 512 of its 32768 query rows against all keys
+        h5, r5 = 7, 512
+        ops5 = [q5[:, h5:h5 + 1, :r5].float().cpu().numpy(), k5[:, h5:h5 + 1].float().cpu().numpy(),
+                np.float32(scale5.item()), v5[:, h5:h5 + 1].float().cpu().numpy()]
+        cpu5, err5 = emitted_c_baseline(
+            oracle, attn5, ops5, 4.0 * r5 * N5 * D5 / 1e12, "TFLOP/s",
+            f"head {h5}, query rows 0..{r5 - 1} against all {N5} keys: 1/{H5 * N5 // r5} of the workload",
+            out5[:, h5:h5 + 1, :r5].cpu().numpy())
+        # C1: the whole workload; the reference's own committed emission when it was built, else the C emitted here
+        got1 = dout.cpu().numpy()
+        if oracle.have_ref():
+            oracle.ref_flash_attention(*demo_in)
+            t0 = time.perf_counter()
+            for _ in range(5):
+                ref1 = oracle.ref_flash_attention(*demo_in)
+            c1_s = (time.perf_counter() - t0) / 5
+            err1 = rel_err(got1, ref1)
+            cpu1 = {"value": c1_flop / c1_s / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference",
+                    "form": "the reference's committed emission ilang-python/annotated-flashattn.c, built unmodified",
+                    "host_cpu": host_cpu_model(), "seconds": c1_s, "sample": "the whole workload"}
+        else:
+            cpu1, err1 = emitted_c_baseline(oracle, demo, demo_in, c1_flop / 1e12, "TFLOP/s", "the whole workload", got1, 5)
 
-        heads = 4  # b = 0, h = 0..3: about 10 s of scalar CPU work
-        qs, ks, vs = (t[0, :heads].float().cpu().numpy() for t in (q, k, v))
-        t0 = time.perf_counter()
-        ref = oracle.attention_tiled(qs, ks, vs, float(scale), 16, 16)
-        cpu_s = time.perf_counter() - t0
-        got = out[0, :heads].cpu().numpy()
-        rel = float(np.abs(got - ref).max() / np.abs(ref).max())
-        cpu = {
-            "value": heads * 4.0 * N * N * D / cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"{heads} (b,h) slices of the workload (N={N}, d={D}; {heads} of {B * H}), {cpu_s:.1f} s, "
-                      f"16x16 tiles as in the reference demo; GPU vs oracle on those slices: rel err {rel:.1e}",
-        }
-
-    # ---- the reference's own CPU-runnable case (BASELINE configs[0]): demo attention, f32 [512,64], no scale,
-    # i:16,j:16 schedule; on the GPU through the f32 kernel, on the host through the reference's emitted C
-    # (oracle/_ref, compiled from the reference tree when it was mounted at build time) or the oracle port
-    c1 = None
-    if not args.no_cpu_baseline:
-        import oracle
-
-        rng = [np.random.default_rng(sd).uniform(-1, 1, (512, 64)).astype(np.float32) for sd in (1, 2, 3)]
-        demo = flash_demo_component(i, I)
-        dq, dk, dv_ = (torch.from_numpy(a).to(dev) for a in rng)
-        dout = torch.empty(512, 64, device=dev)
-        demo.into(dout, dq, dk, dv_)
-        _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), 50, 5)
-        use_ref = oracle.have_ref()
-        host = (lambda: oracle.ref_flash_attention(*rng)) if use_ref else (lambda: oracle.attention_tiled(*rng))
-        host()
-        t0 = time.perf_counter()
-        for _ in range(5):
-            ref1 = host()
-        c1_cpu_s = (time.perf_counter() - t0) / 5
-        c1_flop = 4.0 * 512 * 512 * 64
-        c1_rel = float(np.abs(dout.cpu().numpy() - ref1).max() / np.abs(ref1).max())
-        c1 = {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
-              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": c1_ms,
-              "cpu_baseline": {"value": c1_flop / c1_cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1,
-                               "kind": "reference" if use_ref else "port",
-                               "sample": f"the whole workload, {c1_cpu_s * 1e3:.1f} ms per run; GPU vs host rel err {c1_rel:.1e}"}}
+    def roof(bound, achieved_, peak, unit, summary, kernel, ms):
+        return {"bound": bound, "achieved": achieved_, "peak": peak, "unit": unit, "frac": achieved_ / peak,
+                "traffic": measured_traffic(summary), "kernel": kernel, "kernel_ms": ms}
 
     line = {
         "metric": "attn TFLOP/s & %MFMA peak (B8,H32,N4096,d128); row-softmax HBM GB/s",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "pre_warmup_launches": PRE_WARMUP_LAUNCHES,
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic (NumPy default_rng seeds 1, 2, 3: standard_normal -> bf16)",
         "config": {"workload": "flash_attention_fwd B8 H32 N4096 d128, bf16 in / f32 accumulate / f32 out, "
                                "1/sqrt(d) scale, non-causal (BASELINE configs[3]); compiled from 𝚒 component strings",
                    "schedule": "i:256,j:64 (256 query rows per workgroup, 64-key LDS tiles)", "entry": "i_exec_into_device"},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": measured_traffic("flash_attention_B8_H32_N4096_d128_bf16.md"),
-                     "kernel": "attn_fwd_bf16_d128_bn64_direct_w8", "kernel_ms": kernel_ms},
-        "cpu_baseline": cpu,
+        "roofline": roof("mfma", achieved, PEAK_BF16_TFLOPS, "TFLOP/s", "flash_attention_B8_H32_N4096_d128_bf16.md",
+                         attn_kernel, kernel_ms),
+        "cpu_baseline": cpu, "rel_err": err4,
         "constant_operand_probe": {
             "workload": "the same launch with every element of Q, K, V equal to 0.01 (not the benchmark data)",
             "value": flop / (const_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": const_ms,
             "frac_of_peak": flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
-             "roofline": {"bound": "hbm", "achieved": sm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                          "frac": sm_gbs / PEAK_HBM_GBS, "traffic": measured_traffic("row_softmax_16384x4096_f32.md"),
-                          "kernel": "row_softmax_wave_v16",
-                          "kernel_ms": sm_ms}},
+             "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),
+             "cpu_baseline": cpu2, "rel_err": err2},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
-             "roofline": {"bound": "mfma", "achieved": mm_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                          "frac": mm_tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("gemm_nt_4096x4096x4096_bf16.md"),
-                          "kernel": "gemm_nt_bf16_256x256x64_direct", "kernel_ms": mm_ms}},
+             "roofline": roof("mfma", mm_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_nt_4096x4096x4096_bf16.md", mm_kernel, mm_ms),
+             "cpu_baseline": cpu3, "rel_err": err3},
             {"workload": "flash_attention_fwd B1 H16 N32768 d64, bf16 inputs x 2.0 (BASELINE configs[4])",
              "schedule": "i:512,j:32 (512 query rows per workgroup, 64 per wave; 32-key LDS tiles)",
              "value": c5_tflops, "unit": "TFLOP/s",
-             "roofline": {"bound": "mfma", "achieved": c5_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                          "frac": c5_tflops / PEAK_BF16_TFLOPS,
-                          "traffic": measured_traffic("flash_attention_B1_H16_N32768_d64_bf16.md"),
-                          "kernel": "attn_fwd_bf16_d64_bn32_q64", "kernel_ms": c5_ms}},
-        ] + ([c1] if c1 else []),
+             "roofline": roof("mfma", c5_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "flash_attention_B1_H16_N32768_d64_bf16.md",
+                              c5_kernel, c5_ms),
+             "cpu_baseline": cpu5, "rel_err": err5},
+            {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
+             "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,
+             "cpu_baseline": cpu1, "rel_err": err1},
+        ],
     }
     print(json.dumps(line))
 

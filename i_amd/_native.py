@@ -37,6 +37,13 @@ core.i_error.restype = ctypes.c_char_p
 
 core.i_hip_attention.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, sz, sz, sz, sz, sz, ctypes.c_float, vp]
 core.i_hip_attention.restype = ctypes.c_int
+core.i_hip_attention_ex.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, sz, sz, sz, sz, sz, ctypes.c_float, sz, sz,
+                                    ctypes.c_int, vp]
+core.i_hip_attention_ex.restype = ctypes.c_int
+core.i_hip_program_option.argtypes = [vp, ctypes.c_char_p, ctypes.c_int]
+core.i_hip_program_option.restype = ctypes.c_int
+core.i_hip_program_report.argtypes = [vp]
+core.i_hip_program_report.restype = vp
 core.i_hip_gemm_nt_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nt_bf16.restype = ctypes.c_int
 core.i_hip_gemm_nn_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]

@@ -42,6 +42,7 @@ struct Run {
   std::map<size_t, void*> input_f32;         // bf16 inputs widened for f32 kernels
   std::map<size_t, void*> output_f32;        // f32 staging for bf16 outputs
   Workspace* workspace = nullptr;            // when set, temporaries are carved out of it and nothing is allocated
+  std::vector<std::string> notes;            // one line per dispatched kernel: what ran, on which tile
 
   size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
   size_t extent(const Extent<size_t>& e) const {
@@ -183,7 +184,20 @@ std::set<size_t> hand_intermediates(const Recognized& r) {
   return out;
 }
 
-ihip::Err launch_hand(Run& run, const Recognized& r) {
+// "attn_... (tile 256 x 64)", with the schedule's request spelled out when no kernel has that tile
+std::string describe_launch(const ihip::LaunchNote& note, const Recognized& r) {
+  std::string text = note.kernel;
+  if (note.tile_i || note.tile_j) {
+    text += " (tile " + std::to_string(note.tile_i) + " x " + std::to_string(note.tile_j);
+    if ((r.tile_i || r.tile_j) && (r.tile_i != note.tile_i || r.tile_j != note.tile_j))
+      text += "; the schedule asks for " + std::to_string(r.tile_i) + " x " + std::to_string(r.tile_j) +
+              ", which no hand-written kernel has for these operands";
+    text += ")";
+  }
+  return text;
+}
+
+ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* note) {
   switch (r.kind) {
     case Recognized::Attention: {
       const auto q = run.shape_of(r.a.buffer), k = run.shape_of(r.b.buffer), v = run.shape_of(r.c.buffer);
@@ -212,7 +226,7 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       }
       return ihip::launch_attention(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), run.raw_ptr(r.c.buffer), out,
                                     bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream,
-                                    r.tile_i);
+                                    ihip::AttentionOptions{r.tile_i, r.tile_j, run.p.attention_f32_scale.load()}, note);
     }
     case Recognized::GemmNT: {
       const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
@@ -228,9 +242,9 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       if (run.dtype_of(r.a.buffer) == DType::F32)
         return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)),
                                         static_cast<const float*>(run.raw_ptr(r.b.buffer)), static_cast<float*>(out), bh,
-                                        a[nb], b[nb], a[nb + 1], run.stream);
+                                        a[nb], b[nb], a[nb + 1], run.stream, note);
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
-                                       a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j);
+                                       a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j, note);
     }
     case Recognized::GemmNN: {
       // b [B.., K, J]: the direct bf16 kernels read it in place; otherwise it is transposed into a stream-ordered
@@ -250,7 +264,7 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
         void* out = nullptr;
         if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
         return ihip::launch_gemm_nn_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh, m, n, k,
-                                         run.stream, r.tile_i, r.tile_j);
+                                         run.stream, r.tile_i, r.tile_j, note);
       }
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
@@ -260,9 +274,9 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
       if (f32)
         return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)), static_cast<const float*>(bt),
-                                        static_cast<float*>(out), bh, m, n, k, run.stream);
+                                        static_cast<float*>(out), bh, m, n, k, run.stream, note);
       return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, static_cast<float*>(out), bh, m, n, k, run.stream,
-                                       r.tile_i, r.tile_j);
+                                       r.tile_i, r.tile_j, note);
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
@@ -275,10 +289,17 @@ ihip::Err launch_hand(Run& run, const Recognized& r) {
       if (ihip::Err e = run.read_f32(r.a.buffer, &in); !e.empty()) return e;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
       const int mode = r.kind == Recognized::RowSoftmax ? 0 : r.kind == Recognized::RowMaxShift ? 1 : r.kind == Recognized::RowNormalize ? 2 : 3;
-      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode);
+      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode, note);
     }
     default: return "no hand-written kernel";
   }
+}
+
+ihip::Err launch_hand(Run& run, const Recognized& r) {
+  ihip::LaunchNote note;
+  const ihip::Err err = launch_hand_noted(run, r, &note);
+  if (err.empty()) run.notes.push_back(note.kernel.empty() ? "nothing to do (empty operands)" : describe_launch(note, r));
+  return err;
 }
 
 // ---------------------------------------------------------------- generated kernels
@@ -335,6 +356,7 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
     fill(nr + i, ptr, dispatch.writes[i]);
   }
 
+  run.notes.push_back("generated kernel " + gk.name + (gk.phases.size() > 1 ? " in " + std::to_string(gk.phases.size()) + " launches" : ""));
   // one launch per phase, in order on the stream
   for (const GenericPhase& ph : gk.phases) {
     size_t total = 1;
@@ -452,6 +474,19 @@ std::string program_code(const Component& component) {
       if (rec[k].has_scale) os << ", scale " << ref_name(rec[k].scale.buffer);
       os << " -> " << ref_name(rec[k].out) << "]; generated form below runs when operands are outside its limits";
     }
+    if (rec[k].kind == Recognized::Attention || rec[k].kind == Recognized::GemmNT || rec[k].kind == Recognized::GemmNN) {
+      // which of the schedule's tiles exist as kernels is a property of the kernel set, known here; which one
+      // runs also depends on the operands (head size, dtype, problem size) and is reported after a run
+      const size_t ti = rec[k].tile_i, tj = rec[k].tile_j;
+      const bool attn = rec[k].kind == Recognized::Attention;
+      const bool known = attn ? (((ti == 64 || ti == 128 || ti == 256) && (tj == 32 || tj == 64)) || (ti == 512 && tj == 32))
+                              : ((ti == 128 && tj == 128) || (ti == 256 && tj == 256));
+      os << "\n//     " << (known ? "the schedule tile selects the kernel with that workgroup tile where the operands allow it"
+                                   : "no hand-written kernel has this tile: the launcher picks one by problem size")
+         << (attn ? " (attention tiles: 64 / 128 / 256 query rows x 32 / 64 keys, 512 x 32 at d = 64)"
+                  : " (GEMM tiles: 128 x 128, 256 x 256)")
+         << "; i_hip_program_report names the kernel that ran";
+    }
     os << "\n//     reads";
     for (BufferRef r : d->reads) os << " " << ref_name(r);
     os << "; writes";
@@ -558,12 +593,33 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
       if (!e.empty()) return finish("kernel f" + std::to_string(step.id) + ": " + e);
     }
   }
+  {
+    std::string report;
+    size_t n = 0;
+    for (const Step& step : plan.exec)
+      if (step.kind == Step::Dispatch && n < run.notes.size()) report += "f" + std::to_string(step.id) + ": " + run.notes[n++] + "\n";
+    std::lock_guard<std::mutex> lock(p.mu);
+    p.last_report = std::move(report);
+  }
   // bf16 outputs that were produced through f32 staging
   for (const auto& [o, tmp] : run.output_f32) {
     const size_t n = product(run.shape_of({BufferRef::Output, o}));
     if (ihip::Err e = ihip::launch_convert(tmp, outputs[o].data, ihip::F32, ihip::BF16, n, stream); !e.empty()) return finish(e);
   }
   return finish({});
+}
+
+std::string set_option(Program& p, const std::string& name, int value) {
+  if (name == "attention.f32_scale") {
+    p.attention_f32_scale.store(value != 0);
+    return {};
+  }
+  return "unknown program option '" + name + "' (known: attention.f32_scale)";
+}
+
+std::string last_report(Program& p) {
+  std::lock_guard<std::mutex> lock(p.mu);
+  return p.last_report;
 }
 
 std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,

@@ -7,6 +7,7 @@
 #pragma once
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <string>
@@ -38,6 +39,10 @@ struct Program {
   bool image_built = false;
   std::mutex mu;
   std::map<int, hipModule_t> modules;  // per device
+  // options (set_option): apply the attention score scale in f32 to every score instead of folding it into Q
+  std::atomic<bool> attention_f32_scale{false};
+  // what the last execute() dispatched: one line per kernel, "f<k>: <kernel name> (tile ...)"; guarded by mu
+  std::string last_report;
 
   ~Program();
 };
@@ -72,6 +77,11 @@ struct Workspace {
 // call allocates and frees no device memory.  Returns "" on success.
 std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
                     hipStream_t stream, Workspace* workspace = nullptr);
+
+// Program options by name; returns "" or the failure text.  Known: "attention.f32_scale" (0 / 1).
+std::string set_option(Program& p, const std::string& name, int value);
+// The kernels the last execute() of this program dispatched, one per line.
+std::string last_report(Program& p);
 
 // What execute() with a workspace would take from it for these operands, in bytes.  Launches nothing.
 std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,

@@ -359,6 +359,28 @@ int i_exec_into_device_noalloc(const i_program* program, const i_device_tensor* 
   }
 }
 
+int i_hip_program_option(i_program* program, const char* name, int value) {
+  if (!program) return fail("null program");
+  if (!name) return fail("null option name");
+  const std::string err = ihipc::set_option(*program->inner, name, value);
+  return err.empty() ? 0 : fail(err);
+}
+
+char* i_hip_program_report(const i_program* program) {
+  if (!program) {
+    icore::set_error("null program");
+    return nullptr;
+  }
+  const std::string text = ihipc::last_report(*program->inner);
+  char* out = static_cast<char*>(std::malloc(text.size() + 1));
+  if (!out) {
+    icore::set_error("out of memory");
+    return nullptr;
+  }
+  std::memcpy(out, text.c_str(), text.size() + 1);
+  return out;
+}
+
 void i_component_free(i_component* component) { delete component; }
 
 void i_program_free(i_program* program) { delete program; }

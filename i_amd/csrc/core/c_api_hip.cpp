@@ -22,6 +22,15 @@ int i_hip_attention(const void* q, const void* k, const void* v, void* o, int in
                                        nullptr, scale, (hipStream_t)stream));
 }
 
+int i_hip_attention_ex(const void* q, const void* k, const void* v, void* o, int in_dtype, int out_dtype, size_t bh,
+                       size_t nq, size_t nk, size_t d, size_t dv, float scale, size_t query_tile, size_t key_tile,
+                       int f32_scale, void* stream) {
+  if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype)) return finish("unknown dtype");
+  return finish(ihip::launch_attention(q, k, v, o, (ihip::DType)in_dtype, (ihip::DType)out_dtype, bh, nq, nk, d, dv,
+                                       nullptr, scale, (hipStream_t)stream,
+                                       ihip::AttentionOptions{query_tile, key_tile, f32_scale != 0}));
+}
+
 int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k, void* stream) {
   return finish(ihip::launch_gemm_nt_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream));
 }

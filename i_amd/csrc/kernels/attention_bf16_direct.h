@@ -63,7 +63,10 @@
 #define ATTN_STAGED_STORE 1
 #endif
 
-template <int DPAD, int BN, int NWAVES>
+// PRECISE: the score scale is applied in f32 to every score (the reference's arithmetic,
+// compiler/src/lower/exec_plan_to_module.rs:605-640) instead of being folded into Q with one more bf16 rounding;
+// the steady state then keeps a reference for its exponentials at either head size.  About 5 % slower.
+template <int DPAD, int BN, int NWAVES, bool PRECISE = false>
 __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int BM = 32 * NWAVES;
   constexpr int KSTEPS = DPAD / 16;       // k-steps of the QK^T contraction
@@ -112,8 +115,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // wave notes (without branching) whether any tile's row sum reached 2^80 and, at the end, whether a row sum
   // fell below 2^-100; if any wave of the workgroup did, the workgroup throws the pass away and computes the item
   // again with the general loop, which takes the running max tile by tile.
-  constexpr bool PRESCALE = DPAD == 64;
-  constexpr bool NOREF = DPAD == 128 && ATTN_NOREF;
+  constexpr bool PRESCALE = DPAD == 64 && !PRECISE;
+  constexpr bool NOREF = DPAD == 128 && ATTN_NOREF && !PRECISE;
   constexpr bool QSCALE = PRESCALE || NOREF;
   // f32 output written through LDS (see the epilogue): 8 KiB of tile memory per wave
   constexpr bool STAGED_STORE = ATTN_STAGED_STORE && NWAVES * 8192 <= 4 * TILE_BYTES;
@@ -154,10 +157,14 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const uint32_t lrow = lane / CH, lch = lane % CH;
   const uint32_t smem0 = lds_address(&smem[0][0][0]);
 
-  // For a full tile the per-lane part of the address is the same for every tile and every wave-load
-  // (the swizzle term does not depend on `it` because NWAVES * RPW rows is a multiple of the swizzle
-  // period); everything that varies is wave-uniform and is folded into the scalar base address.
-  static_assert((NWAVES * RPW / RPB) % CH == 0, "swizzle period");
+  // For a full tile the per-lane part of the address is the same for every tile, and for every wave-load when
+  // the NWAVES * RPW rows between a wave's consecutive wave-loads are a multiple of the swizzle period.  With
+  // fewer waves (KSTRIDE < CH) the K swizzle of wave-load `it` differs from that of wave-load 0 in the bits
+  // (KSTRIDE * it) % CH, which the rows of one wave-load (fewer than KSTRIDE swizzle steps) never reach: one
+  // XOR with a constant.  Everything else that varies is wave-uniform and is folded into the scalar base address.
+  constexpr int KSTRIDE = NWAVES * RPW / RPB;  // swizzle steps between consecutive wave-loads of a wave
+  static_assert((KSTRIDE & (KSTRIDE - 1)) == 0 && (KSTRIDE % CH == 0 || CH % KSTRIDE == 0), "swizzle period");
+  static_assert((NWAVES * RPW / RPB) % (CH / 4) == 0, "V swizzle period");
   const uint32_t lane_row = wave * RPW + lrow;
   const uint32_t koff_lane = lrow * RB + 16 * (lch ^ ((lane_row / RPB) % CH));
   const uint32_t voff_lane = lrow * RB + 16 * (lch ^ (4 * ((lane_row / RPB) % (CH / 4))));
@@ -165,7 +172,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   auto request_full_one = [&](uint32_t tile, int buf, int it, auto want_k) {
     const uint32_t w = wave + NWAVES * it;
     const size_t byte0 = (size_t)tile * TILE_BYTES + w * 1024;
-    if constexpr (decltype(want_k)::value) dma16(K + byte0, koff_lane, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+    if constexpr (decltype(want_k)::value)
+      dma16(K + byte0, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
     else dma16(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
   };
 
@@ -173,7 +181,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   auto request_k_one = [&](uint32_t tile, int buf, int it) {
     if (tile < nfull_tiles) {
       const uint32_t w = wave + NWAVES * it;
-      dma16(K + (size_t)tile * TILE_BYTES + w * 1024, koff_lane, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+      dma16(K + (size_t)tile * TILE_BYTES + w * 1024, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)),
+            smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
     } else if (tile * BN < p.nk) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;
@@ -354,7 +363,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int NPRE = DT + NQK;        // slots that carry the exponentials (all before the first PV slot of the tile)
   constexpr int NMAIN = NPV - DT;       // PV slots of the trip that owns the tile
   constexpr int XLEAD = ATTN_XLEAD;
-  static_assert(NPAIR == 16 && 2 * WLW <= NPRE && XLEAD >= 0 && XLEAD < NQK, "slot shape");
+  static_assert(NPAIR % 4 == 0 && 2 * WLW <= NPRE && XLEAD >= 0 && XLEAD < NQK, "slot shape");
 
   struct Carry {
     bf16x8 a[DT];  // V^T operands of the last 16-key group
@@ -373,7 +382,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // written in.  pq and the row-sum parts live across trips: the first NEARLY pairs of a tile (its key groups 0
   // and 1) are computed one trip early, in the output slots of the previous tile, which otherwise carry no
   // vector work at all, while the score slots are the crowded ones.
-  constexpr int NEARLY = 8;
+  // (With fewer than four key groups per tile there is no output slot after which a group's registers are free
+  // within the same trip, and every pair is computed in the score slots.)
+  constexpr int NEARLY = BN / 16 >= 4 ? 8 : 0;
   f32x16 negmb16 = zero16;  // PRESCALE: -reference in every element, the addend of a score tile's first MFMA
   u32x4 pq[NPAIR / 4];
   float psum[2] = {0.0f, 0.0f};
@@ -513,7 +524,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const int s4 = m / DT, t = m % DT;
       o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[NQK + m], __builtin_bit_cast(bf16x8, pq[s4]), o[t], 0, 0, 0);
       // key groups 0 and 1 of tile j+1, each once the MFMAs that read the group's old registers have been issued
-      if (m >= DT && m < 3 * DT) {
+      if (NEARLY > 0 && m >= DT && m < 3 * DT) {
 #pragma unroll
         for (int pr = (m - DT) * 4 / DT; pr < (m - DT + 1) * 4 / DT; ++pr) exp_pair_from(s_next, pr, mb);
       }

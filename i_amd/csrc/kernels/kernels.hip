@@ -20,20 +20,30 @@
 ATTN_BF16(64, 64, 4, 2)
 ATTN_BF16(128, 64, 4, 2)
 
-// attn_fwd_bf16_d<D>_bn<BN>_direct: d == dv == D, K/V tiles loaded from global memory straight into LDS;
-// ..._w8: eight waves (256 queries) per workgroup, one workgroup per CU
-#define ATTN_BF16_DIRECT(DPAD, BN, NW, OCC)                                                                        \
-  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN##_direct(AttnParams p) { \
-    attn_fwd_bf16_direct_body<DPAD, BN, NW>(p);                                                                    \
+// attn_fwd_bf16_d<D>_bn<BN>_direct[_w2|_w8][_f32scale]: d == dv == D, K/V tiles of BN keys loaded from global memory
+// straight into LDS; 4 waves (128 queries) per workgroup, _w2: two waves (64 queries), _w8: eight waves (256
+// queries, one workgroup per CU); _f32scale: the score scale is applied in f32 instead of being folded into Q
+#define ATTN_BF16_DIRECT(DPAD, BN, NW, OCC, SUFFIX, PRECISE)                                                     \
+  extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN##_direct##SUFFIX(AttnParams p) { \
+    attn_fwd_bf16_direct_body<DPAD, BN, NW, PRECISE>(p);                                                         \
   }
-ATTN_BF16_DIRECT(64, 64, 4, 2)
-ATTN_BF16_DIRECT(128, 64, 4, 2)
-extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d128_bn64_direct_w8(AttnParams p) {
-  attn_fwd_bf16_direct_body<128, 64, 8>(p);
-}
-extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn64_direct_w8(AttnParams p) {
-  attn_fwd_bf16_direct_body<64, 64, 8>(p);
-}
+ATTN_BF16_DIRECT(64, 64, 4, 2, , false)
+ATTN_BF16_DIRECT(128, 64, 4, 2, , false)
+ATTN_BF16_DIRECT(128, 64, 8, 1, _w8, false)
+ATTN_BF16_DIRECT(64, 64, 8, 1, _w8, false)
+ATTN_BF16_DIRECT(128, 64, 2, 1, _w2, false)
+ATTN_BF16_DIRECT(64, 64, 2, 1, _w2, false)
+// 32-key tiles (the schedule's j:32)
+ATTN_BF16_DIRECT(128, 32, 2, 1, _w2, false)
+ATTN_BF16_DIRECT(128, 32, 4, 2, , false)
+ATTN_BF16_DIRECT(128, 32, 8, 1, _w8, false)
+ATTN_BF16_DIRECT(64, 32, 2, 1, _w2, false)
+ATTN_BF16_DIRECT(64, 32, 4, 2, , false)
+// f32 score scale
+ATTN_BF16_DIRECT(128, 64, 4, 2, _f32scale, true)
+ATTN_BF16_DIRECT(128, 64, 8, 1, _w8_f32scale, true)
+ATTN_BF16_DIRECT(64, 64, 4, 2, _f32scale, true)
+ATTN_BF16_DIRECT(64, 64, 8, 1, _w8_f32scale, true)
 // d = 64 with 64 queries per wave (attention_bf16_q64.h): 8 waves, 512 query rows per workgroup, 32-key tiles
 extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(AttnParams p) {
   attn_fwd_bf16_q64_body<64, 32, 8>(p);

@@ -22,7 +22,7 @@ bool attention_supported(DType in_dtype, size_t d, size_t dv) {
 
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
-                     size_t query_tile) {
+                     const AttentionOptions& options, LaunchNote* note) {
   if (!attention_supported(in_dtype, d, dv))
     return "attention kernel: unsupported operands (need 0 < d, dv <= 128; bf16 needs d, dv % 8 == 0)";
   if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
@@ -33,26 +33,31 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   if (!q || !k || !v || !o) return "attention kernel: null device pointer";
 
   const size_t dmax = d > dv ? d : dv;
+  const size_t query_tile = options.query_tile, key_tile = options.key_tile;
   // Kernel choice for bf16:
-  //   d == dv in {64, 128}: direct-to-LDS kernel; a 256-query workgroup (8 waves) halves the
-  //     L2 -> LDS traffic per query; the schedule's query tile (128 / 256) decides, and without one the
-  //     larger workgroup is used on long key loops when it still leaves at least two workgroups per CU and does
-  //     not pad nq by much
-  //   otherwise: register-staged kernel with guarded columns
-  //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512): the
-  //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs
-  // ILANG_ATTN_WAVES=4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
+  //   d == dv in {64, 128}: direct-to-LDS kernels, templated on the workgroup's query rows (64 / 128 / 256 = 2 / 4 / 8
+  //     waves) and on the key tile in LDS (32 / 64).  The schedule's tile decides when such a kernel exists.
+  //     Without a usable request: 64-key tiles, and 256 query rows (half the L2 -> LDS traffic per query) on long
+  //     key loops when that still leaves at least two workgroups per CU and does not pad nq by much, else 128.
+  //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512 x 32): the
+  //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs.
+  //   otherwise: register-staged kernel with guarded columns (always multiplies the scores in f32)
+  // ILANG_ATTN_WAVES=2|4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
   // d == 64 only) and ILANG_ATTN_NO_DIRECT=1 forces the register-staged kernel; both exist so that tests can
   // reach every kernel with small inputs.
-  unsigned bm = 128;
+  unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
   const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct) {
-    if (query_tile == 128 || query_tile == 256) bm = (unsigned)query_tile;  // the schedule's i split
-    else if (d == 64 && (query_tile == 512 || (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256 &&
-                                               10 * ((nq + 511) / 512 * 512) <= 11 * ((nq + 127) / 128 * 128))))
+    const bool tile_known = query_tile == 64 || query_tile == 128 || query_tile == 256;
+    if (key_tile == 32 && !options.f32_scale && tile_known && !(d == 64 && query_tile == 256)) bn = 32;
+    if (tile_known && !(options.f32_scale && query_tile == 64)) bm = (unsigned)query_tile;  // the schedule's i split
+    else if (d == 64 && !options.f32_scale &&
+             ((query_tile == 512 && (key_tile == 32 || key_tile == 0)) ||
+              (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256 &&
+               10 * ((nq + 511) / 512 * 512) <= 11 * ((nq + 127) / 128 * 128))))
       q64 = true;
     else if (bh * ((nq + 255) / 256) >= 2 * 256 && nk >= 2560 &&
              10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128))
@@ -61,13 +66,15 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
                  // than 10 % of idle query rows
     if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
       const int waves = std::atoi(w);
-      q64 = waves == 64 && d == 64;
+      q64 = waves == 64 && d == 64 && !options.f32_scale;
       if (!q64) {
-        if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8 (or 64 for d = 64)";
+        if (waves != 2 && waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 2, 4 or 8 (or 64 for d = 64)";
         bm = 32u * (unsigned)waves;
+        if (options.f32_scale && bm == 64) bm = 128;
+        if (d == 64 && bm == 256) bn = 64;
       }
     }
-    if (q64) bm = 512;
+    if (q64) { bm = 512; bn = 32; }
   }
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o;
@@ -77,23 +84,31 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.scale_ptr = scale_ptr;
   p.scale_value = scale;
 
-  const char* name;
+  std::string name;
+  unsigned threads = 2 * bm;  // one query per lane of a half-wave: 32 queries per wave
   if (in_dtype == BF16) {
-    if (direct && q64) name = "attn_fwd_bf16_d64_bn32_q64";
-    else if (direct)
-      name = d == 64 ? (bm == 256 ? "attn_fwd_bf16_d64_bn64_direct_w8" : "attn_fwd_bf16_d64_bn64_direct")
-                     : (bm == 256 ? "attn_fwd_bf16_d128_bn64_direct_w8" : "attn_fwd_bf16_d128_bn64_direct");
-    else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
+    if (direct && q64) {
+      name = "attn_fwd_bf16_d64_bn32_q64";
+      threads = bm;
+    } else if (direct) {
+      name = "attn_fwd_bf16_d" + std::to_string(d) + "_bn" + std::to_string(bn) + "_direct";
+      if (bm == 64) name += "_w2";
+      if (bm == 256) name += "_w8";
+      if (options.f32_scale) name += "_f32scale";
+    } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
+  } else {
+    name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
+    bn = 32;
   }
-  else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
+  if (note) *note = LaunchNote{name, bm, bn};
 
   const size_t groups = (bh + 7) / 8 * 8;  // heads padded to the XCD count
   const size_t grid = groups * p.nqt;
   if (grid > kMaxGrid) return "attention kernel: grid too large";
   hipFunction_t fn;
-  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, 1, 1, q64 ? bm : 2 * bm, &p, sizeof(p), stream);
+  if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
+  return launch(fn, (unsigned)grid, 1, 1, threads, &p, sizeof(p), stream);
 }
 
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }
@@ -110,7 +125,7 @@ static unsigned pick_direct_tile(size_t t256, size_t t128) {
 }
 
 Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n) {
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note) {
   if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || !fits_u32(k) || !fits_u32(bh)) return "gemm_nt kernel: extent exceeds 32 bits";
@@ -140,9 +155,9 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
       const size_t grid = ((nsb + 7) / 8 * 8) * 32;
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
-      if (Err e = builtin_function(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct", &fn);
-          !e.empty())
-        return e;
+      const char* name = tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct";
+      if (note) *note = LaunchNote{name, tile, tile};
+      if (Err e = builtin_function(name, &fn); !e.empty()) return e;
       return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
     }
   }
@@ -152,6 +167,7 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   const size_t grid = ((tiles + 7) / 8 * 8) * bh;
   if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
   hipFunction_t fn;
+  if (note) *note = LaunchNote{"gemm_nt_bf16_128x128x64", 128, 128};
   if (Err e = builtin_function("gemm_nt_bf16_128x128x64", &fn); !e.empty()) return e;
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
@@ -171,7 +187,7 @@ static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t til
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return gemm_nn_tile(bh, m, n, k, 0, 0) != 0; }
 
 Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n) {
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note) {
   const unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
   if (tile == 0) return "gemm_nn kernel: needs k % 64 == 0 and n % 8 == 0 (and extents within its offset range)";
   if (bh == 0 || m == 0 || n == 0) return {};
@@ -185,15 +201,16 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_
   const size_t grid = ((nsb + 7) / 8 * 8) * 32;
   if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
   hipFunction_t fn;
-  if (Err e = builtin_function(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct", &fn); !e.empty())
-    return e;
+  const char* name = tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct";
+  if (note) *note = LaunchNote{name, tile, tile};
+  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 32 == 0 && k <= (size_t(1) << 21); }
 
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                       hipStream_t stream) {
+                       hipStream_t stream, LaunchNote* note) {
   if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 32 (at most 2^21)";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || bh > 65535) return "gemm_nt f32 kernel: extent too large";
@@ -211,13 +228,14 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   const size_t grid = ((nsb + 7) / 8 * 8) * 32;
   if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
   hipFunction_t fn;
-  if (Err e = builtin_function(tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct", &fn);
-      !e.empty())
-    return e;
+  const char* name = tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct";
+  if (note) *note = LaunchNote{name, tile, tile};
+  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 
-Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode) {
+Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode,
+                       LaunchNote* note) {
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
@@ -230,12 +248,14 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
     while ((size_t)256 * nv < cols) nv *= 2;
     const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
     const std::string name = std::string("row_") + kOps[mode] + "_wave_" + (vec ? "v" : "s") + std::to_string(nv);
+    if (note) *note = LaunchNote{name, 0, 0};
     if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
     const size_t grid = (rows + 3) / 4;  // four wavefronts (rows) per workgroup
     if (grid > kMaxGrid) return "row_softmax kernel: grid too large";
     return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
   }
   if (rows > kMaxGrid) return "row_softmax kernel: grid too large";
+  if (note) *note = LaunchNote{std::string("row_") + kOps[mode] + "_block", 0, 0};
   if (Err e = builtin_function((std::string("row_") + kOps[mode] + "_block").c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
 }

@@ -3,6 +3,7 @@
 // kernel variant, and enqueue it on `stream`.  All pointers are device memory.
 #pragma once
 #include <cstddef>
+#include <string>
 
 #include "hip_rt.h"
 
@@ -10,38 +11,53 @@ namespace ihip {
 
 enum DType { F32 = 0, BF16 = 1 };
 
+// What a launcher did with a request: the kernel it enqueued and, for tiled kernels, the workgroup tile that kernel
+// works on, so that callers can report a schedule tile that no kernel has.
+struct LaunchNote {
+  std::string kernel;         // name in the code object
+  size_t tile_i = 0, tile_j = 0;  // rows x columns (attention: query rows x keys) per workgroup step
+};
+
 // o[bh,nq,dv] = softmax(s * q[bh,nq,d] k[bh,nk,d]^T) v[bh,nk,dv],  s = scale * (scale_ptr ? *scale_ptr : 1)
 // in_dtype applies to q, k, v; out_dtype to o (F32 or BF16; BF16 only with bf16 inputs).
 // scale_ptr, when given, is a rank-0 f32 operand in device memory, read by the kernel.
-// query_tile is the query-row tile the schedule asks for (the product of the split factors of the row
-// index; 0 = no preference): 128 and 256 select the 4- and 8-wave workgroup of the direct-to-LDS kernel, any other
-// value leaves the choice to the launcher.
+// query_tile x key_tile is the tile the schedule asks for (the products of the split factors of the row and of
+// the key index; 0 = no preference).  The direct-to-LDS kernels (bf16, d == dv in {64, 128}) exist for
+// query tiles 64 / 128 / 256 (2, 4, 8 waves) with key tiles 32 / 64 (no 256 x 32 at d = 64), and for 512 x 32 at
+// d = 64 (64 queries per wave); any other request leaves the choice to the launcher's size heuristic.
+// f32_scale: apply the score scale in f32 to every score, as the reference does, instead of folding it into Q
+// with one more bf16 rounding (direct kernels only; the other kernels always multiply in f32).
+struct AttentionOptions {
+  size_t query_tile = 0, key_tile = 0;
+  bool f32_scale = false;
+};
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
-                     size_t query_tile = 0);
+                     const AttentionOptions& options = {}, LaunchNote* note = nullptr);
 bool attention_supported(DType in_dtype, size_t d, size_t dv);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,n,k]^T, a and b bf16
 // tile_m x tile_n is the output tile the schedule asks for (0 = no preference): 256 x 256 and 128 x 128 select
 // the kernel with that workgroup tile (when its requirements hold), anything else leaves the choice to the launcher.
 Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr);
 bool gemm_nt_bf16_supported(size_t k);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
 // Needs k % 64 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
 Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0);
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr);
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
 
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 32 == 0
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                       hipStream_t stream);
+                       hipStream_t stream, LaunchNote* note = nullptr);
 bool gemm_nt_f32_supported(size_t k);
 
 // y[rows,cols] = row softmax of x, f32
 // mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize); 3: y = exp(x)
-Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0);
+Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0,
+                       LaunchNote* note = nullptr);
 
 // dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  An NN product that the direct kernels cannot read runs as transpose + NT kernel.
 Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,

@@ -296,6 +296,19 @@ class Component:
         finally:
             core.i_string_free(text)
 
+    def option(self, name, value):
+        """Sets an option of the compiled program (``i_hip_program_option``), e.g. ``"attention.f32_scale", 1``."""
+        nat.check(core.i_hip_program_option(self._compile(), name.encode(), int(value)))
+        return self
+
+    def report(self):
+        """The kernels the last run dispatched, one line per kernel of the plan (``i_hip_program_report``)."""
+        text = nat.check_ptr(core.i_hip_program_report(self._compile()))
+        try:
+            return ctypes.string_at(text).decode()
+        finally:
+            core.i_string_free(text)
+
     def _result_extents(self, program, operands):
         count = core.i_output_count(program)
         ranks = (_sz * max(count, 1))()

@@ -10,6 +10,9 @@ The referee is any callable that returns the expected outputs for the given
 inputs (torch tensors), or, when none is given, the first candidate: schedules
 never change what is computed, so every candidate must agree with it.  The
 tolerance is relative to the largest magnitude of the referee's output.
+A referee that is slow (the C the reference backend emits, on one host core)
+may cover only part of each output: `view` cuts that part out of a candidate's
+outputs before the comparison.
 
     from i_amd import Component as i
     from i_amd.search import grid, search
@@ -32,6 +35,7 @@ class Result:
     error: Optional[float]   # max |out - referee| / max |referee| over all outputs
     plan: str                # first line of the backend plan for kernel f0 (which kernel form runs)
     failure: Optional[str] = None  # compile / run error text, or "mismatch"
+    kernels: str = ""        # what the run dispatched (Component.report()): kernel names and their tiles
 
 
 def grid(**factors: Sequence) -> List[str]:
@@ -72,7 +76,7 @@ def _time_ms(torch, fn, repeats: int, warmup: int) -> float:
 
 def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Sequence, rtol: float,
            referee: Optional[Callable[..., Sequence]] = None, repeats: int = 10, warmup: int = 2,
-           out_dtype=None) -> List[Result]:
+           out_dtype=None, view: Optional[Callable] = None) -> List[Result]:
     """Run build(schedule) for every schedule on `inputs` (ROCm torch tensors).
 
     Returns one Result per schedule, fastest first; candidates that fail to compile, fail to run or
@@ -93,7 +97,9 @@ def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Seq
             comp = build(schedule)
             got = comp.exec_torch(*inputs, out_dtype=out_dtype)
             got = [got] if torch.is_tensor(got) else list(got)
-            got = [g.float() for g in got]
+            full = got
+            got = [(view(g) if view else g).float() for g in got]
+            kernels = comp.report().strip()
         except RuntimeError as e:
             results.append(Result(schedule, None, None, "", failure=str(e)))
             continue
@@ -109,11 +115,11 @@ def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Seq
                 scale = float(e.abs().max()) or 1.0
                 err = max(err, float((g - e).abs().max()) / scale)
         if not err <= rtol:  # also catches NaN
-            results.append(Result(schedule, None, err, plan, failure="mismatch"))
+            results.append(Result(schedule, None, err, plan, failure="mismatch", kernels=kernels))
             continue
-        outs = [torch.empty_like(g, dtype=out_dtype or torch.float32) for g in got]
+        outs = [torch.empty_like(g, dtype=out_dtype or torch.float32) for g in full]
         target = outs[0] if len(outs) == 1 else outs
         ms = _time_ms(torch, lambda: comp.into(target, *inputs), repeats, warmup)
-        results.append(Result(schedule, ms, err, plan))
+        results.append(Result(schedule, ms, err, plan, kernels=kernels))
     results.sort(key=lambda r: (r.failure is not None, r.ms if r.ms is not None else float("inf")))
     return results

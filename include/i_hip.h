@@ -86,6 +86,34 @@ int i_hip_attention(const void* q, const void* k, const void* v, void* o,
                     float scale, void* stream);
 
 /*
+ * i_hip_attention with the schedule spelled out: query_tile x key_tile is the workgroup tile the schedule's split
+ * factors ask for (README.md:139-163; 0 = no preference).  bf16 operands with d == dv in {64, 128} have kernels
+ * for query tiles 64 / 128 / 256 with key tiles 32 / 64 (not 256 x 32 at d = 64) and for 512 x 32 at d = 64;
+ * any other request leaves the choice to the launcher.  f32_scale != 0 applies the score scale in f32 to every
+ * score, the reference's arithmetic (compiler/src/lower/exec_plan_to_module.rs:605-640), instead of folding
+ * scale * log2(e) into Q with one more bf16 rounding: about 5 % slower, and the error against an f32 computation
+ * no longer grows with the magnitude of the scores.  f32 operands and the other bf16 kernels always multiply in f32.
+ */
+int i_hip_attention_ex(const void* q, const void* k, const void* v, void* o,
+                       int in_dtype, int out_dtype,
+                       size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
+                       float scale, size_t query_tile, size_t key_tile, int f32_scale, void* stream);
+
+/*
+ * Options of a compiled program, by name (i_compile has no options argument, core/i.h:44).  Known:
+ *   "attention.f32_scale"  0 (default) / 1: what f32_scale is to i_hip_attention_ex, for the program's attention kernels
+ * Returns 0, or -1 with the text in i_error() for an unknown name.  Takes effect from the next i_exec*.
+ */
+int i_hip_program_option(i_program* program, const char* name, int value);
+
+/*
+ * What the last i_exec* of this program dispatched, one line per kernel of the plan that i_code prints:
+ * "f0: attn_fwd_bf16_d128_bn64_direct_w8 (tile 256 x 64)"; a schedule tile that no hand-written kernel has for
+ * the operands is spelled out on that line.  Heap string, free with i_string_free; NULL + i_error on failure.
+ */
+char* i_hip_program_report(const i_program* program);
+
+/*
  * mm_t,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,n,k]  with bf16 a, b and f32 c:
  * the fused kernel for  i("ik*jk~ijk") >> i("+ijk~ij ... k0")  (README.md:16;
  * same nest as annotated-flashattn.c:57-89).  Requires k % 8 == 0.

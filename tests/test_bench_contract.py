@@ -45,7 +45,13 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert roof["bound"] == "mfma" and roof["unit"] == "TFLOP/s" and roof["peak"] == 2500.0
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9
     cpu = rec["cpu_baseline"]
-    assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    assert cpu["kind"] == "port" and cpu["form"].startswith("emitted-c") and cpu["cores"] == 1 and cpu["value"] > 0 and cpu["sample"] and cpu["host_cpu"]
+    assert rec["pre_warmup_launches"] == 41 and rec["rel_err"] <= 2e-2
+    assert rec["roofline"]["kernel"] == "attn_fwd_bf16_d128_bn64_direct_w8"
+    second = rec["secondary"]
+    assert len(second) == 4
+    for entry, bar in zip(second, (1e-4, 2e-2, 2e-2, 1e-4)):
+        assert entry["cpu_baseline"]["value"] > 0 and entry["rel_err"] <= bar, entry["workload"]
     # the value is work over wall time of exactly `steps` calls
     flop = 4.0 * 8 * 32 * 4096 * 4096 * 128
     assert abs(rec["value"] - flop / (rec["ms_per_step"] * 1e-3) / 1e12) / rec["value"] < 1e-6

@@ -331,6 +331,74 @@ def test_config5_long_sequence_slice_vs_oracle(torch):
     close(got[:, :, rows], ref, RTOL_BF16)
 
 
+def np_inputs(shape, amp=1.0):
+    """The operand recipe of the BASELINE configurations: NumPy default_rng(seed).standard_normal, seeds 1, 2, 3."""
+    return [oracle.to_bf16_f32(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(amp))
+            for seed in (1, 2, 3)]
+
+
+def test_config4_full_size_with_the_benchmark_schedule_vs_oracle(torch):
+    """B8 H32 N4096 d128 with the schedule bench.py times, i:256,j:64 (the 8-wave direct kernel), at full size:
+    four (b, h) slices, first and last 32 query rows of each (the first and the last workgroup of a head, and rows
+    of its first and last wave), against the oracle on identical inputs."""
+    B, H, N, D = 8, 32, 4096, 128
+    q, k, v = np_inputs((B, H, N, D))
+    scale = np.float32(1.0 / np.sqrt(D))
+    comp = flash("i:256,j:64", prefix="bh", scaled=True)
+    got = comp.exec_torch(torch.from_numpy(q).cuda().bfloat16(), torch.from_numpy(k).cuda().bfloat16(),
+                          torch.tensor(scale, device="cuda"), torch.from_numpy(v).cuda().bfloat16())
+    assert "attn_fwd_bf16_d128_bn64_direct_w8 (tile 256 x 64)" in comp.report()
+    rows = np.r_[0:32, N - 32:N]
+    for b, h in ((0, 0), (3, 17), (7, 31), (5, 8)):
+        ref = oracle.attention_tiled(q[b, h][rows], k[b, h], v[b, h], scale)
+        close(got[b, h][torch.from_numpy(rows).cuda()].cpu().numpy(), ref, RTOL_BF16)
+
+
+def test_config5_full_size_with_the_benchmark_schedule_vs_oracle(torch):
+    """B1 H16 N32768 d64, inputs x 2.0, with the schedule bench.py times, i:512,j:32 (64 queries per wave), on all
+    16 heads at once: three heads x first and last 32 query rows against the oracle."""
+    B, H, N, D = 1, 16, 32768, 64
+    q, k, v = np_inputs((B, H, N, D), amp=2.0)
+    scale = np.float32(1.0 / np.sqrt(D))
+    comp = flash("i:512,j:32", prefix="bh", scaled=True)
+    got = comp.exec_torch(torch.from_numpy(q).cuda().bfloat16(), torch.from_numpy(k).cuda().bfloat16(),
+                          torch.tensor(scale, device="cuda"), torch.from_numpy(v).cuda().bfloat16())
+    assert "attn_fwd_bf16_d64_bn32_q64 (tile 512 x 32)" in comp.report()
+    rows = np.r_[0:32, N - 32:N]
+    for h in (0, 7, 15):
+        ref = oracle.attention_tiled(q[0, h][rows], k[0, h], v[0, h], scale)
+        close(got[0, h][torch.from_numpy(rows).cuda()].cpu().numpy(), ref, RTOL_BF16)
+
+
+def test_schedule_tiles_reach_the_kernels_and_unknown_tiles_are_reported(torch):
+    """The i and j splits of the attention schedule select the kernel with that workgroup tile; a tile that no
+    kernel has is reported, in the plan and after the run, instead of being replaced silently."""
+    B, H, N, D = 1, 2, 640, 128
+    q, k, v = (torch.from_numpy(a).cuda().bfloat16() for a in np_inputs((B, H, N, D)))
+    sd = torch.tensor(np.float32(1.0 / np.sqrt(D)), device="cuda")
+    outs = {}
+    for ti, tj, name in ((64, 32, "d128_bn32_direct_w2"), (64, 64, "d128_bn64_direct_w2"), (128, 32, "d128_bn32_direct "),
+                         (128, 64, "d128_bn64_direct "), (256, 32, "d128_bn32_direct_w8"), (256, 64, "d128_bn64_direct_w8")):
+        comp = flash(f"i:{ti},j:{tj}", prefix="bh", scaled=True)
+        outs[ti, tj] = comp.exec_torch(q, k, sd, v)
+        assert f"attn_fwd_bf16_{name}" in comp.report() and f"(tile {ti} x {tj})" in comp.report()
+        assert "the schedule tile selects the kernel" in comp._code()
+    ref = outs[128, 64]
+    for out in outs.values():
+        assert (out - ref).abs().max() <= 2e-2 * ref.abs().max()
+    odd = flash("i:16,j:16", prefix="bh", scaled=True)
+    assert "no hand-written kernel has this tile" in odd._code()
+    odd.exec_torch(q, k, sd, v)
+    assert "the schedule asks for 16 x 16, which no hand-written kernel has" in odd.report()
+    # the f32-scale form is a program option
+    precise = flash("i:256,j:64", prefix="bh", scaled=True).option("attention.f32_scale", 1)
+    out = precise.exec_torch(q, k, sd, v)
+    assert "attn_fwd_bf16_d128_bn64_direct_w8_f32scale" in precise.report()
+    assert (out - ref).abs().max() <= 2e-2 * ref.abs().max()
+    with pytest.raises(RuntimeError):
+        precise.option("no.such.option", 1)
+
+
 def test_rescale_stress_max_in_last_tile(torch):
     # every key tile raises the running max of every row
     nq, nk, d = 100, 700, 16

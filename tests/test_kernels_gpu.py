@@ -67,6 +67,22 @@ def gpu_attention(env, q, k, v, scale, bf16, out_bf16=False):
     return od.float().cpu().numpy()
 
 
+def gpu_attention_ex(env, q, k, v, scale, query_tile=0, key_tile=0, f32_scale=False):
+    """bf16 operands, f32 output, through i_hip_attention_ex (the schedule's tile and the scale mode spelled out)."""
+    t = env.torch
+    lead = q.shape[:-2]
+    bh = int(np.prod(lead)) if lead else 1
+    nq, d = q.shape[-2:]
+    nk, dv = v.shape[-2:]
+    qd, kd, vd = (t.from_numpy(a).cuda().to(t.bfloat16).contiguous() for a in (q, k, v))
+    od = t.full(lead + (nq, dv), float("nan"), device="cuda", dtype=t.float32)
+    env.nat.check(env.nat.core.i_hip_attention_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), od.data_ptr(), env.nat.BF16,
+                                                  env.nat.F32, bh, nq, nk, d, dv, scale, query_tile, key_tile,
+                                                  int(f32_scale), env.stream()))
+    t.cuda.synchronize()
+    return od.cpu().numpy()
+
+
 # ------------------------------------------------------------------ attention, f32
 @pytest.mark.parametrize("case", ["u_48x24", "u_64x64", "u_100x40", "n_48x24", "n_33x17"])
 def test_attention_f32_vs_reference_golden(env, golden, case):
@@ -221,6 +237,39 @@ def test_attention_bf16_large_scores_error_growth(env, monkeypatch, d, waves):
         got = gpu_attention(env, q, k, v, scale, bf16=True)
         err = np.abs(got - ref).max() / np.abs(ref).max()
         assert err <= bound, f"inputs x {amp}: error {err} > {bound}"
+
+
+@pytest.mark.parametrize("d,tile", [(128, 128), (128, 256), (64, 128), (64, 256)])
+def test_attention_bf16_f32_scale_keeps_the_bar_at_any_score_magnitude(env, d, tile):
+    """f32_scale: the score scale multiplies every score in f32 (the reference's arithmetic) and Q is not rounded a
+    second time.  Same inputs as above, x 1, x 2 and x 3: the error stays inside the 2e-2 bar, and does not grow
+    with the magnitude of the scores the way the folded form's does."""
+    bh, nq, nk = 2, 200, 1100
+    for amp in (1.0, 2.0, 3.0):
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s) * np.float32(amp)) for s, n in ((1, nq), (2, nk), (3, nk)))
+        scale = float(np.float32(1.0 / np.sqrt(d)))
+        s = np.einsum("bik,bjk->bij", q.astype(np.float64), k.astype(np.float64)) * scale
+        p = np.exp(s - s.max(axis=-1, keepdims=True))
+        ref = np.einsum("bij,bjk->bik", p / p.sum(axis=-1, keepdims=True), v.astype(np.float64))
+        got = gpu_attention_ex(env, q, k, v, scale, query_tile=tile, key_tile=64, f32_scale=True)
+        err = np.abs(got - ref).max() / np.abs(ref).max()
+        assert err <= 1e-2, f"inputs x {amp}: error {err}"
+
+
+@pytest.mark.parametrize("d,query_tile,key_tile", [(128, 64, 64), (128, 64, 32), (128, 128, 32), (128, 256, 32),
+                                                   (128, 128, 64), (128, 256, 64), (64, 64, 64), (64, 64, 32),
+                                                   (64, 128, 32), (64, 128, 64), (64, 256, 64), (64, 512, 32)])
+@pytest.mark.parametrize("f32_scale", [False, True])
+def test_attention_bf16_every_schedule_tile_vs_oracle(env, d, query_tile, key_tile, f32_scale):
+    """Every (query tile, key tile) kernel of the direct-to-LDS family, and the f32-scale form of the tiles that
+    have one, on a ragged problem long enough for the steady-state loop (9 full 64-key tiles + 10 keys), a second
+    problem that is too short for it, and one with a single query and a single key."""
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    for nq, nk in ((300, 9 * 64 + 10), (70, 100), (1, 1)):
+        q, k, v = (oracle.to_bf16_f32(rnd((3, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        got = gpu_attention_ex(env, q, k, v, scale, query_tile, key_tile, f32_scale)
+        assert_close(got, ref, RTOL_BF16)
 
 
 @pytest.mark.parametrize("q64", [False, True])

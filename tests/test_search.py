@@ -46,3 +46,47 @@ def test_search_ranks_schedules_and_flags_failures():
     # without a referee the first candidate that runs is the reference
     again = search(mm_t, ["i:128,j:128", "i:256,j:256"], inputs=(a, b), rtol=2e-2, repeats=3)
     assert all(r.failure is None for r in again)
+
+
+@pytest.mark.gpu
+def test_search_over_attention_tiles_with_the_emitted_c_as_referee():
+    """B8 H32 N4096 d128 (the benchmark's shape): every (query tile, key tile) kernel is a point of the search, the
+    referee is the C the reference backend would emit for the component, run on the host for 64 query rows of one
+    (b, h) slice."""
+    import torch
+
+    from i_amd import I
+
+    B, H, N, D = 8, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q, k, v = (torch.randn(B, H, N, D, device="cuda", generator=g).bfloat16() for _ in range(3))
+    scale = torch.tensor(np.float32(1.0 / np.sqrt(D)), device="cuda")
+
+    def attn(split):
+        p = "bh"
+        mm_t = i(f"{p}ik*{p}jk~{p}ijk | {split} | {p}jii'j'k") >> i(f"+{p}ijk~{p}ij | {split} | {p}jii'j'k0")
+        sc = i(f"{p}ij*.~{p}ij | {split} | {p}ji0i'j'")
+        shift = (I & i(f">{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij-{p}i~{p}ij | {split} | {p}ji01i'j'")
+        ex = i(f"^{p}ij~{p}ij | {split} | {p}ji0i'j'")
+        norm = (I & i(f"+{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij/{p}i~{p}ij | {split} | {p}ji01i'j'")
+        mm = i(f"{p}ij*{p}jk~{p}ikj | {split} | {p}ji0i'kj'") >> i(f"+{p}ikj~{p}ik | {split} | {p}jii'kj'0")
+        return mm_t >> sc >> shift >> ex >> norm >> mm
+
+    b0, h0, rows = 5, 19, slice(4000, 4064)
+
+    def referee(q_, k_, s_, v_):
+        cpu = [t[b0:b0 + 1, h0:h0 + 1].float().cpu().numpy() for t in (q_, k_, v_)]
+        demo_tiles = attn("i:16,j:16")  # owns the handle while the C is emitted; the emitted nest is shape-generic
+        prog = oracle.compile_component(demo_tiles.handle)
+        out = prog.run(np.ascontiguousarray(cpu[0][:, :, rows]), cpu[1], np.float32(s_.item()), cpu[2])
+        return torch.from_numpy(out).cuda()
+
+    ranked = search(attn, grid(i=[64, 128, 256], j=[32, 64]) + ["i:16,j:16"], inputs=(q, k, scale, v), rtol=2e-2,
+                    referee=referee, repeats=5, view=lambda o: o[b0:b0 + 1, h0:h0 + 1, rows])
+    assert all(r.failure is None for r in ranked), [(r.schedule, r.failure, r.error) for r in ranked]
+    names = {r.kernels.split()[1] for r in ranked}
+    assert len(names) >= 6, names
+    assert ranked == sorted(ranked, key=lambda r: r.ms)
+    by = {r.schedule: r for r in ranked}
+    assert "the schedule asks for 16 x 16" in by["i:16,j:16"].kernels
+    assert by["i:256,j:64"].ms < by["i:64,j:32"].ms  # one workgroup per CU with 64-key tiles beats 64-query workgroups
