@@ -87,17 +87,29 @@ def measured_traffic(summary):
 
 def time_steps(torch, fn, steps, warmup):
     """Wall time per step over exactly `steps` calls, and the average launch duration from one pair of events
-    on the launch stream around the timed region (the launches queue back to back on the stream)."""
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    for _ in range(steps):
-        fn()
-    end.record()
-    torch.cuda.synchronize()
+    on the launch stream around the timed region (the launches queue back to back on the stream).
+
+    Python's cyclic garbage collector is switched off for the duration: a full collection in a process that has
+    imported torch pauses the host for 30-40 ms, and when that falls into a window of 200 launches of a 0.1 ms
+    kernel the stream runs dry and the window reads twice its real time (seen as 0.2-0.26 ms for mm_t 4096^3
+    and row softmax, always at the same launch count)."""
+    import gc
+
+    gc.collect()
+    gc.disable()
+    try:
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        start.record()
+        for _ in range(steps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+    finally:
+        gc.enable()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     kernel_ms = start.elapsed_time(end) / steps
     return wall_ms, kernel_ms
@@ -164,9 +176,24 @@ def main():
     def to_dev_bf16(a):
         return torch.from_numpy(a).to(dev).bfloat16()
 
-    # ------------------------------------------------------------------ headline: attention B8 H32 N4096 d128
+    import oracle  # the CPU side of the checks at the end (and bf16 rounding of host data); never on a timed path
+
+    # All operands are generated on the host and moved to HBM before anything is timed: seconds of host-only work
+    # between two timed regions would let the device clock down, and the kernels timed next would read slow.
     B, H, N, D = 8, 32, 4096, 128
     q, k, v = (to_dev_bf16(normal((B, H, N, D), seed)) for seed in (1, 2, 3))
+    rows, cols = 16384, 4096
+    xs = [torch.from_numpy(normal((rows, cols), seed)).to(dev) for seed in (1, 11, 12, 13)]
+    M = 4096
+    a_host = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (M, M)).astype(np.float32))
+    b_host = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (M, M)).astype(np.float32))
+    a, b = to_dev_bf16(a_host), to_dev_bf16(b_host)
+    B5, H5, N5, D5 = 1, 16, 32768, 64
+    q5, k5, v5 = (to_dev_bf16(normal((B5, H5, N5, D5), seed, 2.0)) for seed in (1, 2, 3))
+    demo_in = [np.random.default_rng(sd).uniform(-1, 1, (512, 64)).astype(np.float32) for sd in (1, 2, 3)]
+    dq, dk, dv_ = (torch.from_numpy(t).to(dev) for t in demo_in)
+
+    # ------------------------------------------------------------------ headline: attention B8 H32 N4096 d128
     scale = torch.tensor(np.float32(1.0 / np.sqrt(D)), dtype=torch.float32, device=dev)
     out = torch.empty(B, H, N, D, dtype=torch.float32, device=dev)
     attn = flash_component(i, I, "i:256,j:64")
@@ -189,15 +216,13 @@ def main():
     attn.into(out, q, k, scale, v)  # leave the seeded result in `out` for the parity check below
 
     # ------------------------------------------------------------------ row softmax [16384, 4096] f32 (HBM bound)
-    rows, cols = 16384, 4096
-    x = torch.from_numpy(normal((rows, cols), 1)).to(dev)
+    x = xs[0]
     y = torch.empty_like(x)
     sm = softmax_component(i, I)
     sm.into(y, x)
     sm_kernel = sm.report().split()[1]
     # The timed calls walk four input/output pairs (2 GiB): one pair alone (512 MiB) would be re-read partly out of
     # the 256 MiB Infinity Cache from one step to the next, and that is not HBM bandwidth.
-    xs = [x] + [torch.from_numpy(normal((rows, cols), 10 + n)).to(dev) for n in range(3)]
     ys = [y] + [torch.empty_like(x) for _ in range(3)]
     turn = [0]
 
@@ -216,12 +241,6 @@ def main():
     sm_gbs = sm_bytes / (sm_ms * 1e-3) / 1e9
 
     # ------------------------------------------------------------------ mm_t 4096^3 bf16 (MFMA bound)
-    import oracle  # the CPU side of the checks below; never on the timed path
-
-    M = 4096
-    a_host = oracle.to_bf16_f32(np.random.default_rng(1).uniform(-1, 1, (M, M)).astype(np.float32))
-    b_host = oracle.to_bf16_f32(np.random.default_rng(2).uniform(-1, 1, (M, M)).astype(np.float32))
-    a, b = to_dev_bf16(a_host), to_dev_bf16(b_host)
     c = torch.empty(M, M, device=dev)
     mm = mm_t_component(i)
     mm.into(c, a, b)
@@ -230,8 +249,6 @@ def main():
     mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
 
     # ------------------------------------------------------------------ long-sequence attention B1 H16 N32768 d64, x 2.0
-    B5, H5, N5, D5 = 1, 16, 32768, 64
-    q5, k5, v5 = (to_dev_bf16(normal((B5, H5, N5, D5), seed, 2.0)) for seed in (1, 2, 3))
     scale5 = torch.tensor(np.float32(1.0 / np.sqrt(D5)), dtype=torch.float32, device=dev)
     out5 = torch.empty(B5, H5, N5, D5, dtype=torch.float32, device=dev)
     attn5 = flash_component(i, I, "i:512,j:32")  # 512 query rows per workgroup, 32-key LDS tiles: the d = 64 kernel
@@ -244,13 +261,11 @@ def main():
     # (BASELINE configs[0]): no scale, i:16,j:16, through the f32 kernel.  Timed here, with the other GPU work and
     # before the host legs below: after seconds of CPU-only work the device has clocked down, and a 70 us kernel
     # timed then reads ten times slower.
-    demo_in = [np.random.default_rng(sd).uniform(-1, 1, (512, 64)).astype(np.float32) for sd in (1, 2, 3)]
     demo = flash_demo_component(i, I)
-    dq, dk, dv_ = (torch.from_numpy(t).to(dev) for t in demo_in)
     dout = torch.empty(512, 64, device=dev)
     demo.into(dout, dq, dk, dv_)
     c1_kernel = demo.report().split()[1]
-    _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), 200, 50)
+    _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), short_steps, short_warmup)
     c1_flop = 4.0 * 512 * 512 * 64
 
     if args.calibrate_copy:
@@ -327,9 +342,11 @@ def main():
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
              "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),
+             "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu2, "rel_err": err2},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
              "roofline": roof("mfma", mm_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_nt_4096x4096x4096_bf16.md", mm_kernel, mm_ms),
+             "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu3, "rel_err": err3},
             {"workload": "flash_attention_fwd B1 H16 N32768 d64, bf16 inputs x 2.0 (BASELINE configs[4])",
              "schedule": "i:512,j:32 (512 query rows per workgroup, 64 per wave; 32-key LDS tiles)",
@@ -339,6 +356,7 @@ def main():
              "cpu_baseline": cpu5, "rel_err": err5},
             {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,
+             "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu1, "rel_err": err1},
         ],
     }
