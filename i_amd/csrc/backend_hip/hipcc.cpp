@@ -57,6 +57,52 @@ std::string hipcc_path() {
   return "hipcc";
 }
 
+// The on-disk cache of code objects: a directory that belongs to this user alone ($XDG_CACHE_HOME/ilang_hip or
+// ~/.cache/ilang_hip, else <tmp>/ilang_hip_cache-<uid>), created 0700 and refused when somebody else owns it or
+// others may write to it: what is found there is loaded and run on the GPU.  "" when no usable directory exists.
+std::string private_cache_dir() {
+  std::string dir;
+  if (const char* x = std::getenv("XDG_CACHE_HOME"); x && *x) dir = std::string(x) + "/ilang_hip";
+  else if (const char* h = std::getenv("HOME"); h && *h) {
+    const std::string base = std::string(h) + "/.cache";
+    mkdir(base.c_str(), 0700);  // may exist
+    dir = base + "/ilang_hip";
+  } else {
+    dir = tmp_dir() + "/ilang_hip_cache-" + std::to_string((unsigned long)getuid());
+  }
+  if (mkdir(dir.c_str(), 0700) != 0 && errno != EEXIST) {
+    dir = tmp_dir() + "/ilang_hip_cache-" + std::to_string((unsigned long)getuid());
+    if (mkdir(dir.c_str(), 0700) != 0 && errno != EEXIST) return {};
+  }
+  struct stat st;
+  if (lstat(dir.c_str(), &st) != 0 || !S_ISDIR(st.st_mode) || st.st_uid != getuid() || (st.st_mode & 022) != 0) return {};
+  return dir;
+}
+
+// A cached image is stored behind its full source text (length, text, image): a 64-bit hash names the file, the
+// comparison of the text is what says that the image belongs to this source.
+bool read_cached(const std::string& path, const std::string& key_text, std::vector<char>* image) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) return false;
+  uint64_t n = 0;
+  f.read(reinterpret_cast<char*>(&n), sizeof n);
+  if (!f || n != key_text.size()) return false;
+  std::string text(n, '\0');
+  f.read(text.data(), (std::streamsize)n);
+  if (!f || text != key_text) return false;
+  image->assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+  return !image->empty();
+}
+
+bool write_cached(const std::string& path, const std::string& key_text, const std::vector<char>& image) {
+  std::ofstream f(path, std::ios::binary | std::ios::trunc);
+  const uint64_t n = key_text.size();
+  f.write(reinterpret_cast<const char*>(&n), sizeof n);
+  f.write(key_text.data(), (std::streamsize)n);
+  f.write(image.data(), (std::streamsize)image.size());
+  return (bool)f;
+}
+
 bool read_file(const std::string& path, std::vector<char>* out) {
   std::ifstream f(path, std::ios::binary);
   if (!f) return false;
@@ -79,11 +125,11 @@ std::string hipcc_build(const std::string& source, std::vector<char>* image) {
     }
   }
   const std::string dir = tmp_dir();
-  const std::string cache_dir = dir + "/ilang_hip_cache";
+  const std::string cache_dir = std::getenv("ILANG_NO_DISK_CACHE") == nullptr ? private_cache_dir() : std::string();
   char name[64];
   snprintf(name, sizeof name, "%016llx", (unsigned long long)key);
-  const std::string cached = cache_dir + "/" + name + ".hsaco";
-  if (std::getenv("ILANG_NO_DISK_CACHE") == nullptr && read_file(cached, image)) {
+  const std::string cached = cache_dir + "/" + name + ".hsaco.cache";
+  if (!cache_dir.empty() && read_cached(cached, key_text, image)) {
     std::lock_guard<std::mutex> lock(g_mu);
     g_cache[key] = *image;
     return {};
@@ -138,10 +184,10 @@ std::string hipcc_build(const std::string& source, std::vector<char>* image) {
   std::remove(src_path.c_str());
   std::remove(log_path.c_str());
   if (err.empty()) {
-    if (std::getenv("ILANG_NO_DISK_CACHE") == nullptr) {
-      mkdir(cache_dir.c_str(), 0700);
-      const std::string tmp = cached + "." + std::to_string(getpid());
-      if (std::rename(obj_path.c_str(), tmp.c_str()) == 0) std::rename(tmp.c_str(), cached.c_str());
+    if (!cache_dir.empty()) {
+      const std::string tmp = cached + "." + std::to_string(getpid()) + "." + std::to_string(g_counter.fetch_add(1));
+      if (write_cached(tmp, key_text, *image)) std::rename(tmp.c_str(), cached.c_str());
+      else std::remove(tmp.c_str());
     }
     std::lock_guard<std::mutex> lock(g_mu);
     g_cache[key] = *image;

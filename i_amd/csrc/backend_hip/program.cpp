@@ -330,6 +330,11 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
   Program& p = run.p;
   const GenericKernel& gk = p.generic.kernels[k];
   if (gk.name.empty()) return "kernel " + std::to_string(k) + " has no generated form";
+  // One launch per top-level loop nest (ILANG_HIP_PHASES=1 at compile time) is confined to the emulated runtime:
+  // its one run on a GPU ended in a memory fault whose cause has not been shown, so it must not reach a device.
+  if (gk.phases.size() > 1 && !ihip::runtime_is_emulated())
+    return "kernel " + std::to_string(k) + " was compiled with ILANG_HIP_PHASES=1 (one launch per loop nest), which is "
+           "restricted to the CPU emulation of the runtime; unset it and compile again";
   const size_t R = p.generic.rank;
   const size_t view_bytes = 8 + 16 * R;
   const size_t nr = std::max<size_t>(gk.n_reads, 1), nw = std::max<size_t>(gk.n_writes, 1);

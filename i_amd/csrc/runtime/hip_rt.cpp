@@ -99,6 +99,11 @@ Err launch(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
   return check(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, 0, stream, nullptr, config), "hipModuleLaunchKernel");
 }
 
+bool runtime_is_emulated() {
+  static const bool emulated = dlsym(RTLD_DEFAULT, "ilang_hip_runtime_is_emulated") != nullptr;
+  return emulated;
+}
+
 DryRun::DryRun() { ++g_dry_run; }
 DryRun::~DryRun() { --g_dry_run; }
 

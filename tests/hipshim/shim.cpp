@@ -74,6 +74,8 @@ Err static_scratch(void** ptr) {
 }  // namespace ihip
 
 extern "C" {
+// what ihip::runtime_is_emulated() looks for
+__attribute__((visibility("default"))) int ilang_hip_runtime_is_emulated = 1;
 hipError_t hipGetDevice(int* dev) {
   *dev = 0;
   return hipSuccess;

@@ -485,3 +485,24 @@ def test_non_f32_host_inputs_are_converted_like_the_reference(torch):
     assert np.array_equal(i("+ij~i").exec_numpy(x), x.sum(1).astype(np.float32))
     xt = np.asfortranarray(rnd((5, 6), 1))
     assert np.allclose(i("+ij~i").exec_numpy(xt), xt.sum(1), rtol=1e-5, atol=1e-6)
+
+
+def test_per_nest_launches_are_refused_on_a_real_device():
+    """ILANG_HIP_PHASES=1 (one launch per top-level loop nest of a generated kernel) is confined to the CPU emulation
+    of the runtime: on a device the executor refuses such a kernel before launching it."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    code = ("import torch\n"
+            "from i_amd import Component as i, I\n"
+            "c = (I & i('>ij~i|i:16,j:16|jii\\'j\\'')) >> i('ij-i~ij|i:16,j:16|1jii\\'j\\'')\n"
+            "try:\n"
+            "    c.exec_torch(torch.ones(8, 8, device='cuda'))\n"
+            "    print('RAN')\n"
+            "except RuntimeError as e:\n"
+            "    print('REFUSED' if 'restricted to the CPU emulation' in str(e) else 'OTHER: ' + str(e))\n")
+    env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_HIP_GENERATED_ONLY="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300,
+                       cwd=Path(__file__).resolve().parent.parent)
+    assert r.stdout.strip().splitlines()[-1] == "REFUSED", r.stdout + r.stderr[-1500:]
