@@ -115,6 +115,10 @@ def time_steps(torch, fn, steps, warmup):
     return wall_ms, kernel_ms
 
 
+def sm_bytes_of(rows, cols):
+    return 2.0 * rows * cols * 4  # one read and one write per element
+
+
 def host_cpu_model():
     try:
         for line in Path("/proc/cpuinfo").read_text().splitlines():
@@ -236,8 +240,25 @@ def main():
     short_steps, short_warmup = (max(args.steps, 200), max(args.warmup, 100)) if args.steps >= 20 else (args.steps, args.warmup)
     _, sm_ms = time_steps(torch, softmax_step, short_steps, short_warmup)
     sm.into(y, x)  # the parity check below reads y
-    del xs, ys
-    sm_bytes = 2.0 * rows * cols * 4
+    # the same 256 MiB as rows of 32768 columns: one workgroup of 16 wavefronts per row, the row in registers
+    wide_rows, wide_cols = 2048, 32768
+    xw, yw = [t_.view(wide_rows, wide_cols) for t_ in xs], [t_.view(wide_rows, wide_cols) for t_ in ys]
+    sm.into(yw[0], xw[0])
+    smw_kernel = sm.report().split()[1]
+
+    def wide_step():
+        k_ = turn[0] % 4
+        turn[0] += 1
+        sm.into(yw[k_], xw[k_])
+
+    _, smw_ms = time_steps(torch, wide_step, short_steps, short_warmup)
+    smw_gbs = sm_bytes_of(wide_rows, wide_cols) / (smw_ms * 1e-3) / 1e9
+    sm.into(yw[1], xw[1])
+    wide_got = yw[1][:64].cpu().numpy()   # rows 0..63 of the second buffer pair, checked on the host below
+    wide_in = xw[1][:64].cpu().numpy()
+    sm.into(y, x)
+    del xs, ys, xw, yw
+    sm_bytes = sm_bytes_of(rows, cols)
     sm_gbs = sm_bytes / (sm_ms * 1e-3) / 1e9
 
     # ------------------------------------------------------------------ mm_t 4096^3 bf16 (MFMA bound)
@@ -273,8 +294,8 @@ def main():
         torch.cuda.synchronize()
 
     # ------------------------------------------------------------------ host legs: emitted C on one core, and the checks
-    cpu = cpu2 = cpu3 = cpu5 = cpu1 = None
-    err4 = err2 = err3 = err5 = err1 = None
+    cpu = cpu2 = cpu2w = cpu3 = cpu5 = cpu1 = None
+    err4 = err2 = err2w = err3 = err5 = err1 = None
     if not args.no_cpu_baseline:
         # C4: one (b, h) slice of the workload, 1024 of its 4096 query rows (query tiles and (b, h) pairs are the
         # outermost independent loops of the emitted nest, so the rate carries over to the whole workload)
@@ -290,6 +311,9 @@ def main():
         cpu2, err2 = emitted_c_baseline(
             oracle, sm, [x[:r2].cpu().numpy()], 2.0 * r2 * cols * 4 / 1e9, "GB/s",
             f"rows 0..{r2 - 1} of {rows} (algorithmic bytes of those rows)", y[:r2].cpu().numpy())
+        cpu2w, err2w = emitted_c_baseline(
+            oracle, sm, [wide_in], sm_bytes_of(64, wide_cols) / 1e9, "GB/s",
+            f"rows 0..63 of {wide_rows} (algorithmic bytes of those rows)", wide_got)
         # C3: output tiles are independent; all of k
         m3 = M if args.cpu_full else 1024
         cpu3, err3 = emitted_c_baseline(
@@ -344,6 +368,11 @@ def main():
              "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),
              "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu2, "rel_err": err2},
+            {"workload": "row_softmax f32 [2048,32768]: the same 256 MiB as rows eight times as wide (not a BASELINE "
+                         "configuration; rows of 8192 < cols <= 65536 keep the row in the registers of one workgroup)",
+             "value": smw_gbs, "unit": "GB/s",
+             "roofline": roof("hbm", smw_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_2048x32768_f32.md", smw_kernel, smw_ms),
+             "steps": short_steps, "warmup": short_warmup, "cpu_baseline": cpu2w, "rel_err": err2w},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
              "roofline": roof("mfma", mm_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_nt_4096x4096x4096_bf16.md", mm_kernel, mm_ms),
              "steps": short_steps, "warmup": short_warmup,

@@ -91,9 +91,21 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
   extern "C" __global__ void __launch_bounds__(256) row_##OP##_wave_s##NV(SoftmaxParams p) {       \
     row_softmax_wave_body<NV, false, MODE>(p);                                                     \
   }
+// row_<op>_group_{v,s}<NV>: 8192 < cols <= 4096 * NV, one workgroup of 16 wavefronts per row, row in registers
+// (no s16: element-wise loads of 64 values per lane do not fit 128 registers; such rows take the three-pass kernel)
+#define ROW_GROUP_V(OP, MODE, NV)                                                                  \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_group_v##NV(SoftmaxParams p) {     \
+    row_softmax_group_body<NV, true, MODE>(p);                                                     \
+  }
+#define ROW_GROUP(OP, MODE, NV)                                                                    \
+  ROW_GROUP_V(OP, MODE, NV)                                                                        \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_group_s##NV(SoftmaxParams p) {     \
+    row_softmax_group_body<NV, false, MODE>(p);                                                    \
+  }
 #define ROW_OP(OP, MODE)                                                                           \
   ROW_WAVE(OP, MODE, 1) ROW_WAVE(OP, MODE, 2) ROW_WAVE(OP, MODE, 4) ROW_WAVE(OP, MODE, 8)          \
   ROW_WAVE(OP, MODE, 16) ROW_WAVE(OP, MODE, 32)                                                    \
+  ROW_GROUP(OP, MODE, 4) ROW_GROUP(OP, MODE, 8) ROW_GROUP_V(OP, MODE, 16)                           \
   extern "C" __global__ void __launch_bounds__(1024) row_##OP##_block(SoftmaxParams p) {           \
     row_softmax_block_body<MODE>(p);                                                               \
   }

@@ -118,6 +118,93 @@ __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
   }
 }
 
+// Rows of 8192 < cols <= 65536: one workgroup of 16 wavefronts owns one row, which still lives in registers
+// (NV float4 chunks per lane, cols <= 4096 * NV), so HBM again sees one read and one write per element; the row
+// max and the row sum cross the wavefronts through 16 words of LDS.
+template <int NV, bool VEC, int MODE>
+__device__ __forceinline__ void row_softmax_group_body(const SoftmaxParams& p) {
+  constexpr int NW = 16;
+  __shared__ float red[2][NW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t row = blockIdx.x;
+  const float* __restrict__ x = p.x + (size_t)row * p.cols;
+  float* __restrict__ y = p.y + (size_t)row * p.cols;
+
+  f32x4 r[NV];
+  float mx = -INFINITY;
+  const float pad = MODE == 2 ? 0.0f : -INFINITY;  // neutral for the reduction of the mode
+#pragma unroll
+  for (int t = 0; t < NV; ++t) {
+    const uint32_t col = 4u * (tid + 64 * NW * t);
+    if (VEC) {
+      if (col < p.cols) r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
+      else r[t] = f32x4{pad, pad, pad, pad};
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : pad;
+    }
+    mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
+  }
+  auto store = [&](int t, f32x4 v) {
+    const uint32_t col = 4u * (tid + 64 * NW * t);
+    if (VEC) {
+      if (col < p.cols) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(y + col));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (col + e < p.cols) y[col + e] = v[e];
+    }
+  };
+  // every lane gets the reduction over the 16 wavefronts' partial results, combined in wavefront order
+  auto across_waves = [&](float v, int slot, auto combine) {
+    if (lane == 0) red[slot][wave] = v;
+    __syncthreads();
+    float total = red[slot][0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) total = combine(total, red[slot][w]);
+    return total;
+  };
+  if constexpr (MODE == 3) {  // exp(x), elementwise
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      f32x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = fast_exp2(r[t][e] * I_LOG2_E32);
+      store(t, v);
+    }
+    return;
+  }
+  if constexpr (MODE == 2) {  // row_normalize: x / sum(x)
+    float total = 0.0f;
+#pragma unroll
+    for (int t = 0; t < NV; ++t) total += (r[t][0] + r[t][1]) + (r[t][2] + r[t][3]);
+    total = across_waves(wave_sum(total), 0, [](float a, float b) { return a + b; });
+#pragma unroll
+    for (int t = 0; t < NV; ++t) store(t, r[t] / total);
+    return;
+  }
+  mx = across_waves(wave_max(mx), 0, [](float a, float b) { return fmaxf(a, b); });
+  if constexpr (MODE == 1) {  // row_max_shift: x - max(x)
+#pragma unroll
+    for (int t = 0; t < NV; ++t) store(t, r[t] - mx);
+    return;
+  }
+  const float mb = mx * I_LOG2_E32;
+  float sum = 0.0f;
+#pragma unroll
+  for (int t = 0; t < NV; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v = fast_exp2(__builtin_fmaf(r[t][e], I_LOG2_E32, -mb));
+      r[t][e] = v;
+      sum += v;
+    }
+  sum = across_waves(wave_sum(sum), 1, [](float a, float b) { return a + b; });
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int t = 0; t < NV; ++t) store(t, r[t] * inv);
+}
+
 // Any width: one workgroup per row, three passes over the row (max, sum, write).
 template <int MODE>
 __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {

@@ -255,6 +255,15 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
     return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
   }
   if (rows > kMaxGrid) return "row_softmax kernel: grid too large";
+  const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+  if (cols <= 32768 || (cols <= 65536 && vec)) {
+    // the row still fits the registers of one workgroup of 16 wavefronts: one read and one write per element
+    const int nv = cols <= 16384 ? 4 : cols <= 32768 ? 8 : 16;
+    const std::string name = std::string("row_") + kOps[mode] + "_group_" + (vec ? "v" : "s") + std::to_string(nv);
+    if (note) *note = LaunchNote{name, 0, 0};
+    if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
+    return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
+  }
   if (note) *note = LaunchNote{std::string("row_") + kOps[mode] + "_block", 0, 0};
   if (Err e = builtin_function((std::string("row_") + kOps[mode] + "_block").c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);

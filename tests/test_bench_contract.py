@@ -49,8 +49,8 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert rec["pre_warmup_launches"] == 41 and rec["rel_err"] <= 2e-2
     assert rec["roofline"]["kernel"] == "attn_fwd_bf16_d128_bn64_direct_w8"
     second = rec["secondary"]
-    assert len(second) == 4
-    for entry, bar in zip(second, (1e-4, 2e-2, 2e-2, 1e-4)):
+    assert len(second) == 5
+    for entry, bar in zip(second, (1e-4, 1e-4, 2e-2, 2e-2, 1e-4)):
         assert entry["cpu_baseline"]["value"] > 0 and entry["rel_err"] <= bar, entry["workload"]
     # the value is work over wall time of exactly `steps` calls
     flop = 4.0 * 8 * 32 * 4096 * 4096 * 128

@@ -260,6 +260,21 @@ def test_row_max_shift_and_row_normalize_kernels(torch, rows, cols):
     close(softmax_naive().exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
 
 
+def test_wide_rows_through_the_naive_and_the_row_staged_schedules(torch):
+    """Rows wider than 8192: the fused softmax and the three row kernels of the naive schedule all keep the row in the
+    registers of one workgroup; the report names the kernels."""
+    x = rnd((6, 20000), 4)
+    fused = softmax_rowstaged()
+    close(fused.exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
+    assert "row_softmax_group_v8" in fused.report()
+    three = softmax_naive()
+    close(three.exec_numpy(x), oracle.row_softmax(x), RTOL_F32)
+    assert all(name in three.report() for name in ("row_shift_group_v8", "row_exp_group_v8", "row_norm_group_v8"))
+    ragged = rnd((3, 9001), 5)  # cols % 4 != 0: element-wise loads
+    close(three.exec_numpy(ragged), oracle.row_softmax(ragged), RTOL_F32)
+    assert "row_shift_group_s4" in three.report()
+
+
 def test_naive_attention_uses_both_gemm_forms(torch):
     """The reference's naive attention (flash-attn.py:57-65): mm_t and mm on the MFMA kernels, the rest generated."""
     q, k, v = rnd((96, 64), 1), rnd((96, 64), 2), rnd((96, 64), 3)

@@ -455,7 +455,9 @@ def test_gemm_nt_bf16_full_size_linearity(env):
 
 
 # ------------------------------------------------------------------ row softmax
-@pytest.mark.parametrize("rows,cols", [(16, 8), (1, 1), (33, 1000), (64, 4096), (7, 4099), (5, 8192), (3, 20000)])
+@pytest.mark.parametrize("rows,cols", [(16, 8), (1, 1), (33, 1000), (64, 4096), (7, 4099), (5, 8192), (3, 20000),
+                                       (5, 8196), (4, 16384), (3, 16390), (3, 32768), (2, 40001), (3, 65536), (2, 65538),
+                                       (2, 100000)])
 def test_row_softmax_vs_oracle(env, rows, cols):
     t = env.torch
     x = rnd((rows, cols), 1) * 2
@@ -464,6 +466,22 @@ def test_row_softmax_vs_oracle(env, rows, cols):
     env.nat.check(env.nat.core.i_hip_row_softmax(xd.data_ptr(), yd.data_ptr(), rows, cols, env.stream()))
     t.cuda.synchronize()
     assert_close(yd.cpu().numpy(), oracle.row_softmax(x), RTOL_F32)
+
+
+def test_row_softmax_wide_rows_stay_in_registers(env):
+    """8192 < cols <= 65536: one workgroup per row with the row in registers (one read, one write per element);
+    [2048, 32768] is the same 256 MiB as the benchmark's [16384, 4096]: rows sum to 1 and sampled rows match the
+    oracle.  The three row operations of the naive schedule take the same kernels (checked through the frontend)."""
+    t = env.torch
+    rows, cols = 2048, 32768
+    x = rnd((rows, cols), 1)
+    xd = t.from_numpy(x).cuda()
+    yd = t.full_like(xd, float("nan"))
+    env.nat.check(env.nat.core.i_hip_row_softmax(xd.data_ptr(), yd.data_ptr(), rows, cols, env.stream()))
+    t.cuda.synchronize()
+    assert float((yd.sum(dim=1) - 1).abs().max()) < 1e-4
+    pick = [0, 1, 1023, 2047]
+    assert_close(yd[pick].cpu().numpy(), oracle.row_softmax(x[pick]), RTOL_F32)
 
 
 def test_row_softmax_full_size_properties(env):
