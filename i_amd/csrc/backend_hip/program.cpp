@@ -132,6 +132,18 @@ struct Run {
 };
 
 // ---------------------------------------------------------------- hand-written kernels
+// Head sizes beyond the fused attention kernels (d or dv above 128; the reference's demo uses 2048,
+// ilang-python/flash-attn.py:31-36) run as three hand-written kernels with the score matrix in memory:
+// S = Q K^T (MFMA GEMM), P = softmax(scale * S) row by row in place, O = P V (MFMA GEMM).  What the GEMM kernels
+// need of the extents decides whether that is possible; the score matrix may take up to 16 GiB.
+bool attention_in_parts_usable(DType t, size_t bh, size_t nq, size_t nk, size_t d, size_t dv) {
+  if (bh == 0 || nq == 0 || nk == 0 || d == 0 || dv == 0) return false;
+  if (bh > 65535 || (bh * nq) > 0x7fffffffull || nk > 0xffffffffull) return false;
+  if (bh * nq * nk > (size_t(4) << 30)) return false;  // f32 elements: 16 GiB
+  if (t == DType::F32) return ihip::gemm_nt_f32_supported(d) && ihip::gemm_nt_f32_supported(nk);
+  return ihip::gemm_nt_bf16_supported(d) && ihip::gemm_nt_bf16_supported(nk);
+}
+
 // Returns true when kernel k can run on its hand-written form with these operands.
 bool hand_usable(const Run& run, const Recognized& r) {
   // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
@@ -145,7 +157,12 @@ bool hand_usable(const Run& run, const Recognized& r) {
       if (run.dtype_of(r.b.buffer) != t || run.dtype_of(r.c.buffer) != t) return false;
       const auto q = rows_cols(r.a), v = rows_cols(r.c);
       if (q.size() < 2 || v.size() < 2) return false;
-      return ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back());
+      if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back())) return true;
+      const auto k = rows_cols(r.b);
+      if (k.size() < 2) return false;
+      size_t bh = 1;
+      for (size_t d = 0; d + 2 < q.size(); ++d) bh *= q[d];
+      return attention_in_parts_usable(t, bh, q[q.size() - 2], k[k.size() - 2], q.back(), v.back());
     }
     case Recognized::GemmNT: {
       const DType t = run.dtype_of(r.a.buffer);
@@ -197,6 +214,50 @@ std::string describe_launch(const ihip::LaunchNote& note, const Recognized& r) {
   return text;
 }
 
+ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
+                             const float* scale_ptr, ihip::LaunchNote* note) {
+  void* out = nullptr;
+  if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+  void* scores = nullptr;  // [bh, nq, nk] f32: S, then P in place
+  if (ihip::Err e = run.alloc(&scores, bh * nq * nk * 4); !e.empty()) return e;
+  float* s = static_cast<float*>(scores);
+  const void *q = run.raw_ptr(r.a.buffer), *k = run.raw_ptr(r.b.buffer), *v = run.raw_ptr(r.c.buffer);
+  ihip::LaunchNote first, middle, last;
+  if (ihip::Err e = bf16 ? ihip::launch_gemm_nt_bf16(q, k, s, bh, nq, nk, d, run.stream, 0, 0, &first)
+                         : ihip::launch_gemm_nt_f32(static_cast<const float*>(q), static_cast<const float*>(k), s, bh, nq, nk,
+                                                    d, run.stream, &first);
+      !e.empty())
+    return e;
+  if (ihip::Err e = ihip::launch_row_softmax(s, s, bh * nq, nk, run.stream, 4, &middle, scale_ptr, 1.0f); !e.empty()) return e;
+  if (bf16) {
+    void* pb = nullptr;  // the probabilities rounded to bf16, as the fused kernels round them
+    if (ihip::Err e = run.alloc(&pb, bh * nq * nk * 2); !e.empty()) return e;
+    if (ihip::Err e = ihip::launch_convert(s, pb, ihip::F32, ihip::BF16, bh * nq * nk, run.stream); !e.empty()) return e;
+    if (ihip::gemm_nn_bf16_supported(bh, nq, dv, nk)) {
+      if (ihip::Err e = ihip::launch_gemm_nn_bf16(pb, v, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last);
+          !e.empty())
+        return e;
+    } else {
+      void* vt = nullptr;
+      if (ihip::Err e = run.alloc(&vt, bh * dv * nk * 2); !e.empty()) return e;
+      if (ihip::Err e = ihip::launch_transpose(v, vt, bh, nk, dv, 2, run.stream); !e.empty()) return e;
+      if (ihip::Err e = ihip::launch_gemm_nt_bf16(pb, vt, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last);
+          !e.empty())
+        return e;
+    }
+  } else {
+    void* vt = nullptr;
+    if (ihip::Err e = run.alloc(&vt, bh * dv * nk * 4); !e.empty()) return e;
+    if (ihip::Err e = ihip::launch_transpose(v, vt, bh, nk, dv, 4, run.stream); !e.empty()) return e;
+    if (ihip::Err e = ihip::launch_gemm_nt_f32(s, static_cast<const float*>(vt), static_cast<float*>(out), bh, nq, dv, nk,
+                                               run.stream, &last);
+        !e.empty())
+      return e;
+  }
+  if (note) *note = ihip::LaunchNote{"attention in three kernels (head size above 128): " + first.kernel + ", " + middle.kernel + ", " + last.kernel, 0, 0};
+  return {};
+}
+
 ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* note) {
   switch (r.kind) {
     case Recognized::Attention: {
@@ -216,6 +277,8 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
         if (ihip::Err e = run.read_f32(r.scale.buffer, &sp); !e.empty()) return e;
         scale_ptr = static_cast<const float*>(sp);
       }
+      if (!ihip::attention_supported(bf16 ? ihip::BF16 : ihip::F32, dq, dv))
+        return attention_in_parts(run, r, bf16, bh, nq, nk, dq, dv, scale_ptr, note);
       void* out = nullptr;
       ihip::DType out_dt = ihip::F32;
       if (bf16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16) {

@@ -113,6 +113,7 @@ ROW_OP(softmax, 0)
 ROW_OP(shift, 1)
 ROW_OP(norm, 2)
 ROW_OP(exp, 3)
+ROW_OP(scaled_softmax, 4)  // the middle kernel of attention in three kernels (head sizes above 128)
 
 extern "C" __global__ void __launch_bounds__(256) convert_f32_to_bf16(ConvertParams p) {
   const float* s = reinterpret_cast<const float*>(p.src);

@@ -30,6 +30,9 @@ struct SoftmaxParams {
   const float* x;
   float* y;
   uint32_t rows, cols;
+  // the "softmax of scale * x" kernels only: scale = scale_value * (scale_ptr ? *scale_ptr : 1)
+  const float* scale_ptr;
+  float scale_value;
 };
 
 struct ConvertParams {

@@ -17,7 +17,7 @@
 #include "params.h"
 
 // NV = float4 chunks per lane; covers cols <= 256 * NV.  VEC: cols % 4 == 0.
-// MODE (0 softmax, 1 x - max, 2 x / sum, 3 exp) is a template parameter: as a run-time switch the four bodies
+// MODE (0 softmax, 1 x - max, 2 x / sum, 3 exp, 4 softmax of scale * x) is a template parameter: as a run-time switch the four bodies
 // cost the softmax a third of its registers' worth of occupancy and 13 % of its bandwidth.
 template <int NV, bool VEC, int MODE>
 __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
@@ -30,15 +30,20 @@ __device__ __forceinline__ void row_softmax_wave_body(const SoftmaxParams& p) {
   f32x4 r[NV];
   float mx = -INFINITY;
   const float pad = MODE == 2 ? 0.0f : -INFINITY;  // neutral for the reduction of the mode
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;  // mode 4: softmax(scale * x)
 #pragma unroll
   for (int t = 0; t < NV; ++t) {
     const uint32_t col = 4u * (lane + 64 * t);
     if (VEC) {
-      if (col < p.cols) r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
-      else r[t] = f32x4{pad, pad, pad, pad};
+      if (col < p.cols) {
+        r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
+        if constexpr (MODE == 4) r[t] *= sc;
+      } else {
+        r[t] = f32x4{pad, pad, pad, pad};
+      }
     } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : pad;
+      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? (MODE == 4 ? x[col + e] * sc : x[col + e]) : pad;
     }
     mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
   }
@@ -133,15 +138,20 @@ __device__ __forceinline__ void row_softmax_group_body(const SoftmaxParams& p) {
   f32x4 r[NV];
   float mx = -INFINITY;
   const float pad = MODE == 2 ? 0.0f : -INFINITY;  // neutral for the reduction of the mode
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;  // mode 4: softmax(scale * x)
 #pragma unroll
   for (int t = 0; t < NV; ++t) {
     const uint32_t col = 4u * (tid + 64 * NW * t);
     if (VEC) {
-      if (col < p.cols) r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
-      else r[t] = f32x4{pad, pad, pad, pad};
+      if (col < p.cols) {
+        r[t] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
+        if constexpr (MODE == 4) r[t] *= sc;
+      } else {
+        r[t] = f32x4{pad, pad, pad, pad};
+      }
     } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? x[col + e] : pad;
+      for (int e = 0; e < 4; ++e) r[t][e] = (col + e < p.cols) ? (MODE == 4 ? x[col + e] * sc : x[col + e]) : pad;
     }
     mx = fmaxf(fmaxf(fmaxf(r[t][0], r[t][1]), fmaxf(r[t][2], r[t][3])), mx);
   }
@@ -228,8 +238,9 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
     for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] / total;
     return;
   }
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;  // mode 4: softmax(scale * x)
   float mx = -INFINITY;
-  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) mx = fmaxf(mx, x[j]);
+  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) mx = fmaxf(mx, x[j] * sc);
   mx = wave_max(mx);
   if (lane == 0) red[wave] = mx;
   __syncthreads();
@@ -242,7 +253,7 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
   }
   const float mb = mx * I_LOG2_E32;
   float sum = 0.0f;
-  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) sum += fast_exp2(__builtin_fmaf(x[j], I_LOG2_E32, -mb));
+  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) sum += fast_exp2(__builtin_fmaf(x[j] * sc, I_LOG2_E32, -mb));
   sum = wave_sum(sum);
   if (lane == 0) red[wave] = sum;
   __syncthreads();
@@ -250,5 +261,5 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
   for (int w = 0; w < nw; ++w) sum += red[w];
   const float inv = 1.0f / sum;
   for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x)
-    y[j] = fast_exp2(__builtin_fmaf(x[j], I_LOG2_E32, -mb)) * inv;
+    y[j] = fast_exp2(__builtin_fmaf(x[j] * sc, I_LOG2_E32, -mb)) * inv;
 }

@@ -235,13 +235,14 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
 }
 
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode,
-                       LaunchNote* note) {
+                       LaunchNote* note, const float* scale_ptr, float scale) {
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
-  if (mode < 0 || mode > 3) return "row_softmax kernel: unknown mode";
-  static const char* const kOps[4] = {"softmax", "shift", "norm", "exp"};
-  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols};
+  if (mode < 0 || mode > 4) return "row_softmax kernel: unknown mode";
+  if (mode == 4 && !std::isfinite(scale)) return "row_softmax kernel: unsupported scale (must be finite)";
+  static const char* const kOps[5] = {"softmax", "shift", "norm", "exp", "scaled_softmax"};
+  SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, scale_ptr, scale};
   hipFunction_t fn;
   if (cols <= 8192) {
     int nv = 1;

@@ -55,9 +55,11 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
 bool gemm_nt_f32_supported(size_t k);
 
 // y[rows,cols] = row softmax of x, f32
-// mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize); 3: y = exp(x)
+// mode 0: softmax; 1: y = x - rowmax(x) (row_max_shift); 2: y = x / rowsum(x) (row_normalize); 3: y = exp(x);
+// 4: softmax of s * x with s = scale * (scale_ptr ? *scale_ptr : 1), scale_ptr a rank-0 f32 operand in device memory.
+// y may be x: every kernel has read a row's element before it writes it.
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0,
-                       LaunchNote* note = nullptr);
+                       LaunchNote* note = nullptr, const float* scale_ptr = nullptr, float scale = 1.0f);
 
 // dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  An NN product that the direct kernels cannot read runs as transpose + NT kernel.
 Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,

@@ -120,6 +120,31 @@ def test_reference_demo_flash_and_naive_attention(torch):
         assert np.allclose(got, ref, rtol=3e-4, atol=5e-5, equal_nan=True)  # the demo's own tolerance
 
 
+def test_head_sizes_above_128_run_as_three_hand_written_kernels(torch):
+    """d or dv above 128 (the demo's own shape is [32, 2048], flash-attn.py:31-36): scores by the MFMA GEMM, row
+    softmax in place, output by the MFMA GEMM.  f32 at the demo's shape against the emitted C; bf16 with batch axes,
+    a score scale and ragged query counts at d = 192 and d = 256 (dv = 160) against the oracle."""
+    q, k, v = rnd((32, 2048), 1), rnd((32, 2048), 2), rnd((32, 2048), 3)
+    comp = flash()
+    got = comp.exec_numpy(q, k, v)
+    assert "attention in three kernels" in comp.report() and "gemm_nt_f32" in comp.report()
+    close(got, oracle.compile_component(comp.handle).run(q, k, v), RTOL_F32)
+    for d, dv, nq, nk in ((192, 192, 300, 512), (256, 160, 77, 136)):
+        qb, kb, vb = (oracle.to_bf16_f32(rnd(shape, seed)) for seed, shape in
+                      ((1, (2, 3, nq, d)), (2, (2, 3, nk, d)), (3, (2, 3, nk, dv))))
+        scale = np.float32(1.0 / np.sqrt(d))
+        comp = flash("i:128,j:64", prefix="bh", scaled=True)
+        out = comp.exec_torch(torch.from_numpy(qb).cuda().bfloat16(), torch.from_numpy(kb).cuda().bfloat16(),
+                              torch.tensor(scale, device="cuda"), torch.from_numpy(vb).cuda().bfloat16())
+        assert "attention in three kernels" in comp.report() and "scaled_softmax" in comp.report()
+        close(out.cpu().numpy(), oracle.attention_tiled(qb, kb, vb, scale), RTOL_BF16)
+    # extents the GEMM kernels cannot take (f32 with a key count that is no multiple of 32) still run generated
+    q, k, v = rnd((20, 160), 1), rnd((33, 160), 2), rnd((33, 160), 3)
+    comp = flash()
+    close(comp.exec_numpy(q, k, v), oracle.attention_tiled(q, k, v), RTOL_F32)
+    assert "generated kernel" in comp.report()
+
+
 # ------------------------------------------------------------------ BASELINE config 1
 @pytest.mark.parametrize("split", ["i:16,j:16", "i:32,j:8", "i:128,j:64"])
 def test_config1_demo_attention_f32_vs_emitted_c(torch, split):
