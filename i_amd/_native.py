@@ -46,6 +46,8 @@ core.i_hip_program_report.argtypes = [vp]
 core.i_hip_program_report.restype = vp
 core.i_hip_gemm_nt_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nt_bf16.restype = ctypes.c_int
+core.i_hip_gemm_nt_bf16_ex.argtypes = [vp, vp, vp, ctypes.c_int, sz, sz, sz, sz, sz, sz, vp]
+core.i_hip_gemm_nt_bf16_ex.restype = ctypes.c_int
 core.i_hip_gemm_nn_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nn_bf16.restype = ctypes.c_int
 core.i_hip_gemm_nt_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]

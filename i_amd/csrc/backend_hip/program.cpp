@@ -214,6 +214,11 @@ std::string describe_launch(const ihip::LaunchNote& note, const Recognized& r) {
   return text;
 }
 
+// A product of bf16 operands whose result is a bf16 program output: the GEMM kernels write it themselves.
+bool bf16_result_in_place(const Run& run, const Recognized& r) {
+  return run.dtype_of(r.a.buffer) == DType::BF16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16;
+}
+
 ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
                              const float* scale_ptr, ihip::LaunchNote* note) {
   void* out = nullptr;
@@ -301,13 +306,19 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       }
       if (b[nb + 1] != a[nb + 1]) return "gemm operands disagree on the contracted extent";
       void* out = nullptr;
-      if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
+      ihip::DType out_dt = ihip::F32;
+      if (bf16_result_in_place(run, r)) {  // the kernel rounds its f32 sums to the bf16 output itself
+        out = run.raw_ptr(r.out);
+        out_dt = ihip::BF16;
+      } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
+        return e;
+      }
       if (run.dtype_of(r.a.buffer) == DType::F32)
         return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)),
                                         static_cast<const float*>(run.raw_ptr(r.b.buffer)), static_cast<float*>(out), bh,
                                         a[nb], b[nb], a[nb + 1], run.stream, note);
-      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh,
-                                       a[nb], b[nb], a[nb + 1], run.stream, r.tile_i, r.tile_j, note);
+      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), out, bh, a[nb], b[nb], a[nb + 1],
+                                       run.stream, r.tile_i, r.tile_j, note, out_dt);
     }
     case Recognized::GemmNN: {
       // b [B.., K, J]: the direct bf16 kernels read it in place; otherwise it is transposed into a stream-ordered
@@ -322,24 +333,26 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       const size_t m = a[nb], k = a[nb + 1], n = b[nb + 1];
       if (b[nb] != k) return "gemm operands disagree on the contracted extent";
       const bool f32 = run.dtype_of(r.a.buffer) == DType::F32;
-      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k)) {
-        // the direct kernels read a row-major right operand themselves
-        void* out = nullptr;
-        if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
-        return ihip::launch_gemm_nn_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), static_cast<float*>(out), bh, m, n, k,
-                                         run.stream, r.tile_i, r.tile_j, note);
+      void* out = nullptr;
+      ihip::DType out_dt = ihip::F32;
+      if (bf16_result_in_place(run, r)) {
+        out = run.raw_ptr(r.out);
+        out_dt = ihip::BF16;
+      } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
+        return e;
       }
+      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k))  // the direct kernels read a row-major right operand themselves
+        return ihip::launch_gemm_nn_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), out, bh, m, n, k, run.stream,
+                                         r.tile_i, r.tile_j, note, out_dt);
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
       if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;
       if (ihip::Err e = ihip::launch_transpose(run.raw_ptr(r.b.buffer), bt, bh, k, n, elem, run.stream); !e.empty()) return e;
-      void* out = nullptr;
-      if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
       if (f32)
         return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)), static_cast<const float*>(bt),
                                         static_cast<float*>(out), bh, m, n, k, run.stream, note);
-      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, static_cast<float*>(out), bh, m, n, k, run.stream,
-                                       r.tile_i, r.tile_j, note);
+      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note,
+                                       out_dt);
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:

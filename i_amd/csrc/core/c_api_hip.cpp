@@ -35,6 +35,13 @@ int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t
   return finish(ihip::launch_gemm_nt_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream));
 }
 
+int i_hip_gemm_nt_bf16_ex(const void* a, const void* b, void* c, int out_dtype, size_t bh, size_t m, size_t n, size_t k,
+                          size_t tile_m, size_t tile_n, void* stream) {
+  if (!dtype_ok(out_dtype)) return finish("unknown dtype");
+  return finish(ihip::launch_gemm_nt_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream, tile_m, tile_n, nullptr,
+                                          (ihip::DType)out_dtype));
+}
+
 int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k, void* stream) {
   return finish(ihip::launch_gemm_nn_bf16(a, b, c, bh, m, n, k, (hipStream_t)stream));
 }

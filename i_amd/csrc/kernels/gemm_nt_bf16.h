@@ -48,7 +48,7 @@ __device__ __forceinline__ void gemm_nt_bf16_body(const GemmParams& p) {
 
   const bf16_t* __restrict__ A = reinterpret_cast<const bf16_t*>(p.a) + (size_t)batch * p.m * p.k;
   const bf16_t* __restrict__ B = reinterpret_cast<const bf16_t*>(p.b) + (size_t)batch * p.n * p.k;
-  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
+  float* __restrict__ C = reinterpret_cast<float*>(reinterpret_cast<char*>(p.c) + (size_t)batch * p.m * p.n * (p.out_bf16 ? 2 : 4));
   const uint32_t m0 = tm * BMT, n0 = tn * BNT;
 
   u32x4 areg[A_ITERS], breg[B_ITERS];
@@ -126,7 +126,10 @@ __device__ __forceinline__ void gemm_nt_bf16_body(const GemmParams& p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (row < p.m && col < p.n) C[(size_t)row * p.n + col] = acc[i][j][e];
+        if (row < p.m && col < p.n) {
+          if (p.out_bf16) reinterpret_cast<bf16_t*>(C)[(size_t)row * p.n + col] = (bf16_t)acc[i][j][e];
+          else C[(size_t)row * p.n + col] = acc[i][j][e];
+        }
       }
     }
 }

@@ -82,7 +82,9 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   const size_t brow_bytes = (size_t)p.n * ELEM;  // NN: a row of B is n elements
   const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
   const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;  // n k = k n elements
-  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
+  // (a bf16 output is addressed through the same pointer with half the element size)
+  float* __restrict__ C = reinterpret_cast<float*>(reinterpret_cast<char*>(p.c) +
+                                                   (size_t)batch * p.m * p.n * ((!F32 && p.out_bf16) ? 2 : 4));
   const uint32_t m0 = tm * BMT, n0 = tn * BNT;
 
   // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
@@ -261,15 +263,24 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   // ---- store.  Accumulator layout: column n = c, rows 8 (e / 4) + 4 h + e % 4: every store instruction
   // writes two full 128-byte lines.  C is written once and not read again: non-temporal.
   const bool interior = m0 + BMT <= p.m && n0 + BNT <= p.n;
+  auto store_tile = [&](auto out_is_bf16) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const uint32_t col = n0 + (wn * TN + j) * 32 + c;
+      for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + (wn * TN + j) * 32 + c;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (interior || (row < p.m && col < p.n)) __builtin_nontemporal_store(acc[i][j][e], &C[(size_t)row * p.n + col]);
+        for (int e = 0; e < 16; ++e) {
+          const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+          if (interior || (row < p.m && col < p.n)) {
+            if constexpr (decltype(out_is_bf16)::value)
+              __builtin_nontemporal_store((bf16_t)acc[i][j][e], &reinterpret_cast<bf16_t*>(C)[(size_t)row * p.n + col]);
+            else __builtin_nontemporal_store(acc[i][j][e], &C[(size_t)row * p.n + col]);
+          }
+        }
       }
-    }
+  };
+  // bf16 output (bf16 operands only): the f32 sums are rounded on the way out, half the bytes
+  if (!F32 && p.out_bf16) store_tile(std::true_type{});
+  else store_tile(std::false_type{});
 }

@@ -21,9 +21,10 @@ struct AttnParams {
 struct GemmParams {
   const void* a;   // [bh, m, k]
   const void* b;   // [bh, n, k]
-  void* c;         // [bh, m, n]  f32
+  void* c;         // [bh, m, n]  f32, or bf16 when out_bf16 is set (bf16 operands only)
   uint32_t bh, m, n, k;
   uint32_t tiles_m, tiles_n;
+  uint32_t out_bf16;  // 0: f32 output, 1: the f32 sums are rounded to bf16 on the way out
 };
 
 struct SoftmaxParams {

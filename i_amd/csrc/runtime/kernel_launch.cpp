@@ -124,8 +124,8 @@ static unsigned pick_direct_tile(size_t t256, size_t t128) {
   return e256 >= e128 ? 256 : 128;
 }
 
-Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note) {
+Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype) {
   if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || !fits_u32(k) || !fits_u32(bh)) return "gemm_nt kernel: extent exceeds 32 bits";
@@ -133,6 +133,7 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
   // Direct global -> LDS kernels (need whole 64-wide k slabs and 32-bit byte offsets inside a tile's rows):
   //   256 x 256 tiles  long k loops on grids that fill at least half of the CUs (its prologue and its
   //                    unoverlapped store only pay off there)
@@ -186,8 +187,8 @@ static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t til
 
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return gemm_nn_tile(bh, m, n, k, 0, 0) != 0; }
 
-Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note) {
+Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype) {
   const unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
   if (tile == 0) return "gemm_nn kernel: needs k % 64 == 0 and n % 8 == 0 (and extents within its offset range)";
   if (bh == 0 || m == 0 || n == 0) return {};
@@ -195,6 +196,7 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
   p.tiles_m = (uint32_t)((m + tile - 1) / tile);
   p.tiles_n = (uint32_t)((n + tile - 1) / tile);
   const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs

@@ -36,17 +36,19 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
                      const AttentionOptions& options = {}, LaunchNote* note = nullptr);
 bool attention_supported(DType in_dtype, size_t d, size_t dv);
 
-// c[bh,m,n] (f32) = a[bh,m,k] b[bh,n,k]^T, a and b bf16
+// c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, a and b bf16, sums in f32; c is f32, or bf16 (out_dtype) with the sums rounded on the way out
 // tile_m x tile_n is the output tile the schedule asks for (0 = no preference): 256 x 256 and 128 x 128 select
 // the kernel with that workgroup tile (when its requirements hold), anything else leaves the choice to the launcher.
-Err launch_gemm_nt_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr);
+Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr,
+                        DType out_dtype = F32);
 bool gemm_nt_bf16_supported(size_t k);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
 // Needs k % 64 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
-Err launch_gemm_nn_bf16(const void* a, const void* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr);
+Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
+                        hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr,
+                        DType out_dtype = F32);
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
 
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 32 == 0

@@ -122,6 +122,15 @@ int i_hip_gemm_nt_bf16(const void* a, const void* b, float* c,
                        size_t bh, size_t m, size_t n, size_t k, void* stream);
 
 /*
+ * i_hip_gemm_nt_bf16 with the output element type and the schedule's tile spelled out: c is f32 (I_DTYPE_F32) or
+ * bf16 (I_DTYPE_BF16: the f32 sums are rounded to nearest-even on the way out, half the bytes written);
+ * tile_m x tile_n of 128 x 128 or 256 x 256 selects the kernel with that workgroup tile, 0 leaves the choice to
+ * the launcher.
+ */
+int i_hip_gemm_nt_bf16_ex(const void* a, const void* b, void* c, int out_dtype,
+                          size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n, void* stream);
+
+/*
  * The product with a row-major right operand,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,k,n]  (bf16 a, b, f32 c):
  * the fused kernel for  i("ik*kj~ijk") >> i("+ijk~ij ...")  (ilang-python/test.py:52-56) and for the demo's
  * standalone mm,  i("ij*jk~ikj") >> i("+ikj~ik ...")  (ilang-python/flash-attn.py:51).  Requires k % 64 == 0

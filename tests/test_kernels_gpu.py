@@ -386,6 +386,29 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, dire
     assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("tile", [0, 128, 256])
+def test_gemm_nt_bf16_output_in_bf16(env, monkeypatch, tile):
+    """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
+    result rounded to bf16, bit for bit, for the register-staged kernel (ILANG_GEMM_DIRECT=0) and both tiles."""
+    t = env.torch
+    if tile == 0:
+        monkeypatch.setenv("ILANG_GEMM_DIRECT", "0")
+    for bh, m, n, k in ((2, 300, 260, 128), (1, 512, 512, 576), (3, 1, 1, 64)):
+        a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+        b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
+        ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+        c32 = t.full((bh, m, n), float("nan"), device="cuda")
+        c16 = t.full((bh, m, n), float("nan"), device="cuda", dtype=t.bfloat16)
+        core = env.nat.core
+        env.nat.check(core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), c32.data_ptr(), env.nat.F32, bh, m, n, k,
+                                                  tile, tile, env.stream()))
+        env.nat.check(core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), c16.data_ptr(), env.nat.BF16, bh, m, n, k,
+                                                  tile, tile, env.stream()))
+        t.cuda.synchronize()
+        assert t.equal(c16, c32.bfloat16())
+        assert_close(c32.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
+
+
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 264, 128), (2, 600, 520, 192), (1, 1, 8, 256),
                                       (3, 257, 248, 320), (1, 130, 1000, 64)])
 @pytest.mark.parametrize("direct", ["256", "128"])
