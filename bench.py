@@ -289,6 +289,16 @@ def main():
     _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), short_steps, short_warmup)
     c1_flop = 4.0 * 512 * 512 * 64
 
+    # What this box's matrix cores deliver to the vendor's own GEMM (torch.matmul -> hipBLASLt, bf16 in, bf16 out)
+    # on the same operands as the mm_t line: a practical ceiling for dense bf16 on random data on this box, next to
+    # which the MFMA lines can be read.  Not part of the product path; the shader clock under dense MFMA work on
+    # random operands stays well below the 2.4 GHz the 2.5 PFLOP/s peak is quoted at.
+    lib_ms = None
+    if args.steps >= 20:
+        bt_ = b.t()
+        torch.matmul(a, bt_)
+        _, lib_ms = time_steps(torch, lambda: torch.matmul(a, bt_), short_steps, short_warmup)
+
     if args.calibrate_copy:
         y.copy_(x)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
@@ -363,6 +373,11 @@ def main():
             "workload": "the same launch with every element of Q, K, V equal to 0.01 (not the benchmark data)",
             "value": flop / (const_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": const_ms,
             "frac_of_peak": flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+        "library_gemm_probe": None if lib_ms is None else {
+            "workload": "torch.matmul (hipBLASLt) bf16 4096^3, bf16 out, on the operands of the mm_t line: the vendor "
+                        "library's dense bf16 rate on this box, for reading the MFMA fractions against",
+            "value": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": lib_ms,
+            "frac_of_peak": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
              "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),

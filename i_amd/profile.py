@@ -22,7 +22,7 @@ from collections import namedtuple
 KernelRow = namedtuple("KernelRow", "name calls total_us avg_us min_us max_us share lds_bytes workgroup")
 CounterRow = namedtuple("CounterRow", "kernel counter dispatches avg min max")
 
-_OURS = re.compile(r"^(attn_fwd_|gemm_n[nt]_|row_(softmax|shift|norm|exp)_|transpose_b(16|32)|convert_|f\d+(_p\d+)?$)")
+_OURS = re.compile(r"^(attn_fwd_|gemm_n[nt]_|row_(softmax|shift|norm|exp|scaled_softmax)_|transpose_b(16|32)|convert_|f\d+(_p\d+)?$)")
 
 
 def is_backend_kernel(name):
