@@ -292,78 +292,141 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
     // one statement of the module per action of the plan kernel (a trailing return aside)
     size_t fn_stmts = fn.body.size();
     while (fn_stmts > 0 && fn.body[fn_stmts - 1].kind == MStmt::Return) --fn_stmts;
-    // Splitting into phases is opt-in (ILANG_HIP_PHASES=1): it is verified on the CPU emulation of the runtime
-    // only, see tests/test_generated_kernels_cpu.py.
+    // A body that is a sequence of top-level statements is split into phases (one per loop nest).  Default: the
+    // phases share one launch of one workgroup with barriers between them, provided some nest has parallel loops
+    // (otherwise the kernel stays a single work-item).  ILANG_HIP_PHASES=1: one launch per phase (CPU emulation only).
     const char* want_phases = std::getenv("ILANG_HIP_PHASES");
+    const bool separate_launches = want_phases && want_phases[0] == '1';
     auto ranges = phase_ranges(body);
-    if (fn_stmts != body.size() || !want_phases || want_phases[0] != '1') ranges = {{0, body.size()}};  // one phase, whole body
-    // buffers touched by more than one phase stay in memory
-    std::map<Param, size_t> touched;
+    if (fn_stmts != body.size()) ranges = {{0, body.size()}};  // no statement-by-statement correspondence: one phase
+    auto analyze_all = [&](const std::vector<std::pair<size_t, size_t>>& rs, std::vector<Block<Param>>& bodies,
+                           std::vector<GenericPhase>& phases) {
+      // buffers touched by more than one phase stay in memory
+      std::map<Param, size_t> touched;
+      bodies.clear();
+      phases.clear();
+      for (const auto& [first, last] : rs) {
+        bodies.emplace_back(body.begin() + first, body.begin() + last);
+        Uses u;
+        collect(bodies.back(), u);
+        std::set<Param> seen;
+        for (const auto* a : u.all) seen.insert(a->buffer);
+        for (const Param& b : seen) ++touched[b];
+      }
+      std::set<Param> shared;
+      for (const auto& [b, n] : touched)
+        if (n > 1) shared.insert(b);
+      for (size_t ph = 0; ph < rs.size(); ++ph) {
+        GenericPhase phase;
+        phase.name = rs.size() == 1 || !separate_launches ? info.name : info.name + "_p" + std::to_string(ph);
+        analyze(plan, k, bodies[ph], shared, phase);
+        phases.push_back(std::move(phase));
+      }
+    };
     std::vector<Block<Param>> bodies;
-    for (const auto& [first, last] : ranges) {
-      bodies.emplace_back(body.begin() + first, body.begin() + last);
-      Uses u;
-      collect(bodies.back(), u);
-      std::set<Param> seen;
-      for (const auto* a : u.all) seen.insert(a->buffer);
-      for (const Param& b : seen) ++touched[b];
+    std::vector<GenericPhase> phases;
+    analyze_all(ranges, bodies, phases);
+    bool cooperative = false;
+    if (ranges.size() > 1 && !separate_launches) {
+      for (const GenericPhase& ph : phases) cooperative |= !ph.parallel_loops.empty();
+      if (!cooperative) {  // nothing to spread over work-items: the whole body as one phase, one work-item
+        ranges = {{0, body.size()}};
+        analyze_all(ranges, bodies, phases);
+      }
     }
-    std::set<Param> shared;
-    for (const auto& [b, n] : touched)
-      if (n > 1) shared.insert(b);
+    info.cooperative = cooperative;
 
     const size_t nr = std::max<size_t>(info.n_reads, 1), nw = std::max<size_t>(info.n_writes, 1);
     src << "struct Args_" << info.name << " { View readonlys[" << nr << "]; View writeables[" << nw << "]; };\n";
+    const Step* dispatch = nullptr;
+    for (const Step& st : plan.exec)
+      if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
+    // work-item-private buffers of one phase: a local array, or this work-item's slice of a device buffer
+    auto emit_privates = [&](const GenericPhase& phase, const std::string& pad) {
+      for (const PrivateBuffer& pb : phase.privates) {
+        if (pb.is_static) {
+          src << pad << "float priv" << pb.writeable << "[" << pb.static_size << "];\n";
+          src << pad << "writeables[" << pb.writeable << "].data = priv" << pb.writeable << ";\n";
+        } else {
+          const size_t prank = plan.intermediates[dispatch->writes[pb.writeable].id].layout.size();
+          src << pad << "{ size_t n = 1; for (int d = 0; d < " << prank << "; ++d) n *= writeables[" << pb.writeable
+              << "].layout[d]; writeables[" << pb.writeable << "].data += wi_first * n; }\n";
+        }
+      }
+    };
+    // the statements of one phase spread over the work-items (wi_first, wi_stride); `depth` is the indentation
+    auto emit_spread = [&](const GenericPhase& phase, const std::vector<MStmt>& stmts, int depth) {
+      const std::string pad(2 * depth, ' ');
+      Printer pr;
+      std::vector<std::string> iters;
+      for (size_t id : phase.parallel_loops) iters.push_back("i" + std::to_string(id));
+      for (const std::string& it : iters) {
+        const MStmt* loop = find_loop(stmts, it);
+        if (!loop) lower_error("parallel loop " + it + " not found in kernel body");
+        src << pad << "const size_t n_" << it << " = " << expr_text(*loop->value) << ";\n";
+        pr.parallel.insert(it);
+      }
+      src << pad << "size_t wi_total = 1;\n";
+      for (const std::string& it : iters) src << pad << "wi_total *= n_" << it << ";\n";
+      src << pad << "for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
+      src << pad << "  size_t wi_rest = wi;\n";
+      for (size_t t = iters.size(); t-- > 0;) {
+        src << pad << "  const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
+        src << " wi_rest /= n_" << iters[t] << ";\n";
+      }
+      pr.block(stmts, depth + 1);
+      src << pr.os.str();
+      src << pad << "}\n";
+    };
+    auto phase_stmts = [&](size_t ph) {
+      return std::vector<MStmt>(fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].first : 0),
+                                fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].second : fn_stmts));
+    };
+    if (cooperative) {
+      src << "extern \"C\" __global__ void __launch_bounds__(" << GenericKernel::kCooperativeThreads << ") " << info.name
+          << "(Args_" << info.name << " args) {\n";
+      src << "  const View* readonlys = args.readonlys;\n";
+      src << "  View writeables[" << nw << "];\n";
+      src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
+      src << "  // one workgroup: every loop nest below is spread over its work-items, a barrier orders the nests\n";
+      src << "  const size_t wi_first = threadIdx.x;\n";
+      src << "  const size_t wi_stride = blockDim.x;\n";
+      for (size_t ph = 0; ph < ranges.size(); ++ph) {
+        if (ph > 0) src << "  __syncthreads();\n";
+        src << "  {\n";
+        emit_privates(phases[ph], "    ");
+        if (phases[ph].parallel_loops.empty()) {
+          src << "    if (wi_first == 0) {\n";
+          Printer pr;
+          pr.block(phase_stmts(ph), 3);
+          src << pr.os.str();
+          src << "    }\n";
+        } else {
+          emit_spread(phases[ph], phase_stmts(ph), 2);
+        }
+        src << "  }\n";
+      }
+      src << "}\n\n";
+      for (auto& ph : phases) info.phases.push_back(std::move(ph));
+      continue;
+    }
     for (size_t ph = 0; ph < ranges.size(); ++ph) {
-      GenericPhase phase;
-      phase.name = ranges.size() == 1 ? info.name : info.name + "_p" + std::to_string(ph);
-      analyze(plan, k, bodies[ph], shared, phase);
-      const std::vector<MStmt> stmts(fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].first : 0),
-                                     fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].second : fn_stmts));
+      GenericPhase& phase = phases[ph];
+      const std::vector<MStmt> stmts = phase_stmts(ph);
       src << "extern \"C\" __global__ void __launch_bounds__(64) " << phase.name << "(Args_" << info.name << " args) {\n";
       src << "  const View* readonlys = args.readonlys;\n";
       src << "  View writeables[" << nw << "];\n";
       src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
       src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
       src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
-      for (const PrivateBuffer& pb : phase.privates) {
-        if (pb.is_static) {
-          src << "  float priv" << pb.writeable << "[" << pb.static_size << "];\n";
-          src << "  writeables[" << pb.writeable << "].data = priv" << pb.writeable << ";\n";
-        } else {
-          const Step* dispatch = nullptr;
-          for (const Step& st : plan.exec)
-            if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
-          const size_t prank = plan.intermediates[dispatch->writes[pb.writeable].id].layout.size();
-          src << "  { size_t n = 1; for (int d = 0; d < " << prank << "; ++d) n *= writeables[" << pb.writeable
-              << "].layout[d]; writeables[" << pb.writeable << "].data += wi_first * n; }\n";
-        }
-      }
-      Printer pr;
+      emit_privates(phase, "  ");
       if (phase.parallel_loops.empty()) {
         src << "  if (wi_first != 0) return;\n";
+        Printer pr;
         pr.block(stmts, 1);
         src << pr.os.str();
       } else {
-        std::vector<std::string> iters;
-        for (size_t id : phase.parallel_loops) iters.push_back("i" + std::to_string(id));
-        for (const std::string& it : iters) {
-          const MStmt* loop = find_loop(stmts, it);
-          if (!loop) lower_error("parallel loop " + it + " not found in kernel body");
-          src << "  const size_t n_" << it << " = " << expr_text(*loop->value) << ";\n";
-          pr.parallel.insert(it);
-        }
-        src << "  size_t wi_total = 1;\n";
-        for (const std::string& it : iters) src << "  wi_total *= n_" << it << ";\n";
-        src << "  for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
-        src << "    size_t wi_rest = wi;\n";
-        for (size_t t = iters.size(); t-- > 0;) {
-          src << "    const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
-          src << " wi_rest /= n_" << iters[t] << ";\n";
-        }
-        pr.block(stmts, 2);
-        src << pr.os.str();
-        src << "  }\n";
+        emit_spread(phase, stmts, 1);
       }
       src << "}\n\n";
       info.phases.push_back(std::move(phase));

@@ -24,8 +24,10 @@ struct PrivateBuffer {
 };
 
 // A kernel whose body is a sequence of loop nests (e.g. a row maximum followed by the subtraction that
-// consumes it) is launched as one phase per top-level nest, in order on the stream: every phase gets its own
-// work-item space, and the stream order is the grid-wide dependency between them.
+// consumes it) has one phase per top-level nest.  By default the phases run inside one launch of one workgroup,
+// separated by workgroup barriers (GenericKernel::cooperative).  With ILANG_HIP_PHASES=1 every phase is a launch
+// of its own with its own work-item space, the stream order being the grid-wide dependency between them; that
+// form is confined to the CPU emulation of the runtime.
 struct GenericPhase {
   std::string name;                       // f<k> for a single-phase kernel, f<k>_p<i> otherwise
   std::vector<size_t> parallel_loops;     // loop ids, outermost first (empty: one work-item)
@@ -37,6 +39,11 @@ struct GenericKernel {
   std::string name;                       // f<k>; empty when not emitted
   size_t n_reads = 0, n_writes = 0;
   std::vector<GenericPhase> phases;
+  // A kernel whose body is a sequence of loop nests, some of them parallel: ONE launch of one workgroup of
+  // kCooperativeThreads work-items, every nest spread over them, workgroup barriers between the nests (the phases
+  // then describe the nests of that one launch, not launches of their own).
+  bool cooperative = false;
+  static constexpr unsigned kCooperativeThreads = 1024;
   bool is_private(size_t writeable) const {
     for (const GenericPhase& ph : phases)
       for (const PrivateBuffer& pb : ph.privates)

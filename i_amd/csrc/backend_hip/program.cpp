@@ -408,7 +408,7 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
   if (gk.name.empty()) return "kernel " + std::to_string(k) + " has no generated form";
   // One launch per top-level loop nest (ILANG_HIP_PHASES=1 at compile time) is confined to the emulated runtime:
   // its one run on a GPU ended in a memory fault whose cause has not been shown, so it must not reach a device.
-  if (gk.phases.size() > 1 && !ihip::runtime_is_emulated())
+  if (gk.phases.size() > 1 && !gk.cooperative && !ihip::runtime_is_emulated())
     return "kernel " + std::to_string(k) + " was compiled with ILANG_HIP_PHASES=1 (one launch per loop nest), which is "
            "restricted to the CPU emulation of the runtime; unset it and compile again";
   const size_t R = p.generic.rank;
@@ -437,6 +437,24 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
     fill(nr + i, ptr, dispatch.writes[i]);
   }
 
+  if (gk.cooperative) {
+    // one launch of one workgroup; every nest's work-item-private device buffers get one slice per work-item
+    run.notes.push_back("generated kernel " + gk.name + ": one workgroup of " + std::to_string(GenericKernel::kCooperativeThreads) +
+                        " work-items, " + std::to_string(gk.phases.size()) + " loop nests separated by barriers");
+    const size_t slots = GenericKernel::kCooperativeThreads;
+    for (const GenericPhase& ph : gk.phases)
+      for (const PrivateBuffer& pb : ph.privates) {
+        void* ptr = nullptr;
+        if (!pb.is_static) {
+          const size_t n = std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+          if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
+        }
+        fill(nr + pb.writeable, ptr, dispatch.writes[pb.writeable]);
+      }
+    hipFunction_t fn;
+    if (ihip::Err e = generic_function(p, gk.name, &fn); !e.empty()) return e;
+    return ihip::launch(fn, 1, 1, 1, GenericKernel::kCooperativeThreads, args.data(), args.size(), run.stream);
+  }
   run.notes.push_back("generated kernel " + gk.name + (gk.phases.size() > 1 ? " in " + std::to_string(gk.phases.size()) + " launches" : ""));
   // one launch per phase, in order on the stream
   for (const GenericPhase& ph : gk.phases) {
@@ -572,9 +590,14 @@ std::string program_code(const Component& component) {
     for (BufferRef r : d->reads) os << " " << ref_name(r);
     os << "; writes";
     for (BufferRef r : d->writes) os << " " << ref_name(r);
-    for (const GenericPhase& ph : gen.kernels[k].phases) {
+    if (gen.kernels[k].cooperative)
+      os << "\n//     one workgroup of " << GenericKernel::kCooperativeThreads << " work-items runs the " << gen.kernels[k].phases.size()
+         << " loop nests one after the other, a barrier between them";
+    for (size_t n = 0; n < gen.kernels[k].phases.size(); ++n) {
+      const GenericPhase& ph = gen.kernels[k].phases[n];
       os << "\n//     ";
-      if (gen.kernels[k].phases.size() > 1) os << "launch " << ph.name << ", ";
+      if (gen.kernels[k].cooperative) os << "nest " << n << ", ";
+      else if (gen.kernels[k].phases.size() > 1) os << "launch " << ph.name << ", ";
       os << "work-items:";
       if (ph.parallel_loops.empty()) os << " 1 (no independent outer loop)";
       for (size_t id : ph.parallel_loops) os << " i" << id;

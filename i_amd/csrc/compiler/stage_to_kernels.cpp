@@ -628,9 +628,14 @@ struct KernelBuilder {
       bool semantic_out = false;
       for (const LayoutDim& d : producer.output.layout) semantic_out |= d.semantic;
       if (semantic_out) {
-        // a protected (full-extent) producer is addressed by its semantic indexes
-        // (ids are the producer's own index numbers, looked up among this stage's axes)
-        const Layout layout = semantic_shape_layout(producer.output.shape, st);
+        // A protected (full-extent) producer is addressed by its semantic indexes.  The reference looks the
+        // producer's own index numbers up among this stage's axes (stage_to_kernel_program.rs:1279), which is only
+        // right when both expressions happen to number the shared indexes alike (they do in its demo); when they do
+        // not, e.g. (I & >ij~j) >> ij-j~ij with the maximum staged at the root, it addresses the buffer with the
+        // wrong index and, on non-square operands, out of bounds.  Here dimension d of the producer's output is
+        // this stage's index for dimension d of the operand (the positional match every edge is built on), which
+        // is the same thing wherever the reference's result is defined.
+        const Layout layout = semantic_shape_layout(input.shape, st);
         bool ok = true;
         for (const LayoutDim& d : layout)
           for (SAxisRef r : d.axes) ok &= available(axes, parent, r);

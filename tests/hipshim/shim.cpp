@@ -4,10 +4,13 @@
 //             filled with NaN bit patterns: an out-of-bounds access faults, a read of unwritten memory shows
 //   modules   an "image" is a host shared object (produced by hostcc.py from the generated HIP source);
 //             anything else (the prebuilt gfx950 code object) is refused, so only generated kernels run
-//   launches  run synchronously, one work-item after the other, with blockIdx / threadIdx set per item
+//   launches  run synchronously, one work-item after the other, with blockIdx / threadIdx set per item; a
+//             workgroup of more than 64 work-items runs its work-items as real threads with a working
+//             __syncthreads(), one workgroup after the other
 #include <dlfcn.h>
 #include <elf.h>
 #include <hip/hip_runtime_api.h>
+#include <pthread.h>
 #include <sys/mman.h>
 #include <unistd.h>
 
@@ -17,6 +20,8 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "../../i_amd/csrc/runtime/static_scratch.h"
 
@@ -60,6 +65,10 @@ struct Module {
 struct BigArgs {
   unsigned char bytes[4096];
 };
+struct Function {
+  void *kernel, *set_ids, *set_barrier;
+};
+void wait_on(void* barrier) { pthread_barrier_wait(static_cast<pthread_barrier_t*>(barrier)); }
 }  // namespace
 
 // The product takes its fixed workspace from a file-scope array in device memory (static_scratch.hip, built by
@@ -119,9 +128,10 @@ hipError_t hipModuleGetFunction(hipFunction_t* fn, hipModule_t mod, const char* 
   auto* m = reinterpret_cast<Module*>(mod);
   void* f = dlsym(m->handle, name);
   void* set = dlsym(m->handle, "shim_set_ids");
-  if (!f || !set) return hipErrorNotFound;
-  // a function handle is the pair (kernel, id setter of its library)
-  *fn = reinterpret_cast<hipFunction_t>(new std::pair<void*, void*>(f, set));
+  void* bar = dlsym(m->handle, "shim_set_barrier");
+  if (!f || !set || !bar) return hipErrorNotFound;
+  // a function handle is the triple (kernel, id setter and barrier setter of its library)
+  *fn = reinterpret_cast<hipFunction_t>(new Function{f, set, bar});
   return hipSuccess;
 }
 hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
@@ -137,11 +147,31 @@ hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, uns
   BigArgs args;
   std::memset(&args, 0xEE, sizeof args);
   std::memcpy(&args, buf, size);
-  auto* pair = reinterpret_cast<std::pair<void*, void*>*>(fn);
+  auto* f = reinterpret_cast<Function*>(fn);
   // a by-value struct larger than 16 bytes travels in memory at the start of the argument area, so a kernel
   // that declares a smaller struct reads its prefix of this one
-  auto kernel = reinterpret_cast<void (*)(BigArgs)>(pair->first);
-  auto set_ids = reinterpret_cast<void (*)(unsigned, unsigned, unsigned, unsigned)>(pair->second);
+  auto kernel = reinterpret_cast<void (*)(BigArgs)>(f->kernel);
+  auto set_ids = reinterpret_cast<void (*)(unsigned, unsigned, unsigned, unsigned)>(f->set_ids);
+  auto set_barrier = reinterpret_cast<void (*)(void (*)(void*), void*)>(f->set_barrier);
+  if (bx > 64) {
+    // the work-items of a workgroup run as threads, so that a barrier between two loop nests of a kernel means
+    // what it means on the device: every work-item has finished the first nest before any starts the second
+    for (unsigned block = 0; block < gx; ++block) {
+      pthread_barrier_t barrier;
+      pthread_barrier_init(&barrier, nullptr, bx);
+      std::vector<std::thread> items;
+      for (unsigned t = 0; t < bx; ++t)
+        items.emplace_back([&, t] {
+          set_ids(block, t, bx, gx);
+          set_barrier(wait_on, &barrier);
+          kernel(args);
+          set_barrier(nullptr, nullptr);
+        });
+      for (auto& th : items) th.join();
+      pthread_barrier_destroy(&barrier);
+    }
+    return hipSuccess;
+  }
   // ILANG_SHIM_ORDER=reverse runs the work-items last to first: a result that depends on the order in which
   // work-items run exposes a dependency between them that the parallelisation analysis missed
   const char* order = std::getenv("ILANG_SHIM_ORDER");

@@ -452,3 +452,18 @@ def test_generated_kernels_parallelise_independent_outer_loops():
     assert "work-items: i0 i1 i2 i3; work-item-private: s0[1]" in code
     assert "work-items: i0\n" in i("+ij~i")._code()
     assert "work-items: 1 (no independent outer loop)" in i("+ij~.")._code()
+
+
+def test_vector_staged_at_the_root_is_addressed_through_the_edge():
+    """(I & >ij~j) >> ij-j~ij with the maximum staged at the consumer's root: the two expressions number the shared
+    index differently (output axes first: j is 0 in the producer, 1 in the consumer).  The reference looks the
+    producer's numbers up among the consumer's axes (stage_to_kernel_program.rs:1279) and so subtracts max[i]
+    (out of bounds when rows > columns); this build matches the dimensions positionally.  Where the numbering
+    agrees (the reference's own demo: rows) nothing changes: the golden text above still matches byte for byte."""
+    x = np.random.default_rng(3).standard_normal((21, 9)).astype(np.float32)
+    for order in ("|i:8,j:4|{}ijj'i'", "||{}ij", "|j:4|{}ijj'", "|i:8|{}ii'j", "|i:8,j:4|{}jj'ii'"):
+        comp = (I & i(">ij~j" + order.format(""))) >> i("ij-j~ij" + order.format("1"))
+        got = run_c(comp, x)
+        assert np.array_equal(got, x - x.max(axis=0)), order
+    rows = (I & i(">ij~i|i:8,j:4|jii'j'")) >> i("ij-i~ij|i:8,j:4|1jii'j'")
+    assert np.array_equal(run_c(rows, x), x - x.max(axis=1, keepdims=True))

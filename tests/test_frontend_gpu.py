@@ -541,6 +541,28 @@ def test_non_f32_host_inputs_are_converted_like_the_reference(torch):
     assert np.allclose(i("+ij~i").exec_numpy(xt), xt.sum(1), rtol=1e-5, atol=1e-6)
 
 
+def test_multi_nest_generated_kernels_run_as_one_workgroup(torch, monkeypatch):
+    """Kernels whose body is a sequence of loop nests and that no hand-written kernel covers: one launch of one
+    workgroup of 1024 work-items with barriers between the nests, instead of a single work-item.  A column
+    normalisation (no hand-written form), and the naive three-kernel softmax and the naive attention with every
+    kernel forced into its generated form, against the emitted C."""
+    x = rnd((300, 70), 1)
+    colnorm = (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij")  # the column sums staged at the root: one kernel, two nests
+    close(colnorm.exec_numpy(x), x / x.sum(axis=0), RTOL_F32)
+    close(colnorm.exec_numpy(x), oracle.compile_component(colnorm.handle).run(x), RTOL_F32)
+    assert "one workgroup of 1024 work-items, 2 loop nests separated by barriers" in colnorm.report()
+    xd = torch.from_numpy(x).cuda()
+    assert torch.equal(colnorm.exec_torch(xd), colnorm.exec_torch(xd))  # repeatable
+    monkeypatch.setenv("ILANG_HIP_GENERATED_ONLY", "1")
+    sm = softmax_naive()
+    y = rnd((130, 257), 2)
+    close(sm.exec_numpy(y), oracle.row_softmax(y), RTOL_F32)
+    assert sm.report().count("one workgroup of 1024 work-items") == 2  # row_max_shift and row_normalize
+    q, k, v = rnd((40, 24), 1), rnd((50, 24), 2), rnd((50, 24), 3)
+    nv = naive()
+    close(nv.exec_numpy(q, k, v), oracle.compile_component(nv.handle).run(q, k, v), RTOL_F32)
+
+
 def test_per_nest_launches_are_refused_on_a_real_device():
     """ILANG_HIP_PHASES=1 (one launch per top-level loop nest of a generated kernel) is confined to the CPU emulation
     of the runtime: on a device the executor refuses such a kernel before launching it."""

@@ -86,6 +86,22 @@ print(i('ij+ij~ij').exec_numpy(ones(3, 2), ones(3, 2)).sum())
     assert r.stdout.split() == ["ok"] * 4 + ["12.0"], r.stdout
 
 
+def test_multi_nest_kernels_run_as_one_workgroup_by_default():
+    """A kernel whose body is a sequence of loop nests is one launch of one 1024-work-item workgroup with barriers
+    between the nests (the emulation runs such a workgroup as real threads); a body with nothing to spread over
+    work-items stays one work-item."""
+    env = dict(os.environ, ILANG_NO_TORCH="1")
+    env.pop("ILANG_HIP_PHASES", None)
+    code = ("from i_amd import Component as i, I\n"
+            "print(((I & i('+ij~j||ij')) >> i('ij/j~ij||1ij'))._code())\n"
+            "print(i('+ij~.')._code())")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300).stdout
+    assert "one workgroup of 1024 work-items runs the 2 loop nests one after the other, a barrier between them" in out
+    assert "nest 0, work-items: " in out and "nest 1, work-items: " in out
+    assert "void __launch_bounds__(1024) f0(Args_f0 args)" in out and out.count("__syncthreads();") == 1
+    assert "work-items: 1 (no independent outer loop)" in out
+
+
 def test_phase_plan_is_reported(shim_lib):
     env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_NO_TORCH="1")
     code = ("from i_amd import Component as i, I\n"
