@@ -66,8 +66,34 @@ std::string op_text(Op op, const std::vector<MExprPtr>& args) {
   return "0.0f";
 }
 
+// Every element access of a generated kernel is checked against the element count of its buffer ("cap_r<b>" /
+// "cap_w<b>", computed once per kernel from the view's layout): a load outside reads 0, a store outside is
+// dropped.  The loop nests and index expressions come from the schedule's lowering, and a schedule whose lowering
+// is not sound for the given extents (the reference accepts such schedules and reads or writes past its malloc'd
+// buffers) must not become a GPU memory fault.  ILANG_HIP_UNCHECKED=1 prints plain accesses (the CPU emulation
+// uses it so that its guard pages keep finding such lowerings).
+thread_local bool g_checked_accesses = true;
+
+// `base[idx]` with base = readonlys[b].data or writeables[b].data: fills the capacity variable's name
+bool buffer_access(const MExpr& e, std::string* cap) {
+  if (e.kind != MExpr::Index) return false;
+  const MExpr& base = *e.args[0];
+  if (base.kind != MExpr::Field || base.field != MField::Data) return false;
+  const MExpr* view = base.args[0].get();
+  while (view->kind == MExpr::Cast) view = view->args[0].get();
+  if (view->kind != MExpr::Index || view->args[0]->kind != MExpr::Ident || view->args[1]->kind != MExpr::Usize) return false;
+  const std::string& array = view->args[0]->ident;
+  if (array != "readonlys" && array != "writeables") return false;
+  *cap = (array == "readonlys" ? "cap_r" : "cap_w") + std::to_string(view->args[1]->usize);
+  return true;
+}
+
 std::string expr_text(const MExpr& e) {
   auto b = [&](const char* sym) { return "(" + expr_text(*e.args[0]) + " " + sym + " " + expr_text(*e.args[1]) + ")"; };
+  if (std::string cap; g_checked_accesses && buffer_access(e, &cap)) {
+    const std::string idx = expr_text(*e.args[1]);
+    return "((" + idx + ") < " + cap + " ? " + expr_text(*e.args[0]) + "[" + idx + "] : 0.0f)";
+  }
   switch (e.kind) {
     case MExpr::Usize: return "(size_t)" + std::to_string(e.usize);
     case MExpr::Scalar: return scalar_text(e.scalar);
@@ -235,7 +261,16 @@ struct Printer {
   }
   void stmt(const MStmt& s, int depth) {
     switch (s.kind) {
-      case MStmt::Set: line(depth, expr_text(*s.dst) + " = " + expr_text(*s.value) + ";"); break;
+      case MStmt::Set: {
+        std::string cap;
+        if (g_checked_accesses && buffer_access(*s.dst, &cap)) {
+          const std::string idx = expr_text(*s.dst->args[1]);
+          line(depth, "if ((" + idx + ") < " + cap + ") " + expr_text(*s.dst->args[0]) + "[" + idx + "] = " + expr_text(*s.value) + ";");
+        } else {
+          line(depth, expr_text(*s.dst) + " = " + expr_text(*s.value) + ";");
+        }
+        break;
+      }
       case MStmt::Loop:
         if (parallel.count(s.ident)) {
           block(s.body, depth);
@@ -268,6 +303,8 @@ const MStmt* find_loop(const std::vector<MStmt>& stmts, const std::string& iter)
 }  // namespace
 
 GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const std::vector<bool>& emit) {
+  const char* unchecked = std::getenv("ILANG_HIP_UNCHECKED");
+  g_checked_accesses = !(unchecked && unchecked[0] == '1');
   GenericModule out;
   out.kernels.resize(plan.kernels.size());
   size_t rank = 1;
@@ -341,6 +378,25 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
     const Step* dispatch = nullptr;
     for (const Step& st : plan.exec)
       if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
+    // element counts of the kernel's views, for the checked accesses: the product of the layout extents (a
+    // work-item-private slice or array has the same layout as the buffer it stands for)
+    auto emit_capacities = [&](const std::string& pad) {
+      if (!g_checked_accesses) return;
+      auto rank_of = [&](BufferRef r) {
+        return (r.kind == BufferRef::Input ? plan.inputs.at(r.id) : r.kind == BufferRef::Intermediate ? plan.intermediates.at(r.id)
+                                                                                                     : plan.outputs.at(r.id)).layout.size();
+      };
+      for (size_t b = 0; dispatch && b < dispatch->reads.size(); ++b) {
+        src << pad << "const size_t cap_r" << b << " = (size_t)1";
+        for (size_t d = 0; d < rank_of(dispatch->reads[b]); ++d) src << " * readonlys[" << b << "].layout[" << d << "]";
+        src << ";\n";
+      }
+      for (size_t b = 0; dispatch && b < dispatch->writes.size(); ++b) {
+        src << pad << "const size_t cap_w" << b << " = (size_t)1";
+        for (size_t d = 0; d < rank_of(dispatch->writes[b]); ++d) src << " * writeables[" << b << "].layout[" << d << "]";
+        src << ";\n";
+      }
+    };
     // work-item-private buffers of one phase: a local array, or this work-item's slice of a device buffer
     auto emit_privates = [&](const GenericPhase& phase, const std::string& pad) {
       for (const PrivateBuffer& pb : phase.privates) {
@@ -391,6 +447,7 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
       src << "  // one workgroup: every loop nest below is spread over its work-items, a barrier orders the nests\n";
       src << "  const size_t wi_first = threadIdx.x;\n";
       src << "  const size_t wi_stride = blockDim.x;\n";
+      emit_capacities("  ");
       for (size_t ph = 0; ph < ranges.size(); ++ph) {
         if (ph > 0) src << "  __syncthreads();\n";
         src << "  {\n";
@@ -419,6 +476,7 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
       src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
       src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
       src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
+      emit_capacities("  ");
       emit_privates(phase, "  ");
       if (phase.parallel_loops.empty()) {
         src << "  if (wi_first != 0) return;\n";

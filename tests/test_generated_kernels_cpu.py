@@ -27,8 +27,10 @@ def shim_lib():
 def run_cases(shim_lib, extra_env):
     env = dict(os.environ)
     env.pop("ILANG_HIP_PHASES", None)
+    # ILANG_HIP_UNCHECKED: plain accesses instead of the bounds-checked ones the product emits, so that an access
+    # outside a buffer still hits a guard page here and names a lowering that is not sound
     env.update({"ILANG_CORE_LIB": str(shim_lib), "ILANG_HIPCC": str(SHIM / "hostcc.py"), "ILANG_HIP_GENERATED_ONLY": "1",
-                "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1"})
+                "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1", "ILANG_HIP_UNCHECKED": "1"})
     env.update(extra_env)
     r = subprocess.run([sys.executable, str(SHIM / "run_cases.py")], env=env, capture_output=True, text=True, timeout=900)
     last = [l for l in r.stdout.splitlines() if l.startswith("CASE")][-1:] or ["(none started)"]
@@ -49,6 +51,39 @@ def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
     """Work-items run last to first: a dependency between work-items would change the result."""
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse"})
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
+
+
+def test_checked_accesses_give_the_same_results(shim_lib):
+    """The form the product emits by default: every access checked against its buffer's element count."""
+    run_cases(shim_lib, {"ILANG_HIP_UNCHECKED": "0"})
+
+
+def test_schedules_with_unsound_lowerings_cannot_fault(shim_lib):
+    """Schedules the reference accepts but lowers to loop nests that read past their buffers (a column reduction
+    recomputed under its consumer's loops over the reduced index: its tail guard mixes the loops of both stages;
+    found by random schedules on this emulation).  The reference reads heap garbage there; the generated kernels
+    check every access, so on a device this is a wrong result for a schedule that was wrong already, not a memory
+    fault.  Unchecked, each of these hits a guard page."""
+    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"), ILANG_HIP_GENERATED_ONLY="1",
+               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
+    code = """
+import sys
+import numpy as np
+from i_amd import Component as i, I
+cases = [(">ij~j|i:4:2,j:4|jij'i'i''", "ij-j~ij|i:4:2,j:4|jij'i'i''1", (13, 10)),
+         (">ij~j|i:2,j:3|jii'j'", "ij-j~ij|i:2,j:3|jii'1j'", (5, 6)),
+         ("+ij~j|i:8|ii'j", "ij-j~ij|i:8|ii'j1", (10, 9))]
+a, b, shape = cases[int(sys.argv[1])]
+x = np.random.default_rng(1).standard_normal(shape).astype(np.float32)
+out = ((I & i(a)) >> i(b)).exec_numpy(x)
+print("ran", out.shape == shape)
+"""
+    for n in range(3):
+        r = subprocess.run([sys.executable, "-c", code, str(n)], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300)
+        assert r.returncode == 0 and "ran True" in r.stdout, (n, r.returncode, r.stderr[-500:])
+        unchecked = subprocess.run([sys.executable, "-c", code, str(n)], env=dict(env, ILANG_HIP_UNCHECKED="1"),
+                                   capture_output=True, text=True, cwd=ROOT, timeout=300)
+        assert unchecked.returncode == -11, (n, unchecked.returncode)  # SIGSEGV on a guard page: the access is real
 
 
 def test_fixed_workspace_entry_matches_on_the_cpu(shim_lib):
