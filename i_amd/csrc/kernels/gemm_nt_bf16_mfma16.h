@@ -1,0 +1,218 @@
+// C[m,n] = sum_k A[m,k] * B[n,k]  (bf16 in, f32 accumulate, f32 or bf16 out) on gfx950, large-tile form on
+// v_mfma_f32_16x16x32_bf16.
+//
+// Same device form of the fused 𝚒 nest  i("ik*jk~ijk") >> i("+ijk~ij ... k0")  (README.md:16;
+// annotated-flashattn.c:57-89) as gemm_nt_bf16_direct.h, with the same slabs, the same global -> LDS transfers,
+// the same swizzle and the same workgroup -> tile mapping; what differs is the matrix instruction and what
+// follows from it.  On operands that toggle the datapath (anything but constants) the chip sustains more
+// 16x16x32 MFMAs per second than 32x32x16 ones under its power limit, at the same operand traffic from LDS.
+//
+//   workgroup   WM x WN waves; a wave owns (BT / WM) x (BT / WN) of the tile as TM x TN accumulators of
+//               16 x 16 (256 x 256 with 2 x 4 waves: 8 x 4 accumulators, 128 registers)
+//   operands    a lane holds 8 consecutive k of one row: row = lane % 16 of the 16-row fragment, 16-byte
+//               chunk 4 ks + lane / 16 of the 128-byte slab row (ks = 0, 1: two k-steps of 32 per slab).
+//               The 16 rows one quarter-wave reads with one ds_read_b128 fall into 16 different bank groups
+//               because the chunk is XOR-ed with (row / 2) % 8 on the way in.
+//   roles       the B rows are passed as the instruction's first operand and the A rows as its second, so
+//               a lane ends up with C[m = lane % 16][n = 4 (lane / 16) .. + 3] of each accumulator: four
+//               consecutive columns, one 16-byte (f32) or 8-byte (bf16) store
+//   registers   operand fragments are refilled in place: fragment i of A is reloaded with the next k-step's
+//               rows right after its last MFMA of this k-step; the B fragments alternate between two sets
+//   trips       as in gemm_nt_bf16_direct.h one trip runs from barrier to barrier, opens with the last k-step
+//               of the previous slab (operands carried across the barrier in registers) and requests slab
+//               s + 1 into the buffer that slab s - 1 has just left
+//   edges       a tile that lies wholly inside C (EDGE = false) steps from one wave-load to the next by a scalar
+//               add on the base address and keeps one per-lane offset; a tile that overhangs m or n
+//               (EDGE = true) re-reads the last valid row for the rows past the end, which makes the offset
+//               of every wave-load a per-lane value, recomputed at each request, and checks what it stores
+//   store       plain (cached) stores: the tile leaves through L2, and the write-back to memory overlaps
+//               whatever runs next
+// Requires k % 64 == 0.
+#pragma once
+#include <type_traits>
+
+#include "common.h"
+#include "params.h"
+
+template <int BT, int WM, int WN, bool EDGE>
+__device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* smem_base, uint32_t tm, uint32_t tn) {
+  constexpr int RB = 128;            // bytes per slab row: 64 k of bf16
+  constexpr int BK = 64;
+  constexpr int NWAVES = WM * WN;
+  constexpr int TM = BT / WM / 16;   // 16-row fragments of A per wave
+  constexpr int TN = BT / WN / 16;   // 16-row fragments of B per wave
+  constexpr int CH = RB / 16;        // 16-byte chunks per row
+  constexpr int RPW = 64 / CH;       // rows per wave-load
+  constexpr int SLAB = BT * RB;
+  constexpr int WL = SLAB / 1024;    // wave-loads per slab
+  constexpr int WLW = WL / NWAVES;
+  static_assert(WL % NWAVES == 0 && NWAVES % 2 == 0 && TM >= 2 && TN >= 2, "slab shape");
+  char (*smem)[2][SLAB] = reinterpret_cast<char (*)[2][SLAB]>(smem_base);  // [buffer][A, B]
+  const uint32_t batch = blockIdx.y;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  const uint32_t c16 = lane & 15, g = lane >> 4;
+
+  const size_t row_bytes = (size_t)p.k * 2;
+  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
+  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;
+  char* __restrict__ C = reinterpret_cast<char*>(p.c) + (size_t)batch * p.m * p.n * (p.out_bf16 ? 2 : 4);
+  const uint32_t m0 = tm * BT, n0 = tn * BT;
+
+  // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
+  // (row 8 w + lane / 8, chunk lane % 8) and it fetches chunk (lane % 8) ^ ((row / 2) % 8) of that row.
+  // w = wave + NWAVES it with NWAVES even, so (row / 2) % 8 = (4 (wave % 2) + lane / 16) % 8 for every `it`.
+  const uint32_t lrow = lane / CH, lch = lane % CH;
+  const uint32_t gch = lch ^ ((4 * (wave & 1) + lane / 16) % CH);
+  const uint32_t smem0 = lds_address(&smem[0][0][0]);
+  // Per-lane byte offset of this lane's 16 bytes from the first row of its wave-load.  EDGE: from the tile's
+  // first row, with the row clamped, recomputed at every request (held in registers it would cost 2 WLW of
+  // them; the empty asm keeps the compiler from hoisting the values back out of the loop).
+  const uint32_t rbase = wave * RPW + lrow, ch_bytes = 16 * gch;
+  const uint32_t voff0 = rbase * (uint32_t)row_bytes + ch_bytes;
+  const size_t it_stride = (size_t)(NWAVES * RPW) * row_bytes;  // bytes from one wave-load of a wave to its next
+  const uint32_t lim_a = p.m - 1 - m0, lim_b = p.n - 1 - n0;
+  auto row_offset = [&](int it, uint32_t lim) {
+    uint32_t r = rbase;
+    asm volatile("" : "+v"(r));
+    r += NWAVES * RPW * it;
+    return (r < lim ? r : lim) * (uint32_t)row_bytes + ch_bytes;
+  };
+  const char* a_tile = A + (size_t)m0 * row_bytes;
+  const char* b_tile = B + (size_t)n0 * row_bytes;
+  auto request = [&](uint32_t s, int buf, int r) {  // request r of the 2 WLW that bring slab s into `buf`
+    const int it = r % WLW;
+    const uint32_t w = wave + NWAVES * it;
+    const size_t k_byte = (size_t)s * RB;
+    const uint32_t to_a = smem0 + (2 * buf + 0) * SLAB + w * 1024, to_b = smem0 + (2 * buf + 1) * SLAB + w * 1024;
+    if constexpr (EDGE) {
+      if (r < WLW) dma16(a_tile + k_byte, row_offset(it, lim_a), to_a);
+      else dma16(b_tile + k_byte, row_offset(it, lim_b), to_b);
+    } else {
+      if (r < WLW) dma16(a_tile + k_byte + it * it_stride, voff0, to_a);
+      else dma16(b_tile + k_byte + it * it_stride, voff0, to_b);
+    }
+  };
+
+  // ---- LDS -> operands: row c16 of a 16-row fragment, chunk (4 ks + g) ^ ((row / 2) % 8); fragments start at
+  // multiples of 16 rows, which leaves (row / 2) % 8 = c16 / 2
+  uint32_t addr[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) addr[ks] = c16 * RB + 16 * ((4 * ks + g) ^ (c16 / 2));
+  const uint32_t a_rows = wm * TM * 16 * RB, b_rows = wn * TN * 16 * RB;
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const uint32_t nslabs = p.k / BK;
+#pragma unroll
+  for (int r = 0; r < 2 * WLW; ++r) request(0, 0, r);
+  dma_wait_all();
+  __syncthreads();
+
+  bf16x8 a[TM], b0[TN], b1[TN];
+  auto load_a = [&](int buf, int ks, int i) {
+    a[i] = *reinterpret_cast<const bf16x8*>(&smem[buf][0][0] + a_rows + i * 16 * RB + addr[ks]);
+  };
+  auto load_b = [&](int buf, int ks, int j, bf16x8 (&b)[TN]) {
+    b[j] = *reinterpret_cast<const bf16x8*>(&smem[buf][1][0] + b_rows + j * 16 * RB + addr[ks]);
+  };
+  // One k-step: TM x TN MFMAs on (a, bc) while a is refilled in place and bn is filled with the operands of
+  // k-step `ks` of buffer `buf`; `reqs` says whether the slab requests of this trip ride on it.
+  constexpr int NREQ = 2 * WLW, NSLOT = TM * TN;
+  auto kstep = [&](bf16x8 (&bc)[TN], bf16x8 (&bn)[TN], int buf, int ks, bool refill, auto reqs, uint32_t s_req, int req_buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bc[j], a[i], acc[i][j], 0, 0, 0);
+        const int slot = i * TN + j;
+        if (refill) {
+          if (i == 0) load_b(buf, ks, j, bn);
+          if (j == TN - 1) load_a(buf, ks, i);
+        }
+        if constexpr (decltype(reqs)::value) {
+#pragma unroll
+          for (int r = slot * NREQ / NSLOT; r < (slot + 1) * NREQ / NSLOT; ++r) request(s_req, req_buf, r);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  };
+  // Trip for slab s in buffer `buf`: the carried k-step (operands a, b0) while k-step 0 of slab s arrives in
+  // (a, b1) and slab s + 1 is requested; then k-step 0 while k-step 1 arrives in (a, b0), carried into the next
+  // trip.  The last trip has no successor; it requests its own slab once more into the other buffer, which
+  // nobody reads any more: one redundant slab per workgroup instead of a branch in every slot.
+  auto trip = [&](uint32_t s, int buf) {
+    const uint32_t s_req = s + 1 < nslabs ? s + 1 : s;
+    kstep(b0, b1, buf, 0, true, std::true_type{}, s_req, buf ^ 1);
+    kstep(b1, b0, buf, 1, true, std::false_type{}, 0, 0);
+    dma_wait_all();
+    __syncthreads();
+  };
+  // the first trip has no predecessor: its carried MFMAs add zero
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a[i] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b0[j] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+  uint32_t s = 0;
+  for (; s + 2 <= nslabs; s += 2) {  // two per iteration so that the buffer index is a constant
+    trip(s, 0);
+    trip(s + 1, 1);
+  }
+  if (s < nslabs) trip(s, 0);
+  // last k-step of the last slab
+  kstep(b0, b1, 0, 0, false, std::false_type{}, 0, 0);
+
+  // ---- store.  acc[i][j][r] is C[m0 + 16 (wm TM + i) + c16][n0 + 16 (wn TN + j) + 4 g + r]: a lane writes four
+  // consecutive columns at once, a quarter-wave 16 rows of them.  Columns come in fours, so a C whose n is not
+  // a multiple of 4 (or whose base is not 16-byte aligned) is stored element by element.
+  const bool n4 = p.n % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const uint32_t row = m0 + (wm * TM + i) * 16 + c16;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + (wn * TN + j) * 16 + 4 * g;
+      const size_t at = (size_t)row * p.n + col;
+      if (n4 && (!EDGE || (row < p.m && col < p.n))) {
+        if (p.out_bf16) {
+          bf16x4 v;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = (bf16_t)acc[i][j][r];
+          *reinterpret_cast<bf16x4*>(C + 2 * at) = v;
+        } else {
+          *reinterpret_cast<f32x4*>(C + 4 * at) = acc[i][j];
+        }
+      } else if (!EDGE || row < p.m) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (!EDGE || col + r < p.n) {
+            if (p.out_bf16) reinterpret_cast<bf16_t*>(C + 2 * at)[r] = (bf16_t)acc[i][j][r];
+            else reinterpret_cast<float*>(C + 4 * at)[r] = acc[i][j][r];
+          }
+      }
+    }
+  }
+}
+
+template <int BT, int WM, int WN>
+__device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
+  __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
+  // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
+  constexpr uint32_t SBM = 4, SBN = 8, SB = SBM * SBN;
+  const uint32_t nsb_m = (p.tiles_m + SBM - 1) / SBM, nsb_n = (p.tiles_n + SBN - 1) / SBN;
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t sb = (slot / SB) * 8u + xcd, within = slot % SB;
+  if (sb >= nsb_m * nsb_n) return;
+  const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
+  const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
+  if (tm >= p.tiles_m || tn >= p.tiles_n) return;
+  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false>(p, smem, tm, tn);
+  else gemm_nt_mfma16_tile<BT, WM, WN, true>(p, smem, tm, tn);
+}

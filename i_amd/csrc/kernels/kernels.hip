@@ -7,6 +7,7 @@
 #include "attention_f32.h"
 #include "gemm_nt_bf16.h"
 #include "gemm_nt_bf16_direct.h"
+#include "gemm_nt_bf16_mfma16.h"
 #include "row_softmax.h"
 
 // attn_fwd_bf16_d<D>_bn<BN>: d == dv == D exactly; ..._any: d, dv <= D (multiples of 8), guarded columns
@@ -62,11 +63,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64(Gem
 }
 
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct(GemmParams p) {
-  gemm_nt_direct_body<false, 256, 2, 4>(p);
+  gemm_nt_mfma16_body<256, 2, 4>(p);
 }
 // 128 x 128 tiles, 4 waves, two workgroups per CU: mid-size problems
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64_direct(GemmParams p) {
-  gemm_nt_direct_body<false, 128, 2, 2>(p);
+  gemm_nt_mfma16_body<128, 2, 2>(p);
 }
 // row-major right operand: c[m,n] = sum_k a[m,k] * b[k,n]
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nn_bf16_256x256x64_direct(GemmParams p) {
