@@ -409,6 +409,29 @@ def test_gemm_nt_bf16_output_in_bf16(env, monkeypatch, tile):
         assert_close(c32.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("out_bf16", [False, True])
+def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
+    """The direct kernels store four columns per lane when C allows it; a C that starts one element past a
+    16-byte boundary takes the element-wise stores instead.  The elements before and after C stay untouched."""
+    t = env.torch
+    bh, m, n, k = 2, 300, 260, 128
+    a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
+    ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
+    whole = t.full((bh * m * n + 2,), -7.0, device="cuda", dtype=t.bfloat16 if out_bf16 else t.float32)
+    cd = whole[1:-1]
+    assert cd.data_ptr() % 16 != 0
+    env.nat.check(env.nat.core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(),
+                                                      env.nat.BF16 if out_bf16 else env.nat.F32, bh, m, n, k, tile, tile,
+                                                      env.stream()))
+    t.cuda.synchronize()
+    assert whole[0].item() == -7.0 and whole[-1].item() == -7.0
+    ref = oracle.mm_t(a, b)
+    got = cd.float().cpu().numpy().reshape(bh, m, n)
+    assert_close(got, oracle.to_bf16_f32(ref) if out_bf16 else ref, RTOL_BF16)
+
+
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 264, 128), (2, 600, 520, 192), (1, 1, 8, 256),
                                       (3, 257, 248, 320), (1, 130, 1000, 64)])
 @pytest.mark.parametrize("direct", ["256", "128"])
