@@ -1,6 +1,8 @@
-// C[m,n] = sum_k A[m,k] * B[n,k]  (bf16 in, f32 accumulate and f32 out) on gfx950,
-// large-tile form: a 256 x 256 output tile per workgroup, K in slabs of 64, operand
-// slabs moved from global memory straight into LDS.
+// C[m,n] = sum_k A[m,k] * B[n,k]  (f32 accumulate and f32 out) on gfx950, large-tile form on 32 x 32
+// MFMAs: a 256 x 256 output tile per workgroup, K in slabs of 128 bytes per row, operand slabs moved from
+// global memory straight into LDS.  The kernels built from it are the f32-operand ones (F32 = true, see
+// below); bf16 operands run gemm_nt_bf16_mfma16.h, the same design on 16x16x32 MFMAs, which this description
+// of the bf16 form (F32 = false) is the reference point for.
 //
 // Device form of the fused 𝚒 nest  i("ik*jk~ijk") >> i("+ijk~ij ... k0")
 // (README.md:16; annotated-flashattn.c:57-89 shows the same pair with a tile-local
@@ -32,19 +34,10 @@
 #include "common.h"
 #include "params.h"
 
-// NN = true is the same kernel for a row-major right operand, C[m,n] = sum_k A[m,k] * B[k,n] (the reference's
-// test.py matmul  ik*kj~ijk  and the demo's standalone mm  ij*jk~ikj), bf16 only.  A B slab is then [64 k][BT n]:
-// rows of 2 BT bytes, of which one wave-load deposits 1 KiB (2 or 4 rows) contiguously.  The MFMA's B operand
-// wants 8 consecutive k for one n per lane, a column of the slab, which ds_read_b64_tr_b16 delivers: 16 lanes
-// read 4 rows x 32 bytes and each receives one column of it.  The 64-byte group index (one 32-column operand
-// tile of a row) is XOR-ed with row % 4 on the global side, so that the 4 rows a half-wave reads at once fall
-// into the 4 different 64-byte bank ranges.  Requires n % 8 == 0 besides k % 64 == 0.
-//
 // BT x BT output tile per workgroup of WM x WN waves: 256 with 2 x 4 waves (one workgroup per CU) for large
 // problems, 128 with 2 x 2 waves (two workgroups per CU) for problems with too few 256-tiles to fill the chip.
-template <bool F32, int BT, int WM, int WN, bool NN = false>
+template <bool F32, int BT, int WM, int WN>
 __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
-  static_assert(!(NN && F32), "the row-major right operand exists for bf16 only");
   constexpr int BMT = BT, BNT = BT;
   constexpr int ELEM = F32 ? 4 : 2;   // bytes per operand element
   constexpr int BK = 128 / ELEM;      // k per slab: 128-byte slab rows
@@ -79,7 +72,6 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   const int c = lane & 31, h = lane >> 5;
 
   const size_t row_bytes = (size_t)p.k * ELEM;
-  const size_t brow_bytes = (size_t)p.n * ELEM;  // NN: a row of B is n elements
   const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
   const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;  // n k = k n elements
   // (a bf16 output is addressed through the same pointer with half the element size)
@@ -103,25 +95,9 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
     aoff[it] = (ra - m0) * (uint32_t)row_bytes + 16 * gch;
     boff[it] = (rb - n0) * (uint32_t)row_bytes + 16 * gch;
   }
-  // NN: wave-load w of a B slab covers slab rows (k) RPWN w .. + RPWN - 1; this lane's LDS slot is (row, chunk
-  // lane % CHN) and it fetches chunk (lane % CHN) ^ 4 (row % 4) of that row; chunks that start past n re-read
-  // the row's last chunk (their columns are not stored).
-  constexpr int RBN = 2 * BNT;        // bytes per row of an NN slab
-  constexpr int CHN = RBN / 16;       // chunks per row
-  constexpr int RPWN = 1024 / RBN;    // rows per wave-load
-  if constexpr (NN) {
-    const uint32_t last_chunk = (p.n - n0) / 8 - 1;  // n % 8 == 0 and n0 < n
-#pragma unroll
-    for (int it = 0; it < WLW; ++it) {
-      const uint32_t r = (wave + NWAVES * it) * RPWN + lane / CHN;
-      uint32_t ch = (lane % CHN) ^ (4 * (r % 4));
-      ch = ch < last_chunk ? ch : last_chunk;
-      boff[it] = r * (uint32_t)brow_bytes + 16 * ch;
-    }
-  }
   const char* a_tile = A + (size_t)m0 * row_bytes;
-  const char* b_tile = NN ? B + (size_t)n0 * ELEM : B + (size_t)n0 * row_bytes;
-  const size_t b_slab_step = NN ? (size_t)BK * brow_bytes : (size_t)RB;  // bytes from one k slab of B to the next
+  const char* b_tile = B + (size_t)n0 * row_bytes;
+  const size_t b_slab_step = (size_t)RB;  // bytes from one k slab of B to the next
   auto request_slab = [&](uint32_t s, int buf) {
     const size_t k_byte = (size_t)s * RB;
 #pragma unroll
@@ -137,19 +113,7 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   uint32_t addr[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) addr[ks] = c * RB + 16 * ((2 * ks + h) ^ fr);
-  const uint32_t a_rows = wm * TM * 32 * RB, b_rows = NN ? 0u : wn * TN * 32 * RB;
-  // NN: 16-lane block b = lane / 16 covers columns 16 (b & 1) .. + 16 of a 32-column operand tile; lane 4 jj + q
-  // of the block points at row (k) 8 h + jj, columns 4 q .. + 4; a second read 4 rows further down completes
-  // the 8 consecutive k of the half-wave
-  typedef __attribute__((ext_vector_type(4))) short s16x4;
-  typedef __attribute__((ext_vector_type(8))) short s16x8;
-  typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
-  const uint32_t blk = lane >> 4, jj = (lane >> 2) & 3, qq = lane & 3;
-  uint32_t baddr[TN];  // per operand tile j: offset of (row 8 h + jj, this lane's 8 bytes) inside a 16-row k-step
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-    baddr[j] = (8 * h + jj) * RBN + 64 * ((wn * TN + j) ^ jj) + 32 * (blk & 1) + 8 * qq;
-
+  const uint32_t a_rows = wm * TM * 32 * RB, b_rows = wn * TN * 32 * RB;
   f32x16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -177,17 +141,7 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * RB + addr[ks]);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      if constexpr (NN) {
-        // rows 8 h + jj and 8 h + 4 + jj have the same row % 4, hence the same group swizzle
-        const char* ba = sb + 16 * ks * RBN + baddr[j];
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba + 4 * RBN));
-        f.b[j] = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      } else {
-        f.b[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
-      }
-    }
+    for (int j = 0; j < TN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
   };
   auto mfma = [&](const Frags& f, int i, int j) {
     if constexpr (F32) {

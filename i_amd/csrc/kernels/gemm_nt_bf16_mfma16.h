@@ -27,6 +27,18 @@
 //               of every wave-load a per-lane value, recomputed at each request, and checks what it stores
 //   store       plain (cached) stores: the tile leaves through L2, and the write-back to memory overlaps
 //               whatever runs next
+//
+// NN = true is the same kernel for a row-major right operand, C[m,n] = sum_k A[m,k] * B[k,n] (the reference's
+// test.py matmul  ik*kj~ijk  and the demo's standalone mm  ij*jk~ikj).  A B slab is then [64 k][BT n]: rows of
+// 2 BT bytes, of which one wave-load deposits 1 KiB (2 or 4 rows) contiguously, 16 slab rows per round of the
+// workgroup's wave-loads.  The instruction wants 8 consecutive k for one n per lane, a column of the slab,
+// which ds_read_b64_tr_b16 delivers: within a 16-lane block, lane 4 jj + q supplies the address of slab row
+// k0 + jj, columns 4 q .. + 4 of a 16-column fragment, and lane c receives column c of rows k0 .. k0 + 3; two
+// such reads (k0 = 32 ks + 8 (lane / 16) and + 4) complete the lane's 8 k.  Two 16-lane blocks read 8 rows x
+// 32 bytes at a time (rows 0-3 and 8-11 of a k-step, then 4-7 and 12-15, ...), so the 32-byte unit index of a
+// row is XOR-ed, on the global side, with f(row) = row % 4 + 4 ((row / 8) % 2), which sends those 8 rows to 8
+// different bank groups.  Requires n % 8 == 0 as well; 16-byte chunks that start past n re-read the row's last
+// chunk (their columns are not stored).
 // Requires k % 64 == 0.
 #pragma once
 #include <type_traits>
@@ -34,7 +46,7 @@
 #include "common.h"
 #include "params.h"
 
-template <int BT, int WM, int WN, bool EDGE>
+template <int BT, int WM, int WN, bool EDGE, bool NN>
 __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* smem_base, uint32_t tm, uint32_t tn) {
   constexpr int RB = 128;            // bytes per slab row: 64 k of bf16
   constexpr int BK = 64;
@@ -82,13 +94,31 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     return (r < lim ? r : lim) * (uint32_t)row_bytes + ch_bytes;
   };
   const char* a_tile = A + (size_t)m0 * row_bytes;
-  const char* b_tile = B + (size_t)n0 * row_bytes;
+  const char* b_tile = NN ? B + (size_t)n0 * 2 : B + (size_t)n0 * row_bytes;
+  // NN: wave-load w of a B slab covers slab rows (k) RPWN w .. + RPWN - 1; this lane's LDS slot is (row, chunk
+  // lane % CHN) and it fetches chunk (lane % CHN) ^ 2 f(row) of that row.  Rounds of wave-loads are 16 rows apart,
+  // which changes neither f(row) nor the clamp, so one per-lane offset serves every request.
+  constexpr int RBN = 2 * BT;         // bytes per row of an NN slab
+  constexpr int CHN = RBN / 16;       // chunks per row
+  constexpr int RPWN = 1024 / RBN;    // rows per wave-load
+  static_assert(!NN || NWAVES * RPWN == 16, "NN slab rounds");
+  const size_t brow_bytes = (size_t)p.n * 2;  // NN: a row of B is n elements
+  uint32_t boff_nn = 0;
+  if constexpr (NN) {
+    const uint32_t r = wave * RPWN + lane / CHN;
+    const uint32_t last_chunk = (p.n - n0) / 8 - 1;  // n % 8 == 0 and n0 < n
+    uint32_t ch = (lane % CHN) ^ (2 * ((r & 3) | (((r >> 3) & 1) << 2)));
+    ch = ch < last_chunk ? ch : last_chunk;
+    boff_nn = r * (uint32_t)brow_bytes + 16 * ch;
+  }
   auto request = [&](uint32_t s, int buf, int r) {  // request r of the 2 WLW that bring slab s into `buf`
     const int it = r % WLW;
     const uint32_t w = wave + NWAVES * it;
     const size_t k_byte = (size_t)s * RB;
     const uint32_t to_a = smem0 + (2 * buf + 0) * SLAB + w * 1024, to_b = smem0 + (2 * buf + 1) * SLAB + w * 1024;
-    if constexpr (EDGE) {
+    if (r >= WLW && NN) {
+      dma16(b_tile + ((size_t)s * BK + 16 * it) * brow_bytes, boff_nn, to_b);
+    } else if constexpr (EDGE) {
       if (r < WLW) dma16(a_tile + k_byte, row_offset(it, lim_a), to_a);
       else dma16(b_tile + k_byte, row_offset(it, lim_b), to_b);
     } else {
@@ -103,6 +133,16 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) addr[ks] = c16 * RB + 16 * ((4 * ks + g) ^ (c16 / 2));
   const uint32_t a_rows = wm * TM * 16 * RB, b_rows = wn * TN * 16 * RB;
+  // NN: lane 4 jj + qq of block g points at slab row 8 g + jj (+ 32 ks, + 4), columns 4 qq .. + 4 of fragment j;
+  // f(row) = jj + 4 (g % 2) for both reads of a lane
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+  const uint32_t jj = (lane >> 2) & 3, qq = lane & 3;
+  // (fragment j of the wave is unit wn TN + j = (wn TN) ^ j of the row, TN being a power of two that j stays below:
+  // the fragment's address is the first one's with 32 j XOR-ed in, one instruction instead of TN registers)
+  static_assert((TN & (TN - 1)) == 0, "fragments per wave");
+  const uint32_t baddr0 = NN ? (8 * g + jj) * RBN + 32 * ((uint32_t)(wn * TN) ^ (jj | ((g & 1) << 2))) + 8 * qq : 0u;
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -121,7 +161,16 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     a[i] = *reinterpret_cast<const bf16x8*>(&smem[buf][0][0] + a_rows + i * 16 * RB + addr[ks]);
   };
   auto load_b = [&](int buf, int ks, int j, bf16x8 (&b)[TN]) {
-    b[j] = *reinterpret_cast<const bf16x8*>(&smem[buf][1][0] + b_rows + j * 16 * RB + addr[ks]);
+    if constexpr (NN) {
+      uint32_t first = baddr0;
+      asm volatile("" : "+v"(first));  // (keeps the TN addresses from being hoisted into registers of their own)
+      const char* ba = &smem[buf][1][0] + 32 * ks * RBN + (first ^ (32u * j));
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba + 4 * RBN));
+      b[j] = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    } else {
+      b[j] = *reinterpret_cast<const bf16x8*>(&smem[buf][1][0] + b_rows + j * 16 * RB + addr[ks]);
+    }
   };
   // One k-step: TM x TN MFMAs on (a, bc) while a is refilled in place and bn is filled with the operands of
   // k-step `ks` of buffer `buf`; `reqs` says whether the slab requests of this trip ride on it.
@@ -201,7 +250,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   }
 }
 
-template <int BT, int WM, int WN>
+template <int BT, int WM, int WN, bool NN = false>
 __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
   // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
@@ -213,6 +262,6 @@ __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
   const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
   if (tm >= p.tiles_m || tn >= p.tiles_n) return;
-  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false>(p, smem, tm, tn);
-  else gemm_nt_mfma16_tile<BT, WM, WN, true>(p, smem, tm, tn);
+  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN>(p, smem, tm, tn);
+  else gemm_nt_mfma16_tile<BT, WM, WN, true, NN>(p, smem, tm, tn);
 }

@@ -71,10 +71,10 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64_dir
 }
 // row-major right operand: c[m,n] = sum_k a[m,k] * b[k,n]
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nn_bf16_256x256x64_direct(GemmParams p) {
-  gemm_nt_direct_body<false, 256, 2, 4, true>(p);
+  gemm_nt_mfma16_body<256, 2, 4, true>(p);
 }
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nn_bf16_128x128x64_direct(GemmParams p) {
-  gemm_nt_direct_body<false, 128, 2, 2, true>(p);
+  gemm_nt_mfma16_body<128, 2, 2, true>(p);
 }
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_direct(GemmParams p) {
   gemm_nt_direct_body<true, 128, 2, 2>(p);
