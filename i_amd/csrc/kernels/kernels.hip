@@ -5,6 +5,7 @@
 #include "attention_bf16_direct.h"
 #include "attention_bf16_q64.h"
 #include "attention_f32.h"
+#include "attention_f32_direct.h"
 #include "gemm_nt_bf16.h"
 #include "gemm_nt_bf16_direct.h"
 #include "gemm_nt_bf16_mfma16.h"
@@ -54,6 +55,13 @@ extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(
   extern "C" __global__ void __launch_bounds__(NW * 64) attn_fwd_f32_d##DPAD##_bn##BN(AttnParams p) { \
     attn_fwd_f32_body<DPAD, BN, NW>(p);                                                    \
   }
+// d == dv in {64, 128}, K and V tiles moved global -> LDS directly (attention_f32_direct.h)
+#define ATTN_F32_DIRECT(DPAD)                                                                                   \
+  extern "C" __global__ void __launch_bounds__(256, 2) attn_fwd_f32_d##DPAD##_bn32_direct(AttnParams p) {        \
+    attn_fwd_f32_direct_body<DPAD, 4>(p);                                                                       \
+  }
+ATTN_F32_DIRECT(64)
+ATTN_F32_DIRECT(128)
 ATTN_F32(32, 32, 4)
 ATTN_F32(64, 32, 4)
 ATTN_F32(128, 32, 4)

@@ -110,6 +110,38 @@ def test_attention_f32_online_rescale_stress(env):
     assert_close(gpu_attention(env, q, k, v, None, bf16=False), oracle.attention_tiled(q, k, v), RTOL_F32)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("direct", [True, False])
+def test_attention_f32_direct_and_staged_kernels_vs_oracle(env, monkeypatch, d, direct):
+    """f32 operands with d == dv in {64, 128} run the kernel that moves K/V tiles global -> LDS directly, everything
+    else (and ILANG_ATTN_NO_DIRECT=1) the register-staged one: both against the oracle on one tile, partial tiles,
+    several heads (more than the 8 XCDs), ragged query counts, negative and zero scales, and a longer key loop."""
+    if not direct:
+        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+    for bh, nq, nk, scale in ((1, 128, 32, 1.0), (3, 200, 333, 0.11), (2, 77, 130, -0.2), (9, 130, 64, 0.0), (1, 1, 1, 1.0),
+                              (2, 512, 1024, float(np.float32(1.0 / np.sqrt(d))))):
+        q, k, v = (rnd((bh, n, d), sd) for sd, n in ((1, nq), (2, nk), (3, nk)))
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=False), oracle.attention_tiled(q, k, v, scale), RTOL_F32)
+
+
+def test_attention_f32_operands_not_16_byte_aligned(env):
+    """The direct f32 kernel moves 16 bytes per lane; operands that start off a 16-byte boundary take the
+    register-staged kernel and give the same result."""
+    t = env.torch
+    bh, n, d = 2, 100, 64
+    q, k, v = (rnd((bh, n, d), sd) for sd in (1, 2, 3))
+    ref = oracle.attention_tiled(q, k, v, 0.3)
+    bufs = [t.zeros(bh * n * d + 1, device="cuda") for _ in range(4)]
+    views = [b[1:] for b in bufs]
+    for view, a in zip(views[:3], (q, k, v)):
+        view.copy_(t.from_numpy(a).reshape(-1))
+    assert all(x.data_ptr() % 16 != 0 for x in views)
+    env.nat.check(env.nat.core.i_hip_attention(views[0].data_ptr(), views[1].data_ptr(), views[2].data_ptr(), views[3].data_ptr(),
+                                               env.nat.F32, env.nat.F32, bh, n, n, d, d, 0.3, env.stream()))
+    t.cuda.synchronize()
+    assert_close(views[3].cpu().numpy().reshape(bh, n, d), ref, RTOL_F32)
+
+
 # ------------------------------------------------------------------ attention, bf16 in / f32 accumulate
 @pytest.mark.parametrize("bh,nq,nk,d", [(1, 64, 64, 64), (2, 128, 128, 128), (3, 200, 333, 128), (2, 77, 130, 64),
                                         (1, 512, 512, 64), (2, 100, 100, 40), (1, 1, 1, 8)])
