@@ -16,8 +16,9 @@ Prints ONE JSON line.  Besides the headline TFLOP/s it carries
                 bounded sample, with the GPU result checked against it
   secondary     row-softmax [16384,4096] f32 (HBM bound), mm_t 4096^3 bf16, the
                 long-sequence attention B1 H16 N32768 d64 (inputs x 2.0) and the
-                reference's own demo (attention f32 [512,64]), each with its own
-                roofline, cpu_baseline and rel_err
+                reference's own demo (attention f32 [512,64]) and the attention workload
+                in the reference's own arithmetic type (f32 operands, two of the eight
+                batches), each with its own roofline, cpu_baseline and rel_err
 
 Operands follow the recipe of the reference's scripts (NumPy default_rng(seed),
 seeds 1, 2, 3 for the first, second, third operand; ilang-python/flash-attn.py:33-35).
@@ -38,6 +39,7 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+PEAK_F32_TFLOPS = 157.3    # MI355X dense f32 MFMA
 # launches of the headline kernel before the W warm-up steps: the compile-and-first-run call plus 40 more.  The
 # launch time of a fresh process keeps falling over its first two dozen launches (2.2 ms -> 1.8 ms while the
 # clocks settle); this brings the device to that steady state whatever W is.
@@ -289,6 +291,16 @@ def main():
     _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), short_steps, short_warmup)
     c1_flop = 4.0 * 512 * 512 * 64
 
+    # ------------------------------------------------------------------ the attention workload in f32 (the reference's
+    # arithmetic type): batches 2 and 3 of the headline operands as f32, through the same compiled component
+    BF = 2
+    q32, k32, v32 = (t_[2:2 + BF].float() for t_ in (q, k, v))
+    out32 = torch.empty(BF, H, N, D, dtype=torch.float32, device=dev)
+    attn.into(out32, q32, k32, scale, v32)
+    f32_kernel = attn.report().split()[1]
+    _, f32_ms = time_steps(torch, lambda: attn.into(out32, q32, k32, scale, v32), max(args.steps // 5, 3), 2)
+    f32_tflops = 4.0 * BF * H * N * N * D / (f32_ms * 1e-3) / 1e12
+
     # What this box's matrix cores deliver to the vendor's own GEMM (torch.matmul -> hipBLASLt, bf16 in, bf16 out)
     # on the same operands as the mm_t line: a practical ceiling for dense bf16 on random data on this box, next to
     # which the MFMA lines can be read.  Not part of the product path; the shader clock under dense MFMA work on
@@ -304,8 +316,8 @@ def main():
         torch.cuda.synchronize()
 
     # ------------------------------------------------------------------ host legs: emitted C on one core, and the checks
-    cpu = cpu2 = cpu2w = cpu3 = cpu5 = cpu1 = None
-    err4 = err2 = err2w = err3 = err5 = err1 = None
+    cpu = cpu2 = cpu2w = cpu3 = cpu5 = cpu1 = cpuf = None
+    err4 = err2 = err2w = err3 = err5 = err1 = errf = None
     if not args.no_cpu_baseline:
         # C4: one (b, h) slice of the workload, 1024 of its 4096 query rows (query tiles and (b, h) pairs are the
         # outermost independent loops of the emitted nest, so the rate carries over to the whole workload)
@@ -338,6 +350,15 @@ def main():
             oracle, attn5, ops5, 4.0 * r5 * N5 * D5 / 1e12, "TFLOP/s",
             f"head {h5}, query rows 0..{r5 - 1} against all {N5} keys: 1/{H5 * N5 // r5} of the workload",
             out5[:, h5:h5 + 1, :r5].cpu().numpy())
+        # the f32 attention line: (b, h) = (3, 17) of the headline operands again, fewer rows (the emitted C does
+        # the same work per row whatever the operands' origin)
+        rf = 256
+        opsf = [q32[1:2, h0:h0 + 1, :rf].cpu().numpy(), k32[1:2, h0:h0 + 1].cpu().numpy(), np.float32(scale.item()),
+                v32[1:2, h0:h0 + 1].cpu().numpy()]
+        cpuf, errf = emitted_c_baseline(
+            oracle, attn, opsf, 4.0 * rf * N * D / 1e12, "TFLOP/s",
+            f"(b,h) = (3,{h0}), query rows 0..{rf - 1} against all {N} keys: 1/{BF * H * N // rf} of the workload",
+            out32[1:2, h0:h0 + 1, :rf].cpu().numpy())
         # C1: the whole workload; the reference's own committed emission when it was built, else the C emitted here
         got1 = dout.cpu().numpy()
         if oracle.have_ref():
@@ -402,6 +423,12 @@ def main():
              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,
              "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu1, "rel_err": err1},
+            {"workload": f"flash_attention_fwd B{BF} H32 N4096 d128 with f32 operands (batches 2 and 3 of the headline "
+                         "operands as f32, full f32 arithmetic: the reference's own type; not a BASELINE configuration)",
+             "value": f32_tflops, "unit": "TFLOP/s", "dtype": "f32",
+             "roofline": roof("mfma", f32_tflops, PEAK_F32_TFLOPS, "TFLOP/s", "flash_attention_B2_H32_N4096_d128_f32.md",
+                              f32_kernel, f32_ms),
+             "cpu_baseline": cpuf, "rel_err": errf},
         ],
     }
     print(json.dumps(line))

@@ -21,7 +21,8 @@ def test_committed_profile_summaries_give_the_traffic_figures():
     import bench
 
     for name in ("flash_attention_B8_H32_N4096_d128_bf16.md", "row_softmax_16384x4096_f32.md",
-                 "gemm_nt_4096x4096x4096_bf16.md", "flash_attention_B1_H16_N32768_d64_bf16.md"):
+                 "gemm_nt_4096x4096x4096_bf16.md", "flash_attention_B1_H16_N32768_d64_bf16.md",
+                 "flash_attention_B2_H32_N4096_d128_f32.md"):
         traffic = bench.measured_traffic(name)
         assert isinstance(traffic, int) and traffic > 0, name
     assert bench.measured_traffic("no_such_summary.md") is None
@@ -49,9 +50,12 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert rec["pre_warmup_launches"] == 41 and rec["rel_err"] <= 2e-2
     assert rec["roofline"]["kernel"] == "attn_fwd_bf16_d128_bn64_direct_w8"
     second = rec["secondary"]
-    assert len(second) == 5
-    for entry, bar in zip(second, (1e-4, 1e-4, 2e-2, 2e-2, 1e-4)):
+    assert len(second) == 6
+    for entry, bar in zip(second, (1e-4, 1e-4, 2e-2, 2e-2, 1e-4, 1e-4)):
         assert entry["cpu_baseline"]["value"] > 0 and entry["rel_err"] <= bar, entry["workload"]
+    f32_line = second[5]
+    assert f32_line["dtype"] == "f32" and f32_line["roofline"]["peak"] == 157.3
+    assert f32_line["roofline"]["kernel"] == "attn_fwd_f32_d128_bn32_direct"
     # the value is work over wall time of exactly `steps` calls
     flop = 4.0 * 8 * 32 * 4096 * 4096 * 128
     assert abs(rec["value"] - flop / (rec["ms_per_step"] * 1e-3) / 1e12) / rec["value"] < 1e-6
