@@ -165,10 +165,13 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       psum += e;
     }
     l_run = l_run * alpha + psum;
+    // (a factor of exactly 1 in every lane, the usual case once the row maxima have settled, changes nothing)
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+      for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o[t][i] *= alpha;
+    }
 
     // ---- O^T += V^T P^T, one key per half-wave and MFMA
 #pragma unroll
