@@ -2,9 +2,9 @@
 // v_mfma_f32_16x16x32_bf16.
 //
 // Same device form of the fused 𝚒 nest  i("ik*jk~ijk") >> i("+ijk~ij ... k0")  (README.md:16;
-// annotated-flashattn.c:57-89) as gemm_nt_bf16_direct.h, with the same slabs, the same global -> LDS transfers,
-// the same swizzle and the same workgroup -> tile mapping; what differs is the matrix instruction and what
-// follows from it.  On operands that toggle the datapath (anything but constants) the chip sustains more
+// annotated-flashattn.c:57-89) as gemm_nt_f32_direct.h (the f32-operand kernel, on 32 x 32 MFMAs), with the same
+// slabs, the same global -> LDS transfers, the same swizzle and the same workgroup -> tile mapping; what differs
+// is the matrix instruction and what follows from it.  On operands that toggle the datapath (anything but constants) the chip sustains more
 // 16x16x32 MFMAs per second than 32x32x16 ones under its power limit, at the same operand traffic from LDS.
 //
 //   workgroup   WM x WN waves; a wave owns (BT / WM) x (BT / WN) of the tile as TM x TN accumulators of
@@ -18,7 +18,7 @@
 //               consecutive columns, one 16-byte (f32) or 8-byte (bf16) store
 //   registers   operand fragments are refilled in place: fragment i of A is reloaded with the next k-step's
 //               rows right after its last MFMA of this k-step; the B fragments alternate between two sets
-//   trips       as in gemm_nt_bf16_direct.h one trip runs from barrier to barrier, opens with the last k-step
+//   trips       as in gemm_nt_f32_direct.h one trip runs from barrier to barrier, opens with the last k-step
 //               of the previous slab (operands carried across the barrier in registers) and requests slab
 //               s + 1 into the buffer that slab s - 1 has just left
 //   edges       a tile that lies wholly inside C (EDGE = false) steps from one wave-load to the next by a scalar

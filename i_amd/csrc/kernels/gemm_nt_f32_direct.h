@@ -1,45 +1,39 @@
-// C[m,n] = sum_k A[m,k] * B[n,k]  (f32 accumulate and f32 out) on gfx950, large-tile form on 32 x 32
-// MFMAs: a 256 x 256 output tile per workgroup, K in slabs of 128 bytes per row, operand slabs moved from
-// global memory straight into LDS.  The kernels built from it are the f32-operand ones (F32 = true, see
-// below); bf16 operands run gemm_nt_bf16_mfma16.h, the same design on 16x16x32 MFMAs, which this description
-// of the bf16 form (F32 = false) is the reference point for.
+// C[m,n] = sum_k A[m,k] * B[n,k]  for f32 operands (the reference's own arithmetic type; products and sums in
+// f32, f32 out) on gfx950, large-tile form on v_mfma_f32_32x32x2_f32: a 256 x 256 (or 128 x 128) output tile per
+// workgroup, K in slabs of 32, operand slabs moved from global memory straight into LDS.
 //
 // Device form of the fused 𝚒 nest  i("ik*jk~ijk") >> i("+ijk~ij ... k0")
 // (README.md:16; annotated-flashattn.c:57-89 shows the same pair with a tile-local
 // output): tile loops i, j -> workgroups, the k loop is sequential per workgroup,
-// i', j' -> MFMA lanes, and the product never exists outside a register.
+// i', j' -> MFMA lanes, and the product never exists outside a register.  bf16 operands run the same design on
+// 16x16x32 MFMAs (gemm_nt_bf16_mfma16.h).
 //
-//   workgroup   8 waves as 2 (m) x 4 (n); a wave owns 128 x 64 of the tile =
-//               4 x 2 accumulators of v_mfma_f32_32x32x16_bf16 (128 registers)
-//   slabs       A and B slabs are both [256 rows][64 k] bf16 = 128-byte rows.  One
+//   workgroup   8 waves as 2 (m) x 4 (n); a wave owns 128 x 64 of the tile = 4 x 2 accumulators of 32 x 32
+//               (128 registers)
+//   slabs       A and B slabs are both [256 rows][32 k] f32 = 128-byte rows.  One
 //               global_load_lds_dwordx4 of a wave deposits 8 rows (1 KiB) contiguously
 //               in LDS; the 16-byte chunk a lane fetches is XOR-ed with (row / 2) % 8 so
 //               that the 16 rows one quarter-wave reads for an MFMA operand fall into
 //               16 different bank groups.  Two slab buffers: slab s+1 is requested at the
 //               top of iteration s and awaited (vmcnt(0) + barrier) at its end.
-//   operands    both A rows and B rows are K-contiguous, so both MFMA operands are plain
-//               ds_read_b128 of (row, chunk 2 ks + h)
+//   operands    both A rows and B rows are K-contiguous, so both MFMA operands are plain ds_read_b128 of
+//               (row, chunk 2 ks + h).  The instruction's operands are one f32 per lane with k = lane / 32: a
+//               16-byte operand read covers k = 4 (2 ks + h) .. + 3, and element e of it feeds MFMA e of the k-step.
 //   L2          the workgroup ids that land on one XCD (id % 8) fill a block of 4 x 8
 //               tiles, so at any time an XCD streams 1024 rows of A and 2048 rows of B
 //   M, N edges  rows past the end re-read the last valid row and are not stored
-// Requires k % 64 == 0 (the launcher falls back to gemm_nt_bf16.h otherwise).
-//
-// F32 = true is the same kernel for f32 operands (the reference's own arithmetic type): slabs of 32 k
-// (again 128-byte rows, so layout, swizzle and transfers are unchanged) and v_mfma_f32_32x32x2_f32, whose
-// operands are one f32 per lane with k = lane / 32: a 16-byte operand read covers k = 4 (2 ks + h) .. + 3,
-// and element e of it feeds MFMA e of the k-step.  Products and sums stay f32.  Requires k % 32 == 0.
+// Requires k % 32 == 0.
 #pragma once
-#include <type_traits>
 
 #include "common.h"
 #include "params.h"
 
 // BT x BT output tile per workgroup of WM x WN waves: 256 with 2 x 4 waves (one workgroup per CU) for large
 // problems, 128 with 2 x 2 waves (two workgroups per CU) for problems with too few 256-tiles to fill the chip.
-template <bool F32, int BT, int WM, int WN>
-__device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
+template <int BT, int WM, int WN>
+__device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   constexpr int BMT = BT, BNT = BT;
-  constexpr int ELEM = F32 ? 4 : 2;   // bytes per operand element
+  constexpr int ELEM = 4;            // bytes per operand element
   constexpr int BK = 128 / ELEM;      // k per slab: 128-byte slab rows
   constexpr int NWAVES = WM * WN;
   constexpr int TM = BMT / WM / 32;  // 32-row accumulator tiles per wave
@@ -74,9 +68,7 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   const size_t row_bytes = (size_t)p.k * ELEM;
   const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
   const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;  // n k = k n elements
-  // (a bf16 output is addressed through the same pointer with half the element size)
-  float* __restrict__ C = reinterpret_cast<float*>(reinterpret_cast<char*>(p.c) +
-                                                   (size_t)batch * p.m * p.n * ((!F32 && p.out_bf16) ? 2 : 4));
+  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
   const uint32_t m0 = tm * BMT, n0 = tn * BNT;
 
   // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
@@ -135,22 +127,17 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   // MFMAs of the current one issue; the global -> LDS requests for slab s+1 (into the buffer slab s-1 has
   // just left) ride on the carried MFMAs.  Scheduling fences keep the order.
   struct Frags {
-    bf16x8 a[TM], b[TN];
+    f32x4 a[TM], b[TN];
   };
   auto fetch = [&](const char* sa, const char* sb, int ks, Frags& f) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * RB + addr[ks]);
+    for (int i = 0; i < TM; ++i) f.a[i] = *reinterpret_cast<const f32x4*>(sa + i * 32 * RB + addr[ks]);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * RB + addr[ks]);
+    for (int j = 0; j < TN; ++j) f.b[j] = *reinterpret_cast<const f32x4*>(sb + j * 32 * RB + addr[ks]);
   };
   auto mfma = [&](const Frags& f, int i, int j) {
-    if constexpr (F32) {
-      const f32x4 av = __builtin_bit_cast(f32x4, f.a[i]), bv = __builtin_bit_cast(f32x4, f.b[j]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[e], bv[e], acc[i][j], 0, 0, 0);
-    } else {
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
-    }
+    for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][e], f.b[j][e], acc[i][j], 0, 0, 0);
   };
   constexpr int NREQ = 2 * WLW;  // slab requests per wave and trip, dealt out over the TM * TN carried MFMAs
   // The last trip has no successor; it requests its own slab once more into the other buffer, which nobody
@@ -196,9 +183,9 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   };
   Frags ca, cb;  // the first trip has no predecessor: its carried MFMAs add zero
 #pragma unroll
-  for (int i = 0; i < TM; ++i) ca.a[i] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+  for (int i = 0; i < TM; ++i) ca.a[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int j = 0; j < TN; ++j) ca.b[j] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+  for (int j = 0; j < TN; ++j) ca.b[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   uint32_t s = 0;
   for (; s + 2 <= nslabs; s += 2) {  // two per trip so that the buffer index is a constant
     step(s, 0, ca, cb);
@@ -217,24 +204,15 @@ __device__ __forceinline__ void gemm_nt_direct_body(const GemmParams& p) {
   // ---- store.  Accumulator layout: column n = c, rows 8 (e / 4) + 4 h + e % 4: every store instruction
   // writes two full 128-byte lines.  C is written once and not read again: non-temporal.
   const bool interior = m0 + BMT <= p.m && n0 + BNT <= p.n;
-  auto store_tile = [&](auto out_is_bf16) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const uint32_t col = n0 + (wn * TN + j) * 32 + c;
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + (wn * TN + j) * 32 + c;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-          if (interior || (row < p.m && col < p.n)) {
-            if constexpr (decltype(out_is_bf16)::value)
-              __builtin_nontemporal_store((bf16_t)acc[i][j][e], &reinterpret_cast<bf16_t*>(C)[(size_t)row * p.n + col]);
-            else __builtin_nontemporal_store(acc[i][j][e], &C[(size_t)row * p.n + col]);
-          }
-        }
+      for (int e = 0; e < 16; ++e) {
+        const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+        if (interior || (row < p.m && col < p.n)) __builtin_nontemporal_store(acc[i][j][e], &C[(size_t)row * p.n + col]);
       }
-  };
-  // bf16 output (bf16 operands only): the f32 sums are rounded on the way out, half the bytes
-  if (!F32 && p.out_bf16) store_tile(std::true_type{});
-  else store_tile(std::false_type{});
+    }
 }

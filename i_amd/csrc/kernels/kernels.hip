@@ -7,7 +7,7 @@
 #include "attention_f32.h"
 #include "attention_f32_direct.h"
 #include "gemm_nt_bf16.h"
-#include "gemm_nt_bf16_direct.h"
+#include "gemm_nt_f32_direct.h"
 #include "gemm_nt_bf16_mfma16.h"
 #include "row_softmax.h"
 
@@ -85,11 +85,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nn_bf16_128x128x64_dir
   gemm_nt_mfma16_body<128, 2, 2, true>(p);
 }
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_direct(GemmParams p) {
-  gemm_nt_direct_body<true, 128, 2, 2>(p);
+  gemm_nt_f32_direct_body<128, 2, 2>(p);
 }
 // f32 operands, f32 MFMA: the arithmetic type of the reference
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_direct(GemmParams p) {
-  gemm_nt_direct_body<true, 256, 2, 4>(p);
+  gemm_nt_f32_direct_body<256, 2, 4>(p);
 }
 
 // row_<op>_wave_{v,s}<NV> and row_<op>_block for op = softmax, shift (x - row max), norm (x / row sum), exp
