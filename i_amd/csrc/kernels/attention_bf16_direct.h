@@ -66,7 +66,12 @@
 // PRECISE: the score scale is applied in f32 to every score (the reference's arithmetic,
 // compiler/src/lower/exec_plan_to_module.rs:605-640) instead of being folded into Q with one more bf16 rounding;
 // the steady state then keeps a reference for its exponentials at either head size.  About 5 % slower.
-template <int DPAD, int BN, int NWAVES, bool PRECISE = false>
+//
+// PADDED: d == dv = p.d is any multiple of 8 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a lane whose
+// 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before the first
+// transfer, so the columns d .. DPAD - 1 of K and V read as zeros for the whole kernel (Q is padded with zeros in
+// its registers; the output columns past d are not stored).  Global rows are 2 p.d bytes apart.
+template <int DPAD, int BN, int NWAVES, bool PRECISE = false, bool PADDED = false>
 __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int BM = 32 * NWAVES;
   constexpr int KSTEPS = DPAD / 16;       // k-steps of the QK^T contraction
@@ -92,11 +97,13 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31;  // query column within the wave / A-operand row
   const int h = lane >> 5;  // half-wave
-  constexpr uint32_t d = DPAD;
+  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;  // elements per row in global memory
+  const uint32_t RBG = 2 * d;                         // ... and bytes (RB when not PADDED)
+  const uint32_t chunks = d / 8;                      // 16-byte chunks per global row
 
   const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)head * p.nq * d;
-  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RB;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RB;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBG;
 
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
@@ -131,7 +138,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
     u32x4 z = {0, 0, 0, 0};
-    if (qrow < p.nq) z = ldg128(Q + (size_t)qrow * d + 16 * ks + 8 * h);
+    if (qrow < p.nq && (!PADDED || (uint32_t)(16 * ks + 8 * h) < d)) z = ldg128(Q + (size_t)qrow * d + 16 * ks + 8 * h);
     if constexpr (QSCALE) {
       bf16x8 scaled = __builtin_bit_cast(bf16x8, z);
 #pragma unroll
@@ -165,30 +172,42 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int KSTRIDE = NWAVES * RPW / RPB;  // swizzle steps between consecutive wave-loads of a wave
   static_assert((KSTRIDE & (KSTRIDE - 1)) == 0 && (KSTRIDE % CH == 0 || CH % KSTRIDE == 0), "swizzle period");
   static_assert((NWAVES * RPW / RPB) % (CH / 4) == 0, "V swizzle period");
+  static_assert(!PADDED || KSTRIDE % CH == 0, "PADDED needs the per-lane chunk to be the same for every wave-load");
   const uint32_t lane_row = wave * RPW + lrow;
-  const uint32_t koff_lane = lrow * RB + 16 * (lch ^ ((lane_row / RPB) % CH));
-  const uint32_t voff_lane = lrow * RB + 16 * (lch ^ (4 * ((lane_row / RPB) % (CH / 4))));
+  const uint32_t kch_lane = lch ^ ((lane_row / RPB) % CH), vch_lane = lch ^ (4 * ((lane_row / RPB) % (CH / 4)));
+  const uint32_t koff_lane = lrow * RBG + 16 * kch_lane;
+  const uint32_t voff_lane = lrow * RBG + 16 * vch_lane;
+  // a transfer of 16 bytes per lane; PADDED: only by the lanes whose chunk exists in the global row
+  auto dma16_chunk = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t chunk) {
+    if constexpr (PADDED) {
+      if (chunk < chunks) dma16(base, voff, lds_base);
+    } else {
+      dma16(base, voff, lds_base);
+    }
+  };
   // one wave-load of a full tile: `it` of K (want_k) or of V
   auto request_full_one = [&](uint32_t tile, int buf, int it, auto want_k) {
     const uint32_t w = wave + NWAVES * it;
-    const size_t byte0 = (size_t)tile * TILE_BYTES + w * 1024;
+    const size_t byte0 = PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024;
     if constexpr (decltype(want_k)::value)
-      dma16(K + byte0, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
-    else dma16(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+      dma16_chunk(K + byte0, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024,
+                  kch_lane);
+    else dma16_chunk(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch_lane);
   };
 
   // one wave-load of K of any tile index: full tile, partial tile (rows past nk re-read the last row), or none
   auto request_k_one = [&](uint32_t tile, int buf, int it) {
     if (tile < nfull_tiles) {
       const uint32_t w = wave + NWAVES * it;
-      dma16(K + (size_t)tile * TILE_BYTES + w * 1024, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)),
-            smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+      dma16_chunk(K + (PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024),
+                  koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane);
     } else if (tile * BN < p.nk) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;
       uint32_t key = tile * BN + row;
       key = key < p.nk ? key : p.nk - 1;
-      dma16(K, key * RB + 16 * (lch ^ ((row / RPB) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+      const uint32_t kch = lch ^ ((row / RPB) % CH);
+      dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
     }
   };
 
@@ -203,8 +222,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const uint32_t vch = lch ^ (4 * ((row / RPB) % (CH / 4)));
       uint32_t key = key0 + row;
       if constexpr (PARTIAL) key = key < p.nk ? key : p.nk - 1;
-      if constexpr (decltype(want_k)::value) dma16(K, key * RB + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
-      if constexpr (decltype(want_v)::value) dma16(V, key * RB + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+      if constexpr (decltype(want_k)::value) dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
+      if constexpr (decltype(want_v)::value) dma16_chunk(V, key * RBG + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch);
     }
   };
 
@@ -538,6 +557,12 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   };
 
   // tiles 0 and 1 of K and tile 0 of V into LDS, then S(0)
+  if constexpr (PADDED) {
+    // the tile memory, cleared once: what no transfer ever writes (the columns past d) then reads as zero
+    for (uint32_t at = 16 * tid; at < 4 * TILE_BYTES; at += 16 * 64 * NWAVES)
+      *reinterpret_cast<u32x4*>(&smem[0][0][0] + at) = u32x4{0, 0, 0, 0};
+    __syncthreads();
+  }
   auto first_tiles = [&]() {
     request_k(0, 0);
     request_v(0, 0);
@@ -664,7 +689,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           bf16x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(o[t][4 * g + e] * inv);
-          *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
     } else if constexpr (!STAGED_STORE) {
       float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * d;
@@ -675,7 +700,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           f32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
-          *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
     }
   }
@@ -713,7 +738,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
         for (int it = 0; it < 8; ++it) {
           const uint32_t r = 4 * it + (lane >> 4), q = lane & 15;
           const f32x4 w = *reinterpret_cast<const f32x4*>(stage + r * 256 + 16 * (q ^ (r & 15)));
-          if (r < rows_valid) *reinterpret_cast<f32x4*>(O + (size_t)r * d + 64 * half + 4 * q) = w;
+          if (r < rows_valid && (!PADDED || 64 * half + 4 * q < d)) *reinterpret_cast<f32x4*>(O + (size_t)r * d + 64 * half + 4 * q) = w;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }

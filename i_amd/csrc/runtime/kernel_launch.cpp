@@ -48,9 +48,22 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
+  // any other d == dv that is a multiple of 8 below 128: the same kernels with their LDS rows padded to 64 or 128
+  // columns (the f32-scale form excepted: the register-staged kernels multiply in f32 as it is)
+  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 128 && !options.f32_scale;
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
-  const bool direct = exact && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
-  if (direct) {
+  const bool direct = (exact || padded) && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+  if (direct && padded) {
+    // 64-key tiles; 256 query rows per workgroup on the grids where the unpadded kernels take them, else 128
+    if (query_tile == 256 || (query_tile != 128 && bh * ((nq + 255) / 256) >= 2 * 256 && nk >= 2560 &&
+                              10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128)))
+      bm = 256;
+    if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
+      const int waves = std::atoi(w);
+      if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8 for a padded head size";
+      bm = 32u * (unsigned)waves;
+    }
+  } else if (direct) {
     const bool tile_known = query_tile == 64 || query_tile == 128 || query_tile == 256;
     if (key_tile == 32 && !options.f32_scale && tile_known && !(d == 64 && query_tile == 256)) bn = 32;
     if (tile_known && !(options.f32_scale && query_tile == 64)) bm = (unsigned)query_tile;  // the schedule's i split
@@ -91,10 +104,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
       name = "attn_fwd_bf16_d64_bn32_q64";
       threads = bm;
     } else if (direct) {
-      name = "attn_fwd_bf16_d" + std::to_string(d) + "_bn" + std::to_string(bn) + "_direct";
+      name = "attn_fwd_bf16_d" + std::to_string(padded ? (d < 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
       if (bm == 64) name += "_w2";
       if (bm == 256) name += "_w8";
       if (options.f32_scale) name += "_f32scale";
+      if (padded) name += "_pad";
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   } else {

@@ -153,6 +153,41 @@ def test_attention_bf16_vs_oracle(env, bh, nq, nk, d):
     assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
 
 
+@pytest.mark.parametrize("d", [8, 24, 40, 56, 72, 80, 96, 112, 120])
+@pytest.mark.parametrize("waves", ["4", "8", "staged"])
+def test_attention_bf16_head_sizes_between_the_kernel_sizes(env, monkeypatch, d, waves):
+    """d == dv that is a multiple of 8 but neither 64 nor 128 runs the direct-to-LDS kernels with LDS rows padded to
+    64 or 128 columns (4 and 8 waves per workgroup forced in turn; "staged": the register-staged kernel these
+    shapes used to take).  Short and long key loops (the steady state needs four full tiles), partial tiles, ragged
+    query counts, more heads than XCDs, both output types."""
+    if waves == "staged":
+        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+    else:
+        monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    for bh, nq, nk in ((1, 64, 64), (3, 200, 333), (9, 130, 700), (2, 300, 1024)):
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True), ref, RTOL_BF16)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
+
+
+def test_attention_bf16_padded_head_size_keeps_its_neighbours_untouched(env):
+    """The padded kernels store only the first d columns of an output row: the next row's first elements and the
+    element after the last row stay as they were (checked with a guard element around a d = 72 output)."""
+    t = env.torch
+    bh, nq, nk, d = 2, 150, 400, 72
+    q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
+    qd, kd, vd = (t.from_numpy(a).cuda().bfloat16().contiguous() for a in (q, k, v))
+    whole = t.full((bh * nq * d + 8,), -7.0, device="cuda")
+    od = whole[4:-4]
+    env.nat.check(env.nat.core.i_hip_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), od.data_ptr(), env.nat.BF16,
+                                               env.nat.F32, bh, nq, nk, d, d, 0.1, env.stream()))
+    t.cuda.synchronize()
+    assert (whole[:4] == -7.0).all().item() and (whole[-4:] == -7.0).all().item()
+    assert_close(od.cpu().numpy().reshape(bh, nq, d), oracle.attention_tiled(q, k, v, 0.1), RTOL_BF16)
+
+
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("force", [None, "waves8", "q64", "staged"])
 def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
