@@ -27,13 +27,18 @@
 //
 // Requires d == dv == DPAD, 16-byte aligned operands and nk * d * 4 < 2^32 (the launcher falls back to
 // attention_f32.h otherwise).  4 waves (128 queries) per workgroup, two workgroups per CU.
+//
+// PADDED: d == dv = p.d is any multiple of 4 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a lane whose
+// 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before the first
+// transfer, so the columns d .. DPAD - 1 of K and V read as zeros for the whole kernel (Q is padded with zeros in
+// its registers; the output columns past d are not stored).  Global rows are 4 p.d bytes apart.
 #pragma once
 #include <type_traits>
 
 #include "common.h"
 #include "params.h"
 
-template <int DPAD, int NWAVES>
+template <int DPAD, int NWAVES, bool PADDED = false>
 __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   constexpr int BN = 32;
   constexpr int BM = 32 * NWAVES;
@@ -58,11 +63,13 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t c = lane & 31;  // query column within the wave / A-operand row
   const uint32_t h = lane >> 5;  // half-wave
-  constexpr uint32_t d = DPAD;
+  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;  // elements per row in global memory
+  const uint32_t RBG = 4 * d;                         // ... and bytes (RB when not PADDED)
+  const uint32_t chunks = d / 4;                      // 16-byte chunks per global row
 
   const float* __restrict__ Q = reinterpret_cast<const float*>(p.q) + (size_t)head * p.nq * d;
-  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RB;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RB;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBG;
 
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const float qsign = scale_raw < 0.0f ? -1.0f : 1.0f;  // negative scale folded into Q (exact)
@@ -80,10 +87,17 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       const uint32_t row = w * RPW + lrow;  // row within the tile
       uint32_t key = tile * BN + row;
       key = key < p.nk ? key : p.nk - 1;
-      dma16(K, key * RB + 16 * (lch ^ (row % 16)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
-      dma16(V, key * RB + 16 * (lch ^ (8 * ((row >> 2) & 1))), smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+      const uint32_t kch = lch ^ (row % 16), vch = lch ^ (8 * ((row >> 2) & 1));
+      if (!PADDED || kch < chunks) dma16(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
+      if (!PADDED || vch < chunks) dma16(V, key * RBG + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
     }
   };
+  if constexpr (PADDED) {
+    // the tile memory, cleared once: what no transfer ever writes (the columns past d) then reads as zero
+    for (uint32_t at = 16 * tid; at < 4 * TILE_BYTES; at += 16 * 64 * NWAVES)
+      *reinterpret_cast<u32x4*>(&smem[0][0][0] + at) = u32x4{0, 0, 0, 0};
+    __syncthreads();
+  }
   request_tile(0, 0);
 
   // Q^T fragments (B operand): lane (c, h) holds q[row][8 g + 4 h + e] in element e of group g
@@ -92,7 +106,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
 #pragma unroll
   for (int g = 0; g < KG; ++g) {
     f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (qrow < p.nq) z = *reinterpret_cast<const f32x4*>(Q + (size_t)qrow * d + 8 * g + 4 * h);
+    if (qrow < p.nq && (!PADDED || (uint32_t)(8 * g + 4 * h) < d)) z = *reinterpret_cast<const f32x4*>(Q + (size_t)qrow * d + 8 * g + 4 * h);
     qf[g] = z * qsign;
   }
 
@@ -199,7 +213,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
         f32x4 w;
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
-        *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+        if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
       }
   }
 }

@@ -71,6 +71,13 @@ extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(
   }
 ATTN_F32_DIRECT(64)
 ATTN_F32_DIRECT(128)
+// ... head sizes below DPAD that are multiples of 4: LDS rows padded with zeros
+#define ATTN_F32_DIRECT_PAD(DPAD)                                                                               \
+  extern "C" __global__ void __launch_bounds__(256, 2) attn_fwd_f32_d##DPAD##_bn32_direct_pad(AttnParams p) {    \
+    attn_fwd_f32_direct_body<DPAD, 4, true>(p);                                                                 \
+  }
+ATTN_F32_DIRECT_PAD(64)
+ATTN_F32_DIRECT_PAD(128)
 ATTN_F32(32, 32, 4)
 ATTN_F32(64, 32, 4)
 ATTN_F32(128, 32, 4)

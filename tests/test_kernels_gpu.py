@@ -110,12 +110,13 @@ def test_attention_f32_online_rescale_stress(env):
     assert_close(gpu_attention(env, q, k, v, None, bf16=False), oracle.attention_tiled(q, k, v), RTOL_F32)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 36, 60, 96, 100, 124])
 @pytest.mark.parametrize("direct", [True, False])
 def test_attention_f32_direct_and_staged_kernels_vs_oracle(env, monkeypatch, d, direct):
-    """f32 operands with d == dv in {64, 128} run the kernel that moves K/V tiles global -> LDS directly, everything
-    else (and ILANG_ATTN_NO_DIRECT=1) the register-staged one: both against the oracle on one tile, partial tiles,
-    several heads (more than the 8 XCDs), ragged query counts, negative and zero scales, and a longer key loop."""
+    """f32 operands with d == dv that is a multiple of 4 above 32 run the kernel that moves K/V tiles global -> LDS directly
+    (with its LDS rows padded when d is neither 64 nor 128), everything else (and ILANG_ATTN_NO_DIRECT=1) the
+    register-staged one: both against the oracle on one tile, partial tiles, several heads (more than the 8 XCDs),
+    ragged query counts, negative and zero scales, and a longer key loop."""
     if not direct:
         monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
     for bh, nq, nk, scale in ((1, 128, 32, 1.0), (3, 200, 333, 0.11), (2, 77, 130, -0.2), (9, 130, 64, 0.0), (1, 1, 1, 1.0),
