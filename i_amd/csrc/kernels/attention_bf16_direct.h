@@ -13,11 +13,12 @@
 //                   rows would collide in the banks.  The 16-byte chunk index is
 //                   XOR-ed with a function of the row, applied on the GLOBAL side
 //                   (a lane chooses which chunk it fetches for its fixed LDS slot):
-//                     K: chunk ^= (row / RPB) % CH          16 consecutive rows, same
+//                     K: chunk ^= (row / RPB) % KMOD        16 consecutive rows, same
 //                                                           chunk -> 16 different bank groups
-//                     V: chunk ^= 4 * ((row / RPB) % (CH/4)) 4 consecutive rows, same
+//                     V: chunk ^= 4 * ((row / RPB) % VMOD)  4 consecutive rows, same
 //                                                           64-byte group -> 4 different groups
-//                   (RPB = rows per 256 bytes, CH = chunks per row).
+//                   (RPB = rows per 256 bytes, at least 1; KMOD = 16 / RPB and VMOD = 4 / RPB: the chunks and the
+//                   64-byte groups of the 256-byte bank window that a row can be sent to).
 //   LDS -> K operand  ds_read_b128 of row (32 kt + c), chunk (2 ks + h): the A operand of
 //                   v_mfma_f32_32x32x16_bf16 exactly as in attention_bf16.h.
 //   LDS -> V operand  V stays row-major [key][dv]; ds_read_b64_tr_b16 transposes while
@@ -79,12 +80,14 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int DT = DPAD / 32;           // 32-column output tiles
   constexpr int RB = 2 * DPAD;            // bytes per K/V row
   constexpr int CH = RB / 16;             // 16-byte chunks per row (= lanes per row of a wave-load)
-  constexpr int RPB = 256 / RB;           // rows per 256 bytes
+  constexpr int RPB = RB >= 256 ? 1 : 256 / RB;  // rows per 256 bytes (1 for longer rows, which start at the same banks)
+  constexpr int KMOD = 16 / RPB;          // K swizzle: values of the chunk XOR
+  constexpr int VMOD = 4 / RPB;           // V swizzle: values of the 64-byte group XOR
   constexpr int RPW = 64 / CH;            // rows per wave-load
   constexpr int TILE_BYTES = BN * RB;
   constexpr int WL = TILE_BYTES / 1024;   // wave-loads per tile
   constexpr int WLW = WL / NWAVES;        // ... per wave
-  static_assert(RB == 128 || RB == 256, "row size");
+  static_assert(RB == 128 || RB == 256 || RB == 512, "row size");
   static_assert(WL % NWAVES == 0 && WLW >= 1, "tile / wave shape");
   __shared__ __attribute__((aligned(1024))) char smem[2][2][TILE_BYTES];  // [buffer][K, V]
 
@@ -123,7 +126,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // fell below 2^-100; if any wave of the workgroup did, the workgroup throws the pass away and computes the item
   // again with the general loop, which takes the running max tile by tile.
   constexpr bool PRESCALE = DPAD == 64 && !PRECISE;
-  constexpr bool NOREF = DPAD == 128 && ATTN_NOREF && !PRECISE;
+  constexpr bool NOREF = DPAD >= 128 && ATTN_NOREF && !PRECISE;
   constexpr bool QSCALE = PRESCALE || NOREF;
   // f32 output written through LDS (see the epilogue): 8 KiB of tile memory per wave
   constexpr bool STAGED_STORE = ATTN_STAGED_STORE && NWAVES * 8192 <= 4 * TILE_BYTES;
@@ -167,16 +170,22 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // For a full tile the per-lane part of the address is the same for every tile, and for every wave-load when
   // the NWAVES * RPW rows between a wave's consecutive wave-loads are a multiple of the swizzle period.  With
   // fewer waves (KSTRIDE < CH) the K swizzle of wave-load `it` differs from that of wave-load 0 in the bits
-  // (KSTRIDE * it) % CH, which the rows of one wave-load (fewer than KSTRIDE swizzle steps) never reach: one
+  // (KSTRIDE * it) % KMOD, which the rows of one wave-load (fewer than KSTRIDE swizzle steps) never reach: one
   // XOR with a constant.  Everything else that varies is wave-uniform and is folded into the scalar base address.
   constexpr int KSTRIDE = NWAVES * RPW / RPB;  // swizzle steps between consecutive wave-loads of a wave
-  static_assert((KSTRIDE & (KSTRIDE - 1)) == 0 && (KSTRIDE % CH == 0 || CH % KSTRIDE == 0), "swizzle period");
-  static_assert((NWAVES * RPW / RPB) % (CH / 4) == 0, "V swizzle period");
-  static_assert(!PADDED || KSTRIDE % CH == 0, "PADDED needs the per-lane chunk to be the same for every wave-load");
+  static_assert((KSTRIDE & (KSTRIDE - 1)) == 0 && (KSTRIDE % KMOD == 0 || KMOD % KSTRIDE == 0), "swizzle period");
+  static_assert((NWAVES * RPW / RPB) % VMOD == 0, "V swizzle period");
   const uint32_t lane_row = wave * RPW + lrow;
-  const uint32_t kch_lane = lch ^ ((lane_row / RPB) % CH), vch_lane = lch ^ (4 * ((lane_row / RPB) % (CH / 4)));
+  const uint32_t kch_lane = lch ^ ((lane_row / RPB) % KMOD), vch_lane = lch ^ (4 * ((lane_row / RPB) % VMOD));
   const uint32_t koff_lane = lrow * RBG + 16 * kch_lane;
   const uint32_t voff_lane = lrow * RBG + 16 * vch_lane;
+  // K offset of wave-load `it`: the chunk of wave-load 0 with the constant XOR-ed in.  (On the byte offset itself
+  // when the row part cannot reach the chunk bits, i.e. when rows are a power of two long: not PADDED.)
+  auto koff_of = [&](int it) {
+    const uint32_t x = (uint32_t)(KSTRIDE * it) % KMOD;
+    if constexpr (PADDED) return lrow * RBG + 16 * (kch_lane ^ x);
+    else return koff_lane ^ (16u * x);
+  };
   // a transfer of 16 bytes per lane; PADDED: only by the lanes whose chunk exists in the global row
   auto dma16_chunk = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t chunk) {
     if constexpr (PADDED) {
@@ -190,8 +199,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     const uint32_t w = wave + NWAVES * it;
     const size_t byte0 = PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024;
     if constexpr (decltype(want_k)::value)
-      dma16_chunk(K + byte0, koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024,
-                  kch_lane);
+      dma16_chunk(K + byte0, koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024,
+                  kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD));
     else dma16_chunk(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch_lane);
   };
 
@@ -200,13 +209,13 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     if (tile < nfull_tiles) {
       const uint32_t w = wave + NWAVES * it;
       dma16_chunk(K + (PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024),
-                  koff_lane ^ (16u * ((uint32_t)(KSTRIDE * it) % CH)), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane);
+                  koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD));
     } else if (tile * BN < p.nk) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;
       uint32_t key = tile * BN + row;
       key = key < p.nk ? key : p.nk - 1;
-      const uint32_t kch = lch ^ ((row / RPB) % CH);
+      const uint32_t kch = lch ^ ((row / RPB) % KMOD);
       dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
     }
   };
@@ -218,8 +227,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     for (int it = 0; it < WLW; ++it) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;  // row within the tile
-      const uint32_t kch = lch ^ ((row / RPB) % CH);
-      const uint32_t vch = lch ^ (4 * ((row / RPB) % (CH / 4)));
+      const uint32_t kch = lch ^ ((row / RPB) % KMOD);
+      const uint32_t vch = lch ^ (4 * ((row / RPB) % VMOD));
       uint32_t key = key0 + row;
       if constexpr (PARTIAL) key = key < p.nk ? key : p.nk - 1;
       if constexpr (decltype(want_k)::value) dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
@@ -229,14 +238,14 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 
   // ---- LDS -> operands: per-lane byte offsets inside a tile
   // K: row c (+ 32 kt), chunk (2 ks + h) ^ fk, where fk depends on c only
-  const uint32_t fk = (c / RPB) % CH;
+  const uint32_t fk = (c / RPB) % KMOD;
   uint32_t kaddr[KSTEPS];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) kaddr[ks] = c * RB + 16 * ((2 * ks + h) ^ fk);
   // V: 16-lane block b = lane / 16 covers columns 16 (b & 1) .. +16 of a 32-column tile; lane 4 jj + q of
   // the block points at key (4 h + jj), columns 4 q .. +4
   const uint32_t blk = lane >> 4, jj = (lane >> 2) & 3, qq = lane & 3;
-  const uint32_t gv = 4 * (((4 * h + jj) / RPB) % (CH / 4));
+  const uint32_t gv = 4 * (((4 * h + jj) / RPB) % VMOD);
   uint32_t vaddr[DT];
 #pragma unroll
   for (int t = 0; t < DT; ++t)

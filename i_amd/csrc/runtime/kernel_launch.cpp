@@ -14,8 +14,11 @@ constexpr size_t kMaxGrid = 0x7fffffffu;
 bool fits_u32(size_t v) { return v <= 0xffffffffull; }
 }  // namespace
 
-bool attention_supported(DType in_dtype, size_t d, size_t dv) {
-  if (d == 0 || dv == 0 || d > 128 || dv > 128) return false;
+bool attention_supported(DType in_dtype, size_t d, size_t dv, bool f32_scale) {
+  if (d == 0 || dv == 0) return false;
+  // head sizes above 128 up to 256: bf16, d == dv, on the direct kernels only (scale folded into Q)
+  if (d > 128 || dv > 128)
+    return in_dtype == BF16 && d == dv && d <= 256 && d % 8 == 0 && !f32_scale && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
   return true;
 }
@@ -23,8 +26,10 @@ bool attention_supported(DType in_dtype, size_t d, size_t dv) {
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options, LaunchNote* note) {
-  if (!attention_supported(in_dtype, d, dv))
-    return "attention kernel: unsupported operands (need 0 < d, dv <= 128; bf16 needs d, dv % 8 == 0)";
+  if (!attention_supported(in_dtype, d, dv, options.f32_scale))
+    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d == dv <= 256 without the f32-scale "
+           "form; bf16 needs d, dv % 8 == 0)";
+  if (d > 128 && nk * d * 2 >= (size_t(1) << 32)) return "attention kernel: too many keys for a head size above 128";
   if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
   if (in_dtype == F32 && out_dtype != F32) return "attention kernel: f32 inputs produce f32 output";
   if (bh == 0 || nq == 0) return {};
@@ -50,10 +55,14 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
   // any other d == dv that is a multiple of 8 below 128: the same kernels with their LDS rows padded to 64 or 128
   // columns (the f32-scale form excepted: the register-staged kernels multiply in f32 as it is)
-  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 128 && !options.f32_scale;
+  const bool wide = in_dtype == BF16 && d == dv && d > 128;  // (supported: d <= 256, a multiple of 8, scale folded into Q)
+  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 256 && !options.f32_scale;
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
-  const bool direct = (exact || padded) && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
-  if (direct && padded) {
+  const bool direct = (exact || padded || wide) && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+  if (direct && wide) {
+    bm = 128;  // 4 waves, one per SIMD
+    bn = 32;
+  } else if (direct && padded) {
     // 64-key tiles; 256 query rows per workgroup on the grids where the unpadded kernels take them, else 128
     if (query_tile == 256 || (query_tile != 128 && bh * ((nq + 255) / 256) >= 2 * 256 && nk >= 2560 &&
                               10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128)))
@@ -104,11 +113,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
       name = "attn_fwd_bf16_d64_bn32_q64";
       threads = bm;
     } else if (direct) {
-      name = "attn_fwd_bf16_d" + std::to_string(padded ? (d < 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
+      name = "attn_fwd_bf16_d" + std::to_string(wide ? 256 : padded ? (d < 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
       if (bm == 64) name += "_w2";
       if (bm == 256) name += "_w8";
       if (options.f32_scale) name += "_f32scale";
-      if (padded) name += "_pad";
+      if (padded && d != 256) name += "_pad";
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   } else {

@@ -120,23 +120,30 @@ def test_reference_demo_flash_and_naive_attention(torch):
         assert np.allclose(got, ref, rtol=3e-4, atol=5e-5, equal_nan=True)  # the demo's own tolerance
 
 
-def test_head_sizes_above_128_run_as_three_hand_written_kernels(torch):
-    """d or dv above 128 (the demo's own shape is [32, 2048], flash-attn.py:31-36): scores by the MFMA GEMM, row
-    softmax in place, output by the MFMA GEMM.  f32 at the demo's shape against the emitted C; bf16 with batch axes,
-    a score scale and ragged query counts at d = 192 and d = 256 (dv = 160) against the oracle."""
+def test_head_sizes_above_128(torch):
+    """bf16 with d == dv up to 256 runs the fused kernel for 256-column rows (padded when d < 256).  Everything else
+    above 128 (f32, the demo's own shape [32, 2048] of flash-attn.py:31-36; d != dv; the f32-scale form) runs as three
+    hand-written kernels: scores by the MFMA GEMM, row softmax in place, output by the MFMA GEMM.  f32 at the demo's
+    shape against the emitted C; bf16 with batch axes, a score scale and ragged query counts against the oracle."""
     q, k, v = rnd((32, 2048), 1), rnd((32, 2048), 2), rnd((32, 2048), 3)
     comp = flash()
     got = comp.exec_numpy(q, k, v)
     assert "attention in three kernels" in comp.report() and "gemm_nt_f32" in comp.report()
     close(got, oracle.compile_component(comp.handle).run(q, k, v), RTOL_F32)
-    for d, dv, nq, nk in ((192, 192, 300, 512), (256, 160, 77, 136)):
+    for d, dv, nq, nk, fused, f32_scale in ((192, 192, 300, 512, True, False), (256, 256, 130, 700, True, False),
+                                            (256, 160, 77, 136, False, False), (192, 192, 300, 512, False, True)):
         qb, kb, vb = (oracle.to_bf16_f32(rnd(shape, seed)) for seed, shape in
                       ((1, (2, 3, nq, d)), (2, (2, 3, nk, d)), (3, (2, 3, nk, dv))))
         scale = np.float32(1.0 / np.sqrt(d))
         comp = flash("i:128,j:64", prefix="bh", scaled=True)
+        if f32_scale:
+            comp.option("attention.f32_scale", 1)
         out = comp.exec_torch(torch.from_numpy(qb).cuda().bfloat16(), torch.from_numpy(kb).cuda().bfloat16(),
                               torch.tensor(scale, device="cuda"), torch.from_numpy(vb).cuda().bfloat16())
-        assert "attention in three kernels" in comp.report() and "scaled_softmax" in comp.report()
+        if fused:
+            assert "attn_fwd_bf16_d256_bn32_direct" + ("_pad" if d < 256 else "") + " " in comp.report() + " "
+        else:
+            assert "attention in three kernels" in comp.report() and "scaled_softmax" in comp.report()
         close(out.cpu().numpy(), oracle.attention_tiled(qb, kb, vb, scale), RTOL_BF16)
     # extents the GEMM kernels cannot take (f32 with a key count that is no multiple of 32) still run generated
     q, k, v = rnd((20, 160), 1), rnd((33, 160), 2), rnd((33, 160), 3)

@@ -189,6 +189,20 @@ def test_attention_bf16_padded_head_size_keeps_its_neighbours_untouched(env):
     assert_close(od.cpu().numpy().reshape(bh, nq, d), oracle.attention_tiled(q, k, v, 0.1), RTOL_BF16)
 
 
+@pytest.mark.parametrize("d", [136, 160, 192, 224, 256])
+def test_attention_bf16_head_sizes_above_128(env, d):
+    """d == dv in 136 .. 256 (multiples of 8) runs the direct-to-LDS kernel for 256-column rows: one wave per SIMD,
+    32-key tiles, LDS rows padded when d < 256.  One tile, partial tiles, long key loops (the steady state needs four
+    full tiles), ragged query counts, more heads than XCDs, both output types, and scores large enough that the pass
+    without a reference overflows and the second pass takes over."""
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    for bh, nq, nk, amp in ((1, 32, 32, 1.0), (3, 200, 333, 1.0), (9, 130, 700, 1.0), (2, 300, 1024, 1.0), (2, 128, 512, 4.0)):
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s) * np.float32(a)) for s, n, a in ((1, nq, amp), (2, nk, amp), (3, nk, 1.0)))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True), ref, RTOL_BF16 if amp == 1.0 else 6e-2)
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16 if amp == 1.0 else 6e-2)
+
+
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("force", [None, "waves8", "q64", "staged"])
 def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
