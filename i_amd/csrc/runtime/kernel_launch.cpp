@@ -46,6 +46,10 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   //     key loops when that still leaves at least two workgroups per CU and does not pad nq by much, else 128.
   //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512 x 32): the
   //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs.
+  //   d == dv any other multiple of 8 below 128: the 4- and 8-wave kernels with 64-key tiles and their LDS rows
+  //     padded to 64 or 128 columns (not in the f32-scale form).
+  //   d == dv a multiple of 8 above 128 up to 256: the kernel for 256-column rows (padded below 256), 4 waves, one
+  //     per SIMD, 32-key tiles; nothing else exists above 128, so callers ask attention_supported() first.
   //   otherwise: register-staged kernel with guarded columns (always multiplies the scores in f32)
   // ILANG_ATTN_WAVES=2|4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
   // d == 64 only) and ILANG_ATTN_NO_DIRECT=1 forces the register-staged kernel; both exist so that tests can
@@ -53,8 +57,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
-  // any other d == dv that is a multiple of 8 below 128: the same kernels with their LDS rows padded to 64 or 128
-  // columns (the f32-scale form excepted: the register-staged kernels multiply in f32 as it is)
+  // (the f32-scale form excepted: the register-staged kernels multiply in f32 as it is)
   const bool wide = in_dtype == BF16 && d == dv && d > 128;  // (supported: d <= 256, a multiple of 8, scale folded into Q)
   const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 256 && !options.f32_scale;
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
