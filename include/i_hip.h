@@ -77,8 +77,11 @@ int i_exec_into_device_noalloc(const i_program* program,
  * the fused kernel for  mm_t >> [scale] >> row_max_shift >> exp >> row_normalize >> mm
  * (reference emission of the same component: ilang-python/annotated-flashattn.c:52-310,
  * `f0`).  q [bh,nq,d], k [bh,nk,d], v [bh,nk,dv], o [bh,nq,dv], row-major.
- * in_dtype applies to q/k/v, out_dtype to o.  Requires 0 < d,dv <= 128, a finite
- * scale, and d,dv multiples of 8 for bf16.
+ * in_dtype applies to q/k/v, out_dtype to o.  Requires a finite scale and 0 < d,dv <= 128
+ * (bf16: d,dv multiples of 8), or bf16 with d == dv <= 256.  bf16 with d == dv runs the
+ * direct-to-LDS kernels at every such head size (64 and 128 exactly, the others with
+ * zero-padded LDS rows); f32 with d == dv a multiple of 4 from 36 to 128 and 16-byte
+ * aligned operands runs the f32 kernel of the same design.
  */
 int i_hip_attention(const void* q, const void* k, const void* v, void* o,
                     int in_dtype, int out_dtype,
@@ -92,7 +95,8 @@ int i_hip_attention(const void* q, const void* k, const void* v, void* o,
  * any other request leaves the choice to the launcher.  f32_scale != 0 applies the score scale in f32 to every
  * score, the reference's arithmetic (compiler/src/lower/exec_plan_to_module.rs:605-640), instead of folding
  * scale * log2(e) into Q with one more bf16 rounding: about 5 % slower, and the error against an f32 computation
- * no longer grows with the magnitude of the scores.  f32 operands and the other bf16 kernels always multiply in f32.
+ * no longer grows with the magnitude of the scores.  f32 operands and the other bf16 kernels always multiply in f32;
+ * head sizes above 128 have no f32-scale form (-1).
  */
 int i_hip_attention_ex(const void* q, const void* k, const void* v, void* o,
                        int in_dtype, int out_dtype,
