@@ -424,6 +424,12 @@ def test_attention_rejects_unsupported(env):
     rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, 60, 60,
                                       1.0, env.stream())
     assert rc == -1  # bf16 rows must be 16-byte multiples
+    # above 128: bf16 with d == dv <= 256 only, and not in the f32-scale form
+    xb = t.zeros(1, 8, 320, device="cuda", dtype=t.bfloat16)
+    for d, dv, f32_scale in ((192, 128, 0), (264, 264, 0), (192, 192, 1)):
+        rc = env.nat.core.i_hip_attention_ex(xb.data_ptr(), xb.data_ptr(), xb.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, d, dv,
+                                             1.0, 0, 0, f32_scale, env.stream())
+        assert rc == -1 and "unsupported" in env.nat.last_error(), (d, dv, f32_scale)
 
 
 def test_attention_negative_and_zero_scale(env):
