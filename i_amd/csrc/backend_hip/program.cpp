@@ -132,8 +132,8 @@ struct Run {
 };
 
 // ---------------------------------------------------------------- hand-written kernels
-// Head sizes beyond the fused attention kernels (d or dv above 256, above 128 for f32 operands, d != dv or the
-// f32-scale form above 128; the reference's demo uses 2048,
+// Head sizes beyond the fused attention kernels (d or dv above 256, above 128 for f32 operands or d != dv; the
+// reference's demo uses 2048,
 // ilang-python/flash-attn.py:31-36) run as three hand-written kernels with the score matrix in memory:
 // S = Q K^T (MFMA GEMM), P = softmax(scale * S) row by row in place, O = P V (MFMA GEMM).  What the GEMM kernels
 // need of the extents decides whether that is possible; the score matrix may take up to 16 GiB.
@@ -158,8 +158,7 @@ bool hand_usable(const Run& run, const Recognized& r) {
       if (run.dtype_of(r.b.buffer) != t || run.dtype_of(r.c.buffer) != t) return false;
       const auto q = rows_cols(r.a), v = rows_cols(r.c);
       if (q.size() < 2 || v.size() < 2) return false;
-      if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back(), run.p.attention_f32_scale.load()))
-        return true;
+      if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back())) return true;
       const auto k = rows_cols(r.b);
       if (k.size() < 2) return false;
       size_t bh = 1;
@@ -284,7 +283,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
         if (ihip::Err e = run.read_f32(r.scale.buffer, &sp); !e.empty()) return e;
         scale_ptr = static_cast<const float*>(sp);
       }
-      if (!ihip::attention_supported(bf16 ? ihip::BF16 : ihip::F32, dq, dv, run.p.attention_f32_scale.load()))
+      if (!ihip::attention_supported(bf16 ? ihip::BF16 : ihip::F32, dq, dv))
         return attention_in_parts(run, r, bf16, bh, nq, nk, dq, dv, scale_ptr, note);
       void* out = nullptr;
       ihip::DType out_dt = ihip::F32;

@@ -47,17 +47,23 @@ ATTN_BF16_DIRECT(128, 64, 8, 1, _w8_f32scale, true)
 ATTN_BF16_DIRECT(64, 64, 4, 2, _f32scale, true)
 ATTN_BF16_DIRECT(64, 64, 8, 1, _w8_f32scale, true)
 // head sizes below DPAD that are multiples of 8: LDS rows padded with zeros
-#define ATTN_BF16_DIRECT_PAD(DPAD, BN, NW, OCC, SUFFIX)                                                          \
+#define ATTN_BF16_DIRECT_PAD(DPAD, BN, NW, OCC, SUFFIX, PRECISE)                                                 \
   extern "C" __global__ void __launch_bounds__(NW * 64, OCC) attn_fwd_bf16_d##DPAD##_bn##BN##_direct##SUFFIX##_pad(AttnParams p) { \
-    attn_fwd_bf16_direct_body<DPAD, BN, NW, false, true>(p);                                                      \
+    attn_fwd_bf16_direct_body<DPAD, BN, NW, PRECISE, true>(p);                                                    \
   }
-ATTN_BF16_DIRECT_PAD(128, 64, 4, 2, )
-ATTN_BF16_DIRECT_PAD(128, 64, 8, 1, _w8)
-ATTN_BF16_DIRECT_PAD(64, 64, 4, 2, )
-ATTN_BF16_DIRECT_PAD(64, 64, 8, 1, _w8)
+ATTN_BF16_DIRECT_PAD(128, 64, 4, 2, , false)
+ATTN_BF16_DIRECT_PAD(128, 64, 8, 1, _w8, false)
+ATTN_BF16_DIRECT_PAD(64, 64, 4, 2, , false)
+ATTN_BF16_DIRECT_PAD(64, 64, 8, 1, _w8, false)
+ATTN_BF16_DIRECT_PAD(128, 64, 4, 2, _f32scale, true)
+ATTN_BF16_DIRECT_PAD(128, 64, 8, 1, _w8_f32scale, true)
+ATTN_BF16_DIRECT_PAD(64, 64, 4, 2, _f32scale, true)
+ATTN_BF16_DIRECT_PAD(64, 64, 8, 1, _w8_f32scale, true)
 // head sizes above 128 up to 256: one wave per SIMD (all its registers), 128 query rows per workgroup, 32-key tiles
 ATTN_BF16_DIRECT(256, 32, 4, 1, , false)
-ATTN_BF16_DIRECT_PAD(256, 32, 4, 1, )
+ATTN_BF16_DIRECT_PAD(256, 32, 4, 1, , false)
+ATTN_BF16_DIRECT(256, 32, 4, 1, _f32scale, true)
+ATTN_BF16_DIRECT_PAD(256, 32, 4, 1, _f32scale, true)
 // d = 64 with 64 queries per wave (attention_bf16_q64.h): 8 waves, 512 query rows per workgroup, 32-key tiles
 extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(AttnParams p) {
   attn_fwd_bf16_q64_body<64, 32, 8>(p);

@@ -14,11 +14,11 @@ constexpr size_t kMaxGrid = 0x7fffffffu;
 bool fits_u32(size_t v) { return v <= 0xffffffffull; }
 }  // namespace
 
-bool attention_supported(DType in_dtype, size_t d, size_t dv, bool f32_scale) {
+bool attention_supported(DType in_dtype, size_t d, size_t dv) {
   if (d == 0 || dv == 0) return false;
-  // head sizes above 128 up to 256: bf16, d == dv, on the direct kernels only (scale folded into Q)
+  // head sizes above 128 up to 256: bf16, d == dv, on the direct kernels only
   if (d > 128 || dv > 128)
-    return in_dtype == BF16 && d == dv && d <= 256 && d % 8 == 0 && !f32_scale && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+    return in_dtype == BF16 && d == dv && d <= 256 && d % 8 == 0 && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
   return true;
 }
@@ -26,9 +26,8 @@ bool attention_supported(DType in_dtype, size_t d, size_t dv, bool f32_scale) {
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options, LaunchNote* note) {
-  if (!attention_supported(in_dtype, d, dv, options.f32_scale))
-    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d == dv <= 256 without the f32-scale "
-           "form; bf16 needs d, dv % 8 == 0)";
+  if (!attention_supported(in_dtype, d, dv))
+    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d == dv <= 256; bf16 needs d, dv % 8 == 0)";
   if (d > 128 && nk * d * 2 >= (size_t(1) << 32)) return "attention kernel: too many keys for a head size above 128";
   if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
   if (in_dtype == F32 && out_dtype != F32) return "attention kernel: f32 inputs produce f32 output";
@@ -47,7 +46,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512 x 32): the
   //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs.
   //   d == dv any other multiple of 8 below 128: the 4- and 8-wave kernels with 64-key tiles and their LDS rows
-  //     padded to 64 or 128 columns (not in the f32-scale form).
+  //     padded to 64 or 128 columns.
   //   d == dv a multiple of 8 above 128 up to 256: the kernel for 256-column rows (padded below 256), 4 waves, one
   //     per SIMD, 32-key tiles; nothing else exists above 128, so callers ask attention_supported() first.
   //   otherwise: register-staged kernel with guarded columns (always multiplies the scores in f32)
@@ -57,9 +56,8 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
-  // (the f32-scale form excepted: the register-staged kernels multiply in f32 as it is)
-  const bool wide = in_dtype == BF16 && d == dv && d > 128;  // (supported: d <= 256, a multiple of 8, scale folded into Q)
-  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 256 && !options.f32_scale;
+  const bool wide = in_dtype == BF16 && d == dv && d > 128;  // (supported: d <= 256, a multiple of 8)
+  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 256;
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
   const bool direct = (exact || padded || wide) && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct && wide) {

@@ -34,8 +34,7 @@ struct AttentionOptions {
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options = {}, LaunchNote* note = nullptr);
-// (f32_scale: the caller wants the score scale applied in f32, which the kernels for head sizes above 128 do not do)
-bool attention_supported(DType in_dtype, size_t d, size_t dv, bool f32_scale = false);
+bool attention_supported(DType in_dtype, size_t d, size_t dv);
 
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, a and b bf16, sums in f32; c is f32, or bf16 (out_dtype) with the sums rounded on the way out
 // tile_m x tile_n is the output tile the schedule asks for (0 = no preference): 256 x 256 and 128 x 128 select

@@ -95,8 +95,7 @@ int i_hip_attention(const void* q, const void* k, const void* v, void* o,
  * any other request leaves the choice to the launcher.  f32_scale != 0 applies the score scale in f32 to every
  * score, the reference's arithmetic (compiler/src/lower/exec_plan_to_module.rs:605-640), instead of folding
  * scale * log2(e) into Q with one more bf16 rounding: about 5 % slower, and the error against an f32 computation
- * no longer grows with the magnitude of the scores.  f32 operands and the other bf16 kernels always multiply in f32;
- * head sizes above 128 have no f32-scale form (-1).
+ * no longer grows with the magnitude of the scores.  f32 operands and the other bf16 kernels always multiply in f32.
  */
 int i_hip_attention_ex(const void* q, const void* k, const void* v, void* o,
                        int in_dtype, int out_dtype,

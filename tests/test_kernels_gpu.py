@@ -321,10 +321,11 @@ def test_attention_bf16_large_scores_error_growth(env, monkeypatch, d, waves):
         assert err <= bound, f"inputs x {amp}: error {err} > {bound}"
 
 
-@pytest.mark.parametrize("d,tile", [(128, 128), (128, 256), (64, 128), (64, 256)])
+@pytest.mark.parametrize("d,tile", [(128, 128), (128, 256), (64, 128), (64, 256), (96, 128), (96, 256), (40, 128), (40, 256),
+                                    (192, 128), (256, 128)])
 def test_attention_bf16_f32_scale_keeps_the_bar_at_any_score_magnitude(env, d, tile):
     """f32_scale: the score scale multiplies every score in f32 (the reference's arithmetic) and Q is not rounded a
-    second time.  Same inputs as above, x 1, x 2 and x 3: the error stays inside the 2e-2 bar, and does not grow
+    second time (head sizes 64 and 128, and the padded and the 256-column kernels for the others).  Same inputs as above, x 1, x 2 and x 3: the error stays inside the 2e-2 bar, and does not grow
     with the magnitude of the scores the way the folded form's does."""
     bh, nq, nk = 2, 200, 1100
     for amp in (1.0, 2.0, 3.0):
@@ -424,9 +425,9 @@ def test_attention_rejects_unsupported(env):
     rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, 60, 60,
                                       1.0, env.stream())
     assert rc == -1  # bf16 rows must be 16-byte multiples
-    # above 128: bf16 with d == dv <= 256 only, and not in the f32-scale form
+    # above 128: bf16 with d == dv <= 256 only
     xb = t.zeros(1, 8, 320, device="cuda", dtype=t.bfloat16)
-    for d, dv, f32_scale in ((192, 128, 0), (264, 264, 0), (192, 192, 1)):
+    for d, dv, f32_scale in ((192, 128, 0), (264, 264, 0), (136, 256, 1)):
         rc = env.nat.core.i_hip_attention_ex(xb.data_ptr(), xb.data_ptr(), xb.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, d, dv,
                                              1.0, 0, 0, f32_scale, env.stream())
         assert rc == -1 and "unsupported" in env.nat.last_error(), (d, dv, f32_scale)
