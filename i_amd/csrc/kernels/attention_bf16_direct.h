@@ -68,10 +68,11 @@
 // compiler/src/lower/exec_plan_to_module.rs:605-640) instead of being folded into Q with one more bf16 rounding;
 // the steady state then keeps a reference for its exponentials at either head size.  About 5 % slower.
 //
-// PADDED: d == dv = p.d is any multiple of 8 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a lane whose
-// 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before the first
-// transfer, so the columns d .. DPAD - 1 of K and V read as zeros for the whole kernel (Q is padded with zeros in
-// its registers; the output columns past d are not stored).  Global rows are 2 p.d bytes apart.
+// PADDED: d = p.d and dv = p.dv are any multiples of 8 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a
+// lane whose 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before
+// the first transfer, so the columns d .. DPAD - 1 of K and dv .. DPAD - 1 of V read as zeros for the whole kernel
+// (Q is padded with zeros in its registers; the output columns past dv are not stored).  Global rows of Q and K are
+// 2 p.d bytes apart, those of V 2 p.dv (and those of O p.dv elements).
 template <int DPAD, int BN, int NWAVES, bool PRECISE = false, bool PADDED = false>
 __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   constexpr int BM = 32 * NWAVES;
@@ -100,13 +101,14 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31;  // query column within the wave / A-operand row
   const int h = lane >> 5;  // half-wave
-  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;  // elements per row in global memory
-  const uint32_t RBG = 2 * d;                         // ... and bytes (RB when not PADDED)
-  const uint32_t chunks = d / 8;                      // 16-byte chunks per global row
+  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;    // elements per row of Q and K in global memory
+  const uint32_t dv = PADDED ? p.dv : (uint32_t)DPAD;  // ... of V and O
+  const uint32_t RBG = 2 * d, RBGV = 2 * dv;            // bytes per global row of K, of V (RB when not PADDED)
+  const uint32_t chunks = d / 8, chunks_v = dv / 8;     // 16-byte chunks per global row
 
   const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)head * p.nq * d;
   const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBGV;
 
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
@@ -178,7 +180,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const uint32_t lane_row = wave * RPW + lrow;
   const uint32_t kch_lane = lch ^ ((lane_row / RPB) % KMOD), vch_lane = lch ^ (4 * ((lane_row / RPB) % VMOD));
   const uint32_t koff_lane = lrow * RBG + 16 * kch_lane;
-  const uint32_t voff_lane = lrow * RBG + 16 * vch_lane;
+  const uint32_t voff_lane = lrow * RBGV + 16 * vch_lane;
   // K offset of wave-load `it`: the chunk of wave-load 0 with the constant XOR-ed in.  (On the byte offset itself
   // when the row part cannot reach the chunk bits, i.e. when rows are a power of two long: not PADDED.)
   auto koff_of = [&](int it) {
@@ -187,9 +189,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     else return koff_lane ^ (16u * x);
   };
   // a transfer of 16 bytes per lane; PADDED: only by the lanes whose chunk exists in the global row
-  auto dma16_chunk = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t chunk) {
+  auto dma16_chunk = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t chunk, uint32_t row_chunks) {
     if constexpr (PADDED) {
-      if (chunk < chunks) dma16(base, voff, lds_base);
+      if (chunk < row_chunks) dma16(base, voff, lds_base);
     } else {
       dma16(base, voff, lds_base);
     }
@@ -197,11 +199,13 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   // one wave-load of a full tile: `it` of K (want_k) or of V
   auto request_full_one = [&](uint32_t tile, int buf, int it, auto want_k) {
     const uint32_t w = wave + NWAVES * it;
-    const size_t byte0 = PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024;
+    const size_t row0 = (size_t)tile * BN + w * RPW;  // PADDED: first row of the wave-load
     if constexpr (decltype(want_k)::value)
-      dma16_chunk(K + byte0, koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024,
-                  kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD));
-    else dma16_chunk(V + byte0, voff_lane, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch_lane);
+      dma16_chunk(K + (PADDED ? row0 * RBG : (size_t)tile * TILE_BYTES + w * 1024), koff_of(it),
+                  smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD), chunks);
+    else
+      dma16_chunk(V + (PADDED ? row0 * RBGV : (size_t)tile * TILE_BYTES + w * 1024), voff_lane,
+                  smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch_lane, chunks_v);
   };
 
   // one wave-load of K of any tile index: full tile, partial tile (rows past nk re-read the last row), or none
@@ -209,14 +213,14 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
     if (tile < nfull_tiles) {
       const uint32_t w = wave + NWAVES * it;
       dma16_chunk(K + (PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024),
-                  koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD));
+                  koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD), chunks);
     } else if (tile * BN < p.nk) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;
       uint32_t key = tile * BN + row;
       key = key < p.nk ? key : p.nk - 1;
       const uint32_t kch = lch ^ ((row / RPB) % KMOD);
-      dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
+      dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch, chunks);
     }
   };
 
@@ -231,8 +235,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const uint32_t vch = lch ^ (4 * ((row / RPB) % VMOD));
       uint32_t key = key0 + row;
       if constexpr (PARTIAL) key = key < p.nk ? key : p.nk - 1;
-      if constexpr (decltype(want_k)::value) dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch);
-      if constexpr (decltype(want_v)::value) dma16_chunk(V, key * RBG + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch);
+      if constexpr (decltype(want_k)::value) dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch, chunks);
+      if constexpr (decltype(want_v)::value) dma16_chunk(V, key * RBGV + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch, chunks_v);
     }
   };
 
@@ -690,7 +694,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const float inv = 1.0f / half_sum(l_run);
   if (qrow < p.nq) {
     if (p.out_bf16) {
-      bf16_t* O = reinterpret_cast<bf16_t*>(p.o) + ((size_t)head * p.nq + qrow) * d;
+      bf16_t* O = reinterpret_cast<bf16_t*>(p.o) + ((size_t)head * p.nq + qrow) * dv;
 #pragma unroll
       for (int t = 0; t < DT; ++t)
 #pragma unroll
@@ -698,10 +702,10 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           bf16x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(o[t][4 * g + e] * inv);
-          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < dv) *reinterpret_cast<bf16x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
     } else if constexpr (!STAGED_STORE) {
-      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * d;
+      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * dv;
 #pragma unroll
       for (int t = 0; t < DT; ++t)
 #pragma unroll
@@ -709,7 +713,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
           f32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
-          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+          if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < dv) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
         }
     }
   }
@@ -730,7 +734,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       char* stage = &smem[0][0][0] + wave * 8192;
       const uint32_t row0 = qt * BM + wave * 32;  // first query row of this wave
       const uint32_t rows_valid = row0 < p.nq ? (p.nq - row0 < 32u ? p.nq - row0 : 32u) : 0u;
-      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + row0) * d;
+      float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + row0) * dv;
 #pragma unroll
       for (int half = 0; half < DT / 2; ++half) {
 #pragma unroll
@@ -747,7 +751,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
         for (int it = 0; it < 8; ++it) {
           const uint32_t r = 4 * it + (lane >> 4), q = lane & 15;
           const f32x4 w = *reinterpret_cast<const f32x4*>(stage + r * 256 + 16 * (q ^ (r & 15)));
-          if (r < rows_valid && (!PADDED || 64 * half + 4 * q < d)) *reinterpret_cast<f32x4*>(O + (size_t)r * d + 64 * half + 4 * q) = w;
+          if (r < rows_valid && (!PADDED || 64 * half + 4 * q < dv)) *reinterpret_cast<f32x4*>(O + (size_t)r * dv + 64 * half + 4 * q) = w;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }

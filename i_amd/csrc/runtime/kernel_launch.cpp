@@ -16,9 +16,9 @@ bool fits_u32(size_t v) { return v <= 0xffffffffull; }
 
 bool attention_supported(DType in_dtype, size_t d, size_t dv) {
   if (d == 0 || dv == 0) return false;
-  // head sizes above 128 up to 256: bf16, d == dv, on the direct kernels only
+  // head sizes above 128 up to 256: bf16, on the direct kernels only
   if (d > 128 || dv > 128)
-    return in_dtype == BF16 && d == dv && d <= 256 && d % 8 == 0 && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+    return in_dtype == BF16 && d <= 256 && dv <= 256 && d % 8 == 0 && dv % 8 == 0 && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
   return true;
 }
@@ -27,8 +27,9 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options, LaunchNote* note) {
   if (!attention_supported(in_dtype, d, dv))
-    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d == dv <= 256; bf16 needs d, dv % 8 == 0)";
-  if (d > 128 && nk * d * 2 >= (size_t(1) << 32)) return "attention kernel: too many keys for a head size above 128";
+    return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d, dv <= 256; bf16 needs d, dv % 8 == 0)";
+  if ((d > 128 || dv > 128) && nk * (d > dv ? d : dv) * 2 >= (size_t(1) << 32))
+    return "attention kernel: too many keys for a head size above 128";
   if (!std::isfinite(scale)) return "attention kernel: unsupported scale (must be finite)";
   if (in_dtype == F32 && out_dtype != F32) return "attention kernel: f32 inputs produce f32 output";
   if (bh == 0 || nq == 0) return {};
@@ -45,21 +46,22 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   //     key loops when that still leaves at least two workgroups per CU and does not pad nq by much, else 128.
   //     d == 64 on grids with at least two 512-query workgroups per CU (or a schedule tile of 512 x 32): the
   //     64-queries-per-wave kernel, which reads every K/V operand from LDS once for two MFMAs.
-  //   d == dv any other multiple of 8 below 128: the 4- and 8-wave kernels with 64-key tiles and their LDS rows
-  //     padded to 64 or 128 columns.
-  //   d == dv a multiple of 8 above 128 up to 256: the kernel for 256-column rows (padded below 256), 4 waves, one
+  //   any other d, dv that are multiples of 8 up to 128: the 4- and 8-wave kernels with 64-key tiles and their LDS
+  //     rows padded to 64 or 128 columns (the larger of d and dv decides).
+  //   d or dv above 128 up to 256 (multiples of 8): the kernel for 256-column rows (padded below 256), 4 waves, one
   //     per SIMD, 32-key tiles; nothing else exists above 128, so callers ask attention_supported() first.
-  //   otherwise: register-staged kernel with guarded columns (always multiplies the scores in f32)
+  //   otherwise (ILANG_ATTN_NO_DIRECT=1, key offsets beyond 32 bits): register-staged kernel with guarded columns
+  //     (always multiplies the scores in f32)
   // ILANG_ATTN_WAVES=2|4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
   // d == 64 only) and ILANG_ATTN_NO_DIRECT=1 forces the register-staged kernel; both exist so that tests can
   // reach every kernel with small inputs.
   unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
-  const bool wide = in_dtype == BF16 && d == dv && d > 128;  // (supported: d <= 256, a multiple of 8)
-  const bool padded = in_dtype == BF16 && d == dv && !exact && d % 8 == 0 && d >= 8 && d < 256;
+  const bool wide = in_dtype == BF16 && dmax > 128;  // (supported: d, dv <= 256, multiples of 8)
+  const bool padded = in_dtype == BF16 && !exact && d % 8 == 0 && dv % 8 == 0 && !(d == 256 && dv == 256);
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
-  const bool direct = (exact || padded || wide) && nk * d * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+  const bool direct = (exact || padded || wide) && nk * dmax * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   if (direct && wide) {
     bm = 128;  // 4 waves, one per SIMD
     bn = 32;
@@ -114,11 +116,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
       name = "attn_fwd_bf16_d64_bn32_q64";
       threads = bm;
     } else if (direct) {
-      name = "attn_fwd_bf16_d" + std::to_string(wide ? 256 : padded ? (d < 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
+      name = "attn_fwd_bf16_d" + std::to_string(wide ? 256 : padded ? (dmax <= 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
       if (bm == 64) name += "_w2";
       if (bm == 256) name += "_w8";
       if (options.f32_scale) name += "_f32scale";
-      if (padded && d != 256) name += "_pad";
+      if (padded) name += "_pad";
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   } else {

@@ -121,8 +121,8 @@ def test_reference_demo_flash_and_naive_attention(torch):
 
 
 def test_head_sizes_above_128(torch):
-    """bf16 with d == dv up to 256 runs the fused kernel for 256-column rows (padded when d < 256), in the f32-scale
-    form too.  Everything else above 128 (f32, the demo's own shape [32, 2048] of flash-attn.py:31-36; d != dv) runs as three
+    """bf16 with d and dv up to 256 runs the fused kernel for 256-column rows (padded below 256), in the f32-scale
+    form too.  Everything else above 128 (f32, the demo's own shape [32, 2048] of flash-attn.py:31-36; bf16 above 256) runs as three
     hand-written kernels: scores by the MFMA GEMM, row softmax in place, output by the MFMA GEMM.  f32 at the demo's
     shape against the emitted C; bf16 with batch axes, a score scale and ragged query counts against the oracle."""
     q, k, v = rnd((32, 2048), 1), rnd((32, 2048), 2), rnd((32, 2048), 3)
@@ -131,7 +131,7 @@ def test_head_sizes_above_128(torch):
     assert "attention in three kernels" in comp.report() and "gemm_nt_f32" in comp.report()
     close(got, oracle.compile_component(comp.handle).run(q, k, v), RTOL_F32)
     for d, dv, nq, nk, fused, f32_scale in ((192, 192, 300, 512, True, False), (256, 256, 130, 700, True, False),
-                                            (256, 160, 77, 136, False, False), (192, 192, 300, 512, True, True)):
+                                            (256, 160, 77, 136, True, False), (192, 192, 300, 512, True, True), (320, 192, 77, 136, False, False)):
         qb, kb, vb = (oracle.to_bf16_f32(rnd(shape, seed)) for seed, shape in
                       ((1, (2, 3, nq, d)), (2, (2, 3, nk, d)), (3, (2, 3, nk, dv))))
         scale = np.float32(1.0 / np.sqrt(d))
@@ -141,7 +141,7 @@ def test_head_sizes_above_128(torch):
         out = comp.exec_torch(torch.from_numpy(qb).cuda().bfloat16(), torch.from_numpy(kb).cuda().bfloat16(),
                               torch.tensor(scale, device="cuda"), torch.from_numpy(vb).cuda().bfloat16())
         if fused:
-            assert "attn_fwd_bf16_d256_bn32_direct" + ("_f32scale" if f32_scale else "") + ("_pad" if d < 256 else "") + " " in comp.report() + " "
+            assert "attn_fwd_bf16_d256_bn32_direct" + ("_f32scale" if f32_scale else "") + ("_pad" if (d, dv) != (256, 256) else "") + " " in comp.report() + " "
         else:
             assert "attention in three kernels" in comp.report() and "scaled_softmax" in comp.report()
         close(out.cpu().numpy(), oracle.attention_tiled(qb, kb, vb, scale), RTOL_BF16)

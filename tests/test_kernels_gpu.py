@@ -189,6 +189,20 @@ def test_attention_bf16_padded_head_size_keeps_its_neighbours_untouched(env):
     assert_close(od.cpu().numpy().reshape(bh, nq, d), oracle.attention_tiled(q, k, v, 0.1), RTOL_BF16)
 
 
+@pytest.mark.parametrize("d,dv", [(128, 64), (64, 128), (192, 128), (40, 72), (256, 136), (96, 256), (8, 16), (128, 120)])
+@pytest.mark.parametrize("f32_scale", [False, True])
+def test_attention_bf16_different_head_sizes_of_k_and_v(env, d, dv, f32_scale):
+    """d != dv: the padded direct-to-LDS kernels with K rows of d and V rows of dv elements in LDS rows of 64, 128 or
+    256 columns (the larger of the two decides).  Partial tiles, long key loops, ragged query counts, several heads."""
+    scale = float(np.float32(1.0 / np.sqrt(d)))
+    for bh, nq, nk in ((1, 64, 64), (3, 200, 333), (9, 130, 700)):
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, w), s)) for s, n, w in ((1, nq, d), (2, nk, d), (3, nk, dv)))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        assert_close(gpu_attention_ex(env, q, k, v, scale, f32_scale=f32_scale), ref, RTOL_BF16)
+    if not f32_scale:
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
+
+
 @pytest.mark.parametrize("d", [136, 160, 192, 224, 256])
 def test_attention_bf16_head_sizes_above_128(env, d):
     """d == dv in 136 .. 256 (multiples of 8) runs the direct-to-LDS kernel for 256-column rows: one wave per SIMD,
@@ -425,9 +439,9 @@ def test_attention_rejects_unsupported(env):
     rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, 60, 60,
                                       1.0, env.stream())
     assert rc == -1  # bf16 rows must be 16-byte multiples
-    # above 128: bf16 with d == dv <= 256 only
+    # above 128: bf16 with d, dv <= 256, multiples of 8
     xb = t.zeros(1, 8, 320, device="cuda", dtype=t.bfloat16)
-    for d, dv, f32_scale in ((192, 128, 0), (264, 264, 0), (136, 256, 1)):
+    for d, dv, f32_scale in ((192, 132, 0), (264, 264, 0), (136, 260, 1)):
         rc = env.nat.core.i_hip_attention_ex(xb.data_ptr(), xb.data_ptr(), xb.data_ptr(), x.data_ptr(), 1, 0, 1, 8, 8, d, dv,
                                              1.0, 0, 0, f32_scale, env.stream())
         assert rc == -1 and "unsupported" in env.nat.last_error(), (d, dv, f32_scale)
