@@ -28,10 +28,11 @@
 // Requires d == dv == DPAD, 16-byte aligned operands and nk * d * 4 < 2^32 (the launcher falls back to
 // attention_f32.h otherwise).  4 waves (128 queries) per workgroup, two workgroups per CU.
 //
-// PADDED: d == dv = p.d is any multiple of 4 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a lane whose
-// 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before the first
-// transfer, so the columns d .. DPAD - 1 of K and V read as zeros for the whole kernel (Q is padded with zeros in
-// its registers; the output columns past d are not stored).  Global rows are 4 p.d bytes apart.
+// PADDED: d = p.d and dv = p.dv are any multiples of 4 up to DPAD.  The tiles in LDS keep their DPAD-wide rows: a
+// lane whose 16-byte chunk lies past the end of a row fetches nothing, and the tile memory is cleared once before
+// the first transfer, so the columns d .. DPAD - 1 of K and dv .. DPAD - 1 of V read as zeros for the whole kernel
+// (Q is padded with zeros in its registers; the output columns past dv are not stored).  Global rows of Q and K
+// are 4 p.d bytes apart, those of V and O 4 p.dv.
 #pragma once
 #include <type_traits>
 
@@ -63,13 +64,14 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t c = lane & 31;  // query column within the wave / A-operand row
   const uint32_t h = lane >> 5;  // half-wave
-  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;  // elements per row in global memory
-  const uint32_t RBG = 4 * d;                         // ... and bytes (RB when not PADDED)
-  const uint32_t chunks = d / 4;                      // 16-byte chunks per global row
+  const uint32_t d = PADDED ? p.d : (uint32_t)DPAD;    // elements per row of Q and K in global memory
+  const uint32_t dv = PADDED ? p.dv : (uint32_t)DPAD;  // ... of V and O
+  const uint32_t RBG = 4 * d, RBGV = 4 * dv;            // bytes per global row of K, of V (RB when not PADDED)
+  const uint32_t chunks = d / 4, chunks_v = dv / 4;     // 16-byte chunks per global row
 
   const float* __restrict__ Q = reinterpret_cast<const float*>(p.q) + (size_t)head * p.nq * d;
   const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBGV;
 
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const float qsign = scale_raw < 0.0f ? -1.0f : 1.0f;  // negative scale folded into Q (exact)
@@ -89,7 +91,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       key = key < p.nk ? key : p.nk - 1;
       const uint32_t kch = lch ^ (row % 16), vch = lch ^ (8 * ((row >> 2) & 1));
       if (!PADDED || kch < chunks) dma16(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
-      if (!PADDED || vch < chunks) dma16(V, key * RBG + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
+      if (!PADDED || vch < chunks_v) dma16(V, key * RBGV + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
     }
   };
   if constexpr (PADDED) {
@@ -205,7 +207,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   const float l_tot = l_run + xhalf(l_run);
   const float inv = 1.0f / l_tot;
   if (qrow < p.nq) {
-    float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * d;
+    float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * dv;
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
@@ -213,7 +215,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
         f32x4 w;
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = o[t][4 * g + e] * inv;
-        if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < d) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
+        if (!PADDED || (uint32_t)(32 * t + 8 * g + 4 * h) < dv) *reinterpret_cast<f32x4*>(O + 32 * t + 8 * g + 4 * h) = w;
       }
   }
 }

@@ -124,16 +124,17 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   } else {
-    // f32: the direct-to-LDS kernel for d == dv that is a multiple of 4 in 36 .. 128 (16-byte aligned operands, 32-bit
-    // byte offsets inside a head; up to 32 the register-staged kernel with 32-column tiles is the faster one), the
+    // f32: the direct-to-LDS kernel for d, dv multiples of 4 up to 128, the larger above 32 (16-byte aligned operands,
+    // 32-bit byte offsets inside a head; up to 32 the register-staged kernel with 32-column tiles is the faster one), the
     // register-staged kernel with guarded columns otherwise (and under ILANG_ATTN_NO_DIRECT=1)
     auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
-    const bool f32_direct = d == dv && d % 4 == 0 && d > 32 && d <= 128 && nk * d * 4 < (size_t(1) << 32) && aligned16(q) &&
-                            aligned16(k) && aligned16(v) && aligned16(o) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+    const bool f32_direct = d % 4 == 0 && dv % 4 == 0 && dmax > 32 && dmax <= 128 && nk * dmax * 4 < (size_t(1) << 32) &&
+                            aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) &&
+                            std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
     if (f32_direct) {
-      // (head sizes other than 64 and 128: the same kernel with its LDS rows padded to 64 or 128 columns)
-      name = d <= 64 ? "attn_fwd_f32_d64_bn32_direct" : "attn_fwd_f32_d128_bn32_direct";
-      if (d != 64 && d != 128) name += "_pad";
+      // (head sizes other than d == dv in {64, 128}: the same kernel with its LDS rows padded to 64 or 128 columns)
+      name = dmax <= 64 ? "attn_fwd_f32_d64_bn32_direct" : "attn_fwd_f32_d128_bn32_direct";
+      if (!(d == dv && (d == 64 || d == 128))) name += "_pad";
     }
     else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
     bn = 32;

@@ -80,8 +80,8 @@ int i_exec_into_device_noalloc(const i_program* program,
  * in_dtype applies to q/k/v, out_dtype to o.  Requires a finite scale and 0 < d,dv <= 128
  * (f32), 0 < d,dv <= 256 and multiples of 8 (bf16).  bf16 runs the direct-to-LDS kernels
  * at every such head size (d = dv = 64, 128, 256 exactly, the others with zero-padded LDS
- * rows); f32 with d == dv a multiple of 4 from 36 to 128 and 16-byte aligned operands runs
- * the f32 kernel of the same design.
+ * rows); f32 with d and dv multiples of 4, the larger from 36 to 128, and 16-byte aligned
+ * operands runs the f32 kernel of the same design.
  */
 int i_hip_attention(const void* q, const void* k, const void* v, void* o,
                     int in_dtype, int out_dtype,

@@ -125,6 +125,14 @@ def test_attention_f32_direct_and_staged_kernels_vs_oracle(env, monkeypatch, d, 
         assert_close(gpu_attention(env, q, k, v, scale, bf16=False), oracle.attention_tiled(q, k, v, scale), RTOL_F32)
 
 
+@pytest.mark.parametrize("d,dv", [(64, 128), (128, 64), (40, 72), (100, 36), (24, 64)])
+def test_attention_f32_different_head_sizes_of_k_and_v(env, d, dv):
+    """f32 with d != dv (multiples of 4, the larger above 32): the padded form of the direct kernel."""
+    for bh, nq, nk, scale in ((1, 128, 32, 1.0), (3, 200, 333, 0.11), (9, 130, 64, -0.2)):
+        q, k, v = (rnd((bh, n, w), sd) for sd, n, w in ((1, nq, d), (2, nk, d), (3, nk, dv)))
+        assert_close(gpu_attention(env, q, k, v, scale, bf16=False), oracle.attention_tiled(q, k, v, scale), RTOL_F32)
+
+
 def test_attention_f32_operands_not_16_byte_aligned(env):
     """The direct f32 kernel moves 16 bytes per lane; operands that start off a 16-byte boundary take the
     register-staged kernel and give the same result."""
