@@ -152,9 +152,11 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }
 
 // 256 x 256 tiles (one workgroup per CU, 256 at a time) or 128 x 128 tiles (two per CU, 512 at a time) for a
-// problem with enough of either?  The larger tile is about 25 % more efficient per flop, but its last round of
-// workgroups may leave most of the chip idle: 6144^3 is 2.25 rounds of 256-tiles (measured 1070 TFLOP/s) and
-// 4.5 rounds of 128-tiles (1135).  Rounds of the two-per-CU kernel count in halves.
+// problem with enough of either?  The larger tile is about 20 % more efficient per flop (1420 against 1214 TFLOP/s
+// at 4096^3, whole rounds of either), but its last round of workgroups may leave most of the chip idle: 4608^3 is
+// 1.27 rounds of 256-tiles (measured 1037 TFLOP/s) and 2.53 rounds of 128-tiles (1101).  Rounds of the two-per-CU
+// kernel count in halves.  (A model, within 5 % of the better tile from 1024^3 to 8192^3: it misjudges 3072^3 and
+// 6144^3 by 4 % and 2 %.)
 static unsigned pick_direct_tile(size_t t256, size_t t128) {
   const double r256 = (double)t256 / 256.0, r128 = (double)t128 / 512.0;
   const double e256 = 1430.0 * r256 / std::ceil(r256);
