@@ -120,6 +120,28 @@ def test_reference_demo_flash_and_naive_attention(torch):
         assert np.allclose(got, ref, rtol=3e-4, atol=5e-5, equal_nan=True)  # the demo's own tolerance
 
 
+def test_head_sizes_between_and_unequal_through_the_frontend(torch):
+    """The compiled component hands the operands' own d and dv to the launcher: bf16 tensors with d = dv = 96 (batch
+    axes, score scale), d = 40 without a scale, and d = 64 with dv = 128 run the padded direct kernels; f32 tensors
+    with d = dv = 96 the padded f32 kernel.  Against the oracle."""
+    for d, dv, nq, nk, kernel in ((96, 96, 300, 500, "attn_fwd_bf16_d128_bn64_direct_pad"),
+                                  (64, 128, 130, 333, "attn_fwd_bf16_d128_bn64_direct_pad"),
+                                  (40, 40, 77, 200, "attn_fwd_bf16_d64_bn64_direct_pad")):
+        qb, kb, vb = (oracle.to_bf16_f32(rnd(shape, seed)) for seed, shape in
+                      ((1, (2, 3, nq, d)), (2, (2, 3, nk, d)), (3, (2, 3, nk, dv))))
+        scale = np.float32(1.0 / np.sqrt(d))
+        comp = flash("i:128,j:64", prefix="bh", scaled=True)
+        out = comp.exec_torch(torch.from_numpy(qb).cuda().bfloat16(), torch.from_numpy(kb).cuda().bfloat16(),
+                              torch.tensor(scale, device="cuda"), torch.from_numpy(vb).cuda().bfloat16())
+        assert kernel + " " in comp.report() + " ", comp.report()
+        close(out.cpu().numpy(), oracle.attention_tiled(qb, kb, vb, scale), RTOL_BF16)
+    q, k, v = rnd((200, 96), 1), rnd((333, 96), 2), rnd((333, 96), 3)
+    comp = flash()
+    out = comp.exec_torch(*(torch.from_numpy(a).cuda() for a in (q, k, v)))
+    assert "attn_fwd_f32_d128_bn32_direct_pad" in comp.report()
+    close(out.cpu().numpy(), oracle.attention_tiled(q, k, v), RTOL_F32)
+
+
 def test_head_sizes_above_128(torch):
     """bf16 with d and dv up to 256 runs the fused kernel for 256-column rows (padded below 256), in the f32-scale
     form too.  Everything else above 128 (f32, the demo's own shape [32, 2048] of flash-attn.py:31-36; bf16 above 256) runs as three
