@@ -39,14 +39,18 @@
 // row is XOR-ed, on the global side, with f(row) = row % 4 + 4 ((row / 8) % 2), which sends those 8 rows to 8
 // different bank groups.  Requires n % 8 == 0 as well; 16-byte chunks that start past n re-read the row's last
 // chunk (their columns are not stored).
-// Requires k % 64 == 0.
+//
+// KTAIL = true is the same kernel for k that is a multiple of 8 but not of 64: the last slab is partial.  The lanes
+// whose 16-byte chunk (NN: whose slab row of B) lies past k transfer nothing and clear their LDS slot instead, so
+// the slab reads as zeros there and the k loop runs over whole slabs as before.
+// Requires k % 64 == 0, or k % 8 == 0 with KTAIL.
 #pragma once
 #include <type_traits>
 
 #include "common.h"
 #include "params.h"
 
-template <int BT, int WM, int WN, bool EDGE, bool NN>
+template <int BT, int WM, int WN, bool EDGE, bool NN, bool KTAIL>
 __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* smem_base, uint32_t tm, uint32_t tn) {
   constexpr int RB = 128;            // bytes per slab row: 64 k of bf16
   constexpr int BK = 64;
@@ -111,19 +115,35 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     ch = ch < last_chunk ? ch : last_chunk;
     boff_nn = r * (uint32_t)brow_bytes + 16 * ch;
   }
-  auto request = [&](uint32_t s, int buf, int r) {  // request r of the 2 WLW that bring slab s into `buf`
+  const uint32_t nslabs = KTAIL ? (p.k + BK - 1) / BK : p.k / BK;
+  // KTAIL: what exists of the last slab: 16-byte chunks per row (rows of k for an NN slab of B)
+  const uint32_t tail_chunks = (p.k - (nslabs - 1) * BK) / 8;
+  // a transfer of 16 bytes per lane; KTAIL: a lane that has nothing to fetch (`valid` false) clears its slot
+  auto move = [&](const void* base, uint32_t voff, uint32_t lds_base, bool valid) {
+    if constexpr (KTAIL) {
+      if (valid) dma16(base, voff, lds_base);
+      else *reinterpret_cast<u32x4*>(&smem[0][0][0] + (lds_base - smem0) + 16 * lane) = u32x4{0, 0, 0, 0};
+    } else {
+      dma16(base, voff, lds_base);
+    }
+  };
+  // request r of the 2 WLW that bring slab s into `buf`; `tail`: slab s may be the partial one (KTAIL)
+  auto request = [&](uint32_t s, int buf, int r, auto tail) {
     const int it = r % WLW;
     const uint32_t w = wave + NWAVES * it;
     const size_t k_byte = (size_t)s * RB;
     const uint32_t to_a = smem0 + (2 * buf + 0) * SLAB + w * 1024, to_b = smem0 + (2 * buf + 1) * SLAB + w * 1024;
+    const bool whole = !KTAIL || !decltype(tail)::value || s + 1 < nslabs;  // the slab lies inside k
+    const bool valid = whole || gch < tail_chunks;         // ... or this lane's chunk of a K-contiguous row does
     if (r >= WLW && NN) {
-      dma16(b_tile + ((size_t)s * BK + 16 * it) * brow_bytes, boff_nn, to_b);
+      const bool valid_row = whole || (w * RPWN + lane / CHN) < 8 * tail_chunks;
+      move(b_tile + ((size_t)s * BK + 16 * it) * brow_bytes, boff_nn, to_b, valid_row);
     } else if constexpr (EDGE) {
-      if (r < WLW) dma16(a_tile + k_byte, row_offset(it, lim_a), to_a);
-      else dma16(b_tile + k_byte, row_offset(it, lim_b), to_b);
+      if (r < WLW) move(a_tile + k_byte, row_offset(it, lim_a), to_a, valid);
+      else move(b_tile + k_byte, row_offset(it, lim_b), to_b, valid);
     } else {
-      if (r < WLW) dma16(a_tile + k_byte + it * it_stride, voff0, to_a);
-      else dma16(b_tile + k_byte + it * it_stride, voff0, to_b);
+      if (r < WLW) move(a_tile + k_byte + it * it_stride, voff0, to_a, valid);
+      else move(b_tile + k_byte + it * it_stride, voff0, to_b, valid);
     }
   };
 
@@ -150,9 +170,8 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  const uint32_t nslabs = p.k / BK;
 #pragma unroll
-  for (int r = 0; r < 2 * WLW; ++r) request(0, 0, r);
+  for (int r = 0; r < 2 * WLW; ++r) request(0, 0, r, std::true_type{});
   dma_wait_all();
   __syncthreads();
 
@@ -175,7 +194,8 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   // One k-step: TM x TN MFMAs on (a, bc) while a is refilled in place and bn is filled with the operands of
   // k-step `ks` of buffer `buf`; `reqs` says whether the slab requests of this trip ride on it.
   constexpr int NREQ = 2 * WLW, NSLOT = TM * TN;
-  auto kstep = [&](bf16x8 (&bc)[TN], bf16x8 (&bn)[TN], int buf, int ks, bool refill, auto reqs, uint32_t s_req, int req_buf) {
+  auto kstep = [&](bf16x8 (&bc)[TN], bf16x8 (&bn)[TN], int buf, int ks, bool refill, auto reqs, uint32_t s_req, int req_buf,
+                   auto tail) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -188,7 +208,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
         }
         if constexpr (decltype(reqs)::value) {
 #pragma unroll
-          for (int r = slot * NREQ / NSLOT; r < (slot + 1) * NREQ / NSLOT; ++r) request(s_req, req_buf, r);
+          for (int r = slot * NREQ / NSLOT; r < (slot + 1) * NREQ / NSLOT; ++r) request(s_req, req_buf, r, tail);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -197,10 +217,11 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   // (a, b1) and slab s + 1 is requested; then k-step 0 while k-step 1 arrives in (a, b0), carried into the next
   // trip.  The last trip has no successor; it requests its own slab once more into the other buffer, which
   // nobody reads any more: one redundant slab per workgroup instead of a branch in every slot.
-  auto trip = [&](uint32_t s, int buf) {
+  // `tail`: the slab this trip requests may be the partial one (KTAIL), so its requests carry the per-lane test
+  auto trip = [&](uint32_t s, int buf, auto tail) {
     const uint32_t s_req = s + 1 < nslabs ? s + 1 : s;
-    kstep(b0, b1, buf, 0, true, std::true_type{}, s_req, buf ^ 1);
-    kstep(b1, b0, buf, 1, true, std::false_type{}, 0, 0);
+    kstep(b0, b1, buf, 0, true, std::true_type{}, s_req, buf ^ 1, tail);
+    kstep(b1, b0, buf, 1, true, std::false_type{}, 0, 0, std::false_type{});
     dma_wait_all();
     __syncthreads();
   };
@@ -210,13 +231,22 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
 #pragma unroll
   for (int j = 0; j < TN; ++j) b0[j] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
   uint32_t s = 0;
-  for (; s + 2 <= nslabs; s += 2) {  // two per iteration so that the buffer index is a constant
-    trip(s, 0);
-    trip(s + 1, 1);
+  // KTAIL: trip s requests slab s + 1, so the trips before nslabs - 2 request whole slabs; the two or three that
+  // remain after the pairs of them are written out with the per-lane test
+  const uint32_t nplain = KTAIL ? (nslabs > 2 ? (nslabs - 2) & ~1u : 0u) : nslabs;
+  for (; s + 2 <= nplain; s += 2) {  // two per iteration so that the buffer index is a constant
+    trip(s, 0, std::false_type{});
+    trip(s + 1, 1, std::false_type{});
   }
-  if (s < nslabs) trip(s, 0);
+  if constexpr (KTAIL) {
+    if (s < nslabs) trip(s, 0, std::true_type{});
+    if (s + 1 < nslabs) trip(s + 1, 1, std::true_type{});
+    if (s + 2 < nslabs) trip(s + 2, 0, std::true_type{});
+  } else {
+    if (s < nslabs) trip(s, 0, std::false_type{});
+  }
   // last k-step of the last slab
-  kstep(b0, b1, 0, 0, false, std::false_type{}, 0, 0);
+  kstep(b0, b1, 0, 0, false, std::false_type{}, 0, 0, std::false_type{});
 
   // ---- store.  acc[i][j][r] is C[m0 + 16 (wm TM + i) + c16][n0 + 16 (wn TN + j) + 4 g + r]: a lane writes four
   // consecutive columns at once, a quarter-wave 16 rows of them.  Columns come in fours, so a C whose n is not
@@ -250,7 +280,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   }
 }
 
-template <int BT, int WM, int WN, bool NN = false>
+template <int BT, int WM, int WN, bool NN = false, bool KTAIL = false>
 __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
   // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
@@ -262,6 +292,6 @@ __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
   const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
   if (tm >= p.tiles_m || tn >= p.tiles_n) return;
-  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN>(p, smem, tm, tn);
-  else gemm_nt_mfma16_tile<BT, WM, WN, true, NN>(p, smem, tm, tn);
+  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN, KTAIL>(p, smem, tm, tn);
+  else gemm_nt_mfma16_tile<BT, WM, WN, true, NN, KTAIL>(p, smem, tm, tn);
 }

@@ -109,6 +109,19 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nn_bf16_256x256x64_dir
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nn_bf16_128x128x64_direct(GemmParams p) {
   gemm_nt_mfma16_body<128, 2, 2, true>(p);
 }
+// k a multiple of 8 but not of 64: the last slab partial
+extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct_ktail(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 4, false, true>(p);
+}
+extern "C" __global__ void __launch_bounds__(512, 1) gemm_nn_bf16_256x256x64_direct_ktail(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 4, true, true>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_bf16_128x128x64_direct_ktail(GemmParams p) {
+  gemm_nt_mfma16_body<128, 2, 2, false, true>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nn_bf16_128x128x64_direct_ktail(GemmParams p) {
+  gemm_nt_mfma16_body<128, 2, 2, true, true>(p);
+}
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_direct(GemmParams p) {
   gemm_nt_f32_direct_body<128, 2, 2>(p);
 }

@@ -174,10 +174,11 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
-  // Direct global -> LDS kernels (need whole 64-wide k slabs and 32-bit byte offsets inside a tile's rows):
+  // Direct global -> LDS kernels (64-wide k slabs, 32-bit byte offsets inside a tile's rows):
   //   256 x 256 tiles  long k loops on grids that fill at least half of the CUs (its prologue and its
   //                    unoverlapped store only pay off there)
   //   128 x 128 tiles  problems with too few 256-tiles, two workgroups per CU
+  // (k that is no multiple of 64: their _ktail forms, the last slab partial)
   // and the register-staged 128 x 128 kernel for everything else (k % 8 == 0, short k, tiny grids).
   // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; ILANG_GEMM_DIRECT=256 | 128 | 0
   // forces a kernel so that tests can reach each of them at small sizes (1 is read as 256).
@@ -189,16 +190,18 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
     if (tile_m == 256 && tile_n == 256) tile = 256;
     if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
     if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
-    if (tile && k % 64 == 0 && k <= (size_t(1) << 22) && bh <= 65535) {
+    const bool ktail = k % 64 != 0;
+    if (tile && k <= (size_t(1) << 22) && bh <= 65535) {
       p.tiles_m = (uint32_t)((m + tile - 1) / tile);
       p.tiles_n = (uint32_t)((n + tile - 1) / tile);
       const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs
       const size_t grid = ((nsb + 7) / 8 * 8) * 32;
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
-      const char* name = tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct";
+      const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct") +
+                               (ktail ? "_ktail" : "");
       if (note) *note = LaunchNote{name, tile, tile};
-      if (Err e = builtin_function(name, &fn); !e.empty()) return e;
+      if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
       return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
     }
   }
@@ -213,9 +216,10 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
 
-// NN product on the direct kernels: whole 64-wide k slabs, 16-byte chunks along n, 32-bit byte offsets inside a slab
+// NN product on the direct kernels: 64-wide k slabs (the last one may be partial), 16-byte chunks along n, 32-bit byte
+// offsets inside a slab
 static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n) {
-  if (k == 0 || k % 64 != 0 || n % 8 != 0 || k > (size_t(1) << 22) || n > (size_t(1) << 24) || bh > 65535) return 0;
+  if (k == 0 || k % 8 != 0 || n % 8 != 0 || k > (size_t(1) << 22) || n > (size_t(1) << 24) || bh > 65535) return 0;
   if (!fits_u32(m) || !fits_u32(n)) return 0;
   const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
   unsigned tile = t256 >= 128 ? pick_direct_tile(t256, t128) : 128;
@@ -230,7 +234,7 @@ bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return ge
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                         hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype) {
   const unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
-  if (tile == 0) return "gemm_nn kernel: needs k % 64 == 0 and n % 8 == 0 (and extents within its offset range)";
+  if (tile == 0) return "gemm_nn kernel: needs k % 8 == 0 and n % 8 == 0 (and extents within its offset range)";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!a || !b || !c) return "gemm_nn kernel: null device pointer";
   GemmParams p{};
@@ -243,9 +247,10 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   const size_t grid = ((nsb + 7) / 8 * 8) * 32;
   if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
   hipFunction_t fn;
-  const char* name = tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct";
+  const std::string name = std::string(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct") +
+                           (k % 64 != 0 ? "_ktail" : "");
   if (note) *note = LaunchNote{name, tile, tile};
-  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
+  if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 

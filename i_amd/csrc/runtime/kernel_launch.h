@@ -45,7 +45,7 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
 bool gemm_nt_bf16_supported(size_t k);
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
-// Needs k % 64 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
+// Needs k % 8 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                         hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr,
                         DType out_dtype = F32);

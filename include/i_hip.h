@@ -136,7 +136,7 @@ int i_hip_gemm_nt_bf16_ex(const void* a, const void* b, void* c, int out_dtype,
 /*
  * The product with a row-major right operand,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,k,n]  (bf16 a, b, f32 c):
  * the fused kernel for  i("ik*kj~ijk") >> i("+ijk~ij ...")  (ilang-python/test.py:52-56) and for the demo's
- * standalone mm,  i("ij*jk~ikj") >> i("+ikj~ik ...")  (ilang-python/flash-attn.py:51).  Requires k % 64 == 0
+ * standalone mm,  i("ij*jk~ikj") >> i("+ikj~ik ...")  (ilang-python/flash-attn.py:51).  Requires k % 8 == 0
  * and n % 8 == 0; other shapes go through a transpose and i_hip_gemm_nt_bf16.
  */
 int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c,

@@ -330,14 +330,14 @@ def test_wide_rows_through_the_naive_and_the_row_staged_schedules(torch):
 
 
 def test_products_write_bf16_outputs_themselves(torch):
-    """bf16 operands with out_dtype bf16: mm_t, the row-major product and its transposed fallback (k % 64 != 0)
+    """bf16 operands with out_dtype bf16: mm_t and the row-major product (k a multiple of 64, and not)
     store bf16 from the kernel, with no f32 staging and no conversion pass; results equal the f32 results rounded."""
     a = torch.from_numpy(oracle.to_bf16_f32(rnd((300, 128), 1))).cuda().bfloat16()
     b = torch.from_numpy(oracle.to_bf16_f32(rnd((264, 128), 2))).cuda().bfloat16()
     mm_t = i("ik*jk~ijk | i:128,j:128 | jii'j'k") >> i("+ijk~ij | i:128,j:128 | jii'j'k0")
     assert torch.equal(mm_t.exec_torch(a, b, out_dtype=torch.bfloat16), mm_t.exec_torch(a, b).bfloat16())
     nn = i("ik*kj~ijk|i:16,j:16|jii'j'k") >> i("+ijk~ij|i:16,j:16|jii'j'k0")
-    for kk in (128, 72):  # read in place / transposed first
+    for kk in (128, 72):  # whole slabs / a partial last slab
         bt = torch.from_numpy(oracle.to_bf16_f32(rnd((kk, 264), 3))).cuda().bfloat16()
         a2 = torch.from_numpy(oracle.to_bf16_f32(rnd((300, kk), 4))).cuda().bfloat16()
         assert torch.equal(nn.exec_torch(a2, bt, out_dtype=torch.bfloat16), nn.exec_torch(a2, bt).bfloat16())

@@ -497,6 +497,35 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, dire
     assert_close(cd.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
+@pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 8), (1, 300, 264, 40), (2, 600, 520, 136), (1, 1, 8, 200), (3, 257, 256, 1000),
+                                      (1, 128, 128, 72)])
+@pytest.mark.parametrize("nn", [False, True])
+@pytest.mark.parametrize("tile", ["128", "256"])
+def test_gemm_bf16_k_that_is_no_multiple_of_64(env, monkeypatch, bh, m, n, k, nn, tile):
+    """k % 8 == 0 but k % 64 != 0: the direct kernels with a partial last slab (the lanes past k clear their LDS
+    slots), both tile sizes forced here at small sizes; NT and NN, f32 and bf16 output."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile)
+    t = env.torch
+    a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
+    b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
+    ref = oracle.mm_t(a, b)
+    ad = t.from_numpy(a).cuda().bfloat16()
+    bd = t.from_numpy(np.ascontiguousarray(b.transpose(0, 2, 1)) if nn else b).cuda().bfloat16()
+    cd = t.full((bh, m, n), float("nan"), device="cuda")
+    core = env.nat.core
+    if nn:
+        env.nat.check(core.i_hip_gemm_nn_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+    else:
+        env.nat.check(core.i_hip_gemm_nt_bf16(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), bh, m, n, k, env.stream()))
+        c16 = t.full((bh, m, n), float("nan"), device="cuda", dtype=t.bfloat16)
+        env.nat.check(core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), c16.data_ptr(), env.nat.BF16, bh, m, n, k, 0, 0,
+                                                  env.stream()))
+    t.cuda.synchronize()
+    assert_close(cd.cpu().numpy(), ref, RTOL_BF16)
+    if not nn:
+        assert t.equal(c16, cd.bfloat16())
+
+
 @pytest.mark.parametrize("tile", [0, 128, 256])
 def test_gemm_nt_bf16_output_in_bf16(env, monkeypatch, tile):
     """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
@@ -564,7 +593,7 @@ def test_gemm_nn_bf16_rejects_what_the_direct_kernels_cannot_read(env):
     t = env.torch
     x = t.zeros(64 * 72, device="cuda", dtype=t.bfloat16)
     c = t.zeros(64 * 72, device="cuda")
-    for m, n, k in ((64, 60, 64), (64, 64, 40)):
+    for m, n, k in ((64, 60, 64), (64, 64, 36)):
         rc = env.nat.core.i_hip_gemm_nn_bf16(x.data_ptr(), x.data_ptr(), c.data_ptr(), 1, m, n, k, env.stream())
         assert rc == -1 and "gemm_nn" in env.nat.last_error()
 
