@@ -466,6 +466,29 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
       total *= run.extent(resolved);
     }
     if (total == 0) continue;
+    // The wavefront-per-iteration form (reduction loops spread over 64 lanes), when the nest has one: taken when
+    // the reduction is long enough to occupy the lanes and either consecutive lanes read consecutive elements
+    // or there are too few iterations to fill the chip with one work-item each.  ILANG_HIP_WAVE=0|1 overrides.
+    if (!ph.wave_loops.empty()) {
+      const auto& e = ph.wave_extent;
+      const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
+      const size_t reduced = run.extent(Extent<size_t>{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind});
+      bool wave = reduced >= 128 && (ph.wave_contiguous || total < 65536);
+      if (const char* force = std::getenv("ILANG_HIP_WAVE")) wave = force[0] == '1';
+      if (wave) {
+        const size_t waves = std::min<size_t>(total, size_t(1) << 16);
+        const unsigned per_group = GenericPhase::kWaveThreads / 64;
+        for (const PrivateBuffer& pb : ph.privates) fill(nr + pb.writeable, nullptr, dispatch.writes[pb.writeable]);
+        hipFunction_t fn;
+        if (ihip::Err err = generic_function(p, ph.name + "_w", &fn); !err.empty()) return err;
+        run.notes.back() += ", as " + ph.name + "_w: one wavefront per iteration of the parallel loops";
+        if (ihip::Err err = ihip::launch(fn, (unsigned)((waves + per_group - 1) / per_group), 1, 1, GenericPhase::kWaveThreads,
+                                         args.data(), args.size(), run.stream);
+            !err.empty())
+          return err;
+        continue;
+      }
+    }
     size_t threads = ph.parallel_loops.empty() ? 1 : total;
     // dynamic private buffers cost memory per work-item slot: cap the slots
     size_t slot_elems = 0;
@@ -606,6 +629,10 @@ std::string program_code(const Component& component) {
         os << "; work-item-private:";
         for (const auto& pb : ph.privates)
           os << " " << ref_name(d->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
+      }
+      if (!ph.wave_loops.empty()) {
+        os << "\n//     " << ph.name << "_w, one wavefront per work-item of the above (long reductions): over its lanes";
+        for (const WaveLoop& wl : ph.wave_loops) os << " i" << wl.loop;
       }
     }
     os << "\n";

@@ -94,7 +94,21 @@ CASES = {
     "column sum normalize, split j": (lambda: (I & i("+ij~j|j:4|ijj'")) >> i("ij/j~ij|j:4|1ijj'"), [(9, 21)]),
     "mlp with pair": (lambda: (i("ij~ij") | ((i("ij*j~ij") >> i("+ij~i")) >> i(">i~i"))) >> (i("ij*j~ij") >> i("+ij~i")),
                       [(7, 16), (16, 8), (8,)]),
+    # reductions long enough for several rounds of a wavefront's 64 lanes, with ragged ends
+    "row sum 5x300": (lambda: i("+ij~i"), [(5, 300)]),
+    "row max 3x130, split j": (lambda: i(">ij~i|j:16|ijj'"), [(3, 130)]),
+    "row min 70x129": (lambda: i("<ij~i"), [(70, 129)]),
+    "fused matrix-vector product": (lambda: i("ij*j~ij||ij") >> i("+ij~i||ij0"), [(7, 150), (150,)]),
+    "batched row sum": (lambda: i("+bij~bi"), [(3, 5, 200)]),
+    "sum over the two last axes": (lambda: i("+bij~b"), [(3, 9, 70)]),
 }
+
+# the cases with a nest that has a wavefront-per-iteration form (reduction loops spread over 64 lanes)
+WAVE_CASES = ["naive attention ragged", "batched naive attention", "mm_t", "mm_t empty", "matmul unfused",
+              "matmul fused init site", "row sum", "column max", "total", "fanout two outputs", "swapped fanout",
+              "two-level split mm_t", "column min", "product reduction", "mlp with pair", "row sum 5x300",
+              "row max 3x130, split j", "row min 70x129", "fused matrix-vector product", "batched row sum",
+              "sum over the two last axes"]
 
 
 # Components with a reduced vector staged at the root of its consumer are checked against NumPy as well: the emitted
@@ -128,7 +142,8 @@ def main():
     import os
 
     noalloc = os.environ.get("ILANG_SHIM_NOALLOC") == "1"
-    names = sys.argv[1:] or list(CASES)
+    names = sys.argv[1:] or (WAVE_CASES if os.environ.get("ILANG_SHIM_CASES") == "wave" else list(CASES))
+    tolerance = float(os.environ.get("ILANG_SHIM_TOLERANCE", "1e-5"))
     failed = []
     for name in names:
         build, shapes = CASES[name]
@@ -145,7 +160,7 @@ def main():
         for g, r in zip(got, ref):
             scale = float(np.abs(r).max()) if r.size else 1.0
             err = float(np.abs(g - r).max()) / (scale or 1.0) if r.size else 0.0
-            ok = g.shape == r.shape and (r.size == 0 or (np.isfinite(g).all() and err <= 1e-5))
+            ok = g.shape == r.shape and (r.size == 0 or (np.isfinite(g).all() and err <= tolerance))
             if not ok:
                 failed.append(name)
                 print("MISMATCH", name, g.shape, r.shape, err, flush=True)

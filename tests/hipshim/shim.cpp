@@ -11,6 +11,8 @@
 #include <elf.h>
 #include <hip/hip_runtime_api.h>
 #include <pthread.h>
+
+#include <algorithm>
 #include <sys/mman.h>
 #include <unistd.h>
 
@@ -66,7 +68,7 @@ struct BigArgs {
   unsigned char bytes[4096];
 };
 struct Function {
-  void *kernel, *set_ids, *set_barrier;
+  void *kernel, *set_ids, *set_barrier, *set_wave;
 };
 void wait_on(void* barrier) { pthread_barrier_wait(static_cast<pthread_barrier_t*>(barrier)); }
 }  // namespace
@@ -129,9 +131,10 @@ hipError_t hipModuleGetFunction(hipFunction_t* fn, hipModule_t mod, const char* 
   void* f = dlsym(m->handle, name);
   void* set = dlsym(m->handle, "shim_set_ids");
   void* bar = dlsym(m->handle, "shim_set_barrier");
-  if (!f || !set || !bar) return hipErrorNotFound;
-  // a function handle is the triple (kernel, id setter and barrier setter of its library)
-  *fn = reinterpret_cast<hipFunction_t>(new Function{f, set, bar});
+  void* wave = dlsym(m->handle, "shim_set_wave");
+  if (!f || !set || !bar || !wave) return hipErrorNotFound;
+  // a function handle is the kernel with the setters of its library (ids, workgroup barrier, wavefront context)
+  *fn = reinterpret_cast<hipFunction_t>(new Function{f, set, bar, wave});
   return hipSuccess;
 }
 hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
@@ -153,21 +156,30 @@ hipError_t hipModuleLaunchKernel(hipFunction_t fn, unsigned gx, unsigned gy, uns
   auto kernel = reinterpret_cast<void (*)(BigArgs)>(f->kernel);
   auto set_ids = reinterpret_cast<void (*)(unsigned, unsigned, unsigned, unsigned)>(f->set_ids);
   auto set_barrier = reinterpret_cast<void (*)(void (*)(void*), void*)>(f->set_barrier);
+  auto set_wave = reinterpret_cast<void (*)(void (*)(void*), void*, float*)>(f->set_wave);
   if (bx > 64) {
     // the work-items of a workgroup run as threads, so that a barrier between two loop nests of a kernel means
     // what it means on the device: every work-item has finished the first nest before any starts the second
     for (unsigned block = 0; block < gx; ++block) {
       pthread_barrier_t barrier;
       pthread_barrier_init(&barrier, nullptr, bx);
+      // every 64 consecutive work-items are a wavefront with a barrier and exchange slots of its own
+      const unsigned waves = (bx + 63) / 64;
+      std::vector<pthread_barrier_t> wave_barriers(waves);
+      std::vector<float> wave_slots(64 * waves, 0.0f);
+      for (unsigned w = 0; w < waves; ++w) pthread_barrier_init(&wave_barriers[w], nullptr, std::min(64u, bx - 64 * w));
       std::vector<std::thread> items;
       for (unsigned t = 0; t < bx; ++t)
         items.emplace_back([&, t] {
           set_ids(block, t, bx, gx);
           set_barrier(wait_on, &barrier);
+          set_wave(wait_on, &wave_barriers[t / 64], &wave_slots[64 * (t / 64)]);
           kernel(args);
           set_barrier(nullptr, nullptr);
+          set_wave(nullptr, nullptr, nullptr);
         });
       for (auto& th : items) th.join();
+      for (unsigned w = 0; w < waves; ++w) pthread_barrier_destroy(&wave_barriers[w]);
       pthread_barrier_destroy(&barrier);
     }
     return hipSuccess;

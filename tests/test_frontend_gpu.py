@@ -592,6 +592,48 @@ def test_multi_nest_generated_kernels_run_as_one_workgroup(torch, monkeypatch):
     close(nv.exec_numpy(q, k, v), oracle.compile_component(nv.handle).run(q, k, v), RTOL_F32)
 
 
+@pytest.mark.parametrize("wave", ["1", "0", None])
+def test_reduction_nests_in_the_wavefront_form(torch, monkeypatch, wave):
+    """Generated reduction nests have a second form in which a wavefront stands where a work-item stood (the
+    reduction loop spread over 64 lanes, lane shares combined by a butterfly).  Forced on, forced off and left to
+    the launcher (ILANG_HIP_WAVE unset), against NumPy in float64 and, at sizes it finishes quickly, the emitted C."""
+    if wave is None:
+        monkeypatch.delenv("ILANG_HIP_WAVE", raising=False)
+    else:
+        monkeypatch.setenv("ILANG_HIP_WAVE", wave)
+    x = rnd((300, 2500), 1)
+    x64 = x.astype(np.float64)
+    for src, ref in ((">ij~i", x64.max(1)), ("<ij~i", x64.min(1)), ("+ij~i", x64.sum(1)), ("+ij~j", x64.sum(0)),
+                     (">ij~j", x64.max(0)), ("+ij~i|j:16|ijj'", x64.sum(1)), ("+ij~.", x64.sum())):
+        comp = i(src)
+        got = comp.exec_numpy(x)
+        # sums of 2500 unit normals: the bar is relative to the sum of magnitudes, which bounds the rounding error
+        assert np.abs(got - ref).max() <= RTOL_F32 * np.abs(x64).sum(1).max(), src
+        if wave is None and src in (">ij~i", "+ij~i", "+ij~j"):
+            assert "_w: one wavefront per iteration" in comp.report(), comp.report()
+        if wave == "0":
+            assert "_w:" not in comp.report()
+    small = rnd((37, 130), 2)
+    for src in ("+ij~i", ">ij~j", "*ij~i"):
+        comp = i(src)  # (kept alive: the oracle reads the component behind the handle)
+        close(comp.exec_numpy(small * 0.5 + 1), oracle.compile_component(comp.handle).run(small * 0.5 + 1), RTOL_F32)
+    # a product fused into its row sum (a matrix-vector product), then the reference's mlp at a size with long rows
+    w1, v, w2 = rnd((200, 1500), 3), rnd((1500,), 4), rnd((70, 200), 5)
+    fused = i("ij*j~ij||ij") >> i("+ij~i||ij0")
+    close(fused.exec_numpy(w1, v), w1.astype(np.float64) @ v.astype(np.float64), RTOL_F32)
+    mvp = i("ij*j~ij") >> i("+ij~i")
+    mlp = (i("ij~ij") | (mvp >> i(">i~i"))) >> mvp
+    close(mlp.exec_numpy(w2, w1, v), w2.astype(np.float64) @ np.maximum(w1.astype(np.float64) @ v, 0), RTOL_F32)
+    # batched rows, sums over two axes, short rows (which stay with one work-item per row)
+    xb = rnd((5, 33, 700), 6)
+    close(i("+bij~bi").exec_numpy(xb), xb.astype(np.float64).sum(2), RTOL_F32)
+    close(i("+bij~b").exec_numpy(xb), xb.astype(np.float64).sum((1, 2)), 5e-4)
+    close(i(">ij~i").exec_numpy(rnd((5000, 20), 7)), rnd((5000, 20), 7).max(1), RTOL_F32)
+    # the device entry, twice: same bits
+    xd = torch.from_numpy(x).cuda()
+    assert torch.equal(i("+ij~i").exec_torch(xd), i("+ij~i").exec_torch(xd))
+
+
 def test_per_nest_launches_are_refused_on_a_real_device():
     """ILANG_HIP_PHASES=1 (one launch per top-level loop nest of a generated kernel) is confined to the CPU emulation
     of the runtime: on a device the executor refuses such a kernel before launching it."""

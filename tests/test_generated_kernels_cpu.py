@@ -24,7 +24,7 @@ def shim_lib():
     return shim_build.build()
 
 
-def run_cases(shim_lib, extra_env):
+def run_cases(shim_lib, extra_env, names=()):
     env = dict(os.environ)
     env.pop("ILANG_HIP_PHASES", None)
     # ILANG_HIP_UNCHECKED: plain accesses instead of the bounds-checked ones the product emits, so that an access
@@ -32,7 +32,7 @@ def run_cases(shim_lib, extra_env):
     env.update({"ILANG_CORE_LIB": str(shim_lib), "ILANG_HIPCC": str(SHIM / "hostcc.py"), "ILANG_HIP_GENERATED_ONLY": "1",
                 "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1", "ILANG_HIP_UNCHECKED": "1"})
     env.update(extra_env)
-    r = subprocess.run([sys.executable, str(SHIM / "run_cases.py")], env=env, capture_output=True, text=True, timeout=900)
+    r = subprocess.run([sys.executable, str(SHIM / "run_cases.py"), *names], env=env, capture_output=True, text=True, timeout=900)
     last = [l for l in r.stdout.splitlines() if l.startswith("CASE")][-1:] or ["(none started)"]
     assert r.returncode == 0, f"exit {r.returncode}; last case: {last[0]}\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
     assert "failed: []" in r.stdout
@@ -51,6 +51,15 @@ def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
     """Work-items run last to first: a dependency between work-items would change the result."""
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse"})
     run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
+
+
+def test_wavefront_form_of_reduction_nests_matches_too(shim_lib):
+    """ILANG_HIP_WAVE=1 takes the form of a nest in which a wavefront stands where a work-item stood (reduction
+    loops spread over its 64 lanes, lane shares combined by a butterfly) wherever a nest has one; the emulation
+    runs the lanes as 64 threads.  The order of a sum changes, hence the f32 bar instead of 1e-5."""
+    run_cases(shim_lib, {"ILANG_HIP_WAVE": "1", "ILANG_SHIM_CASES": "wave", "ILANG_SHIM_TOLERANCE": "1e-4"})
+    run_cases(shim_lib, {"ILANG_HIP_WAVE": "1", "ILANG_SHIM_TOLERANCE": "1e-4", "ILANG_HIP_UNCHECKED": "0"},
+              names=["row sum 5x300", "fused matrix-vector product", "column max", "mlp with pair"])
 
 
 def test_checked_accesses_give_the_same_results(shim_lib):
