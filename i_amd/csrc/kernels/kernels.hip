@@ -130,7 +130,8 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
   gemm_nt_f32_direct_body<256, 2, 4>(p);
 }
 
-// row_<op>_wave_{v,s}<NV> and row_<op>_block for op = softmax, shift (x - row max), norm (x / row sum), exp
+// row_<op>_wave_{v,s}<NV>, row_<op>_sub_{v,s}<G>, row_<op>_group_{v,s}<NV> and row_<op>_block[_v] for op = softmax,
+// shift (x - row max), norm (x / row sum), exp, scaled_softmax
 #define ROW_WAVE(OP, MODE, NV)                                                                     \
   extern "C" __global__ void __launch_bounds__(256) row_##OP##_wave_v##NV(SoftmaxParams p) {       \
     row_softmax_wave_body<NV, true, MODE>(p);                                                      \
@@ -139,7 +140,7 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
     row_softmax_wave_body<NV, false, MODE>(p);                                                     \
   }
 // row_<op>_group_{v,s}<NV>: 8192 < cols <= 4096 * NV, one workgroup of 16 wavefronts per row, row in registers
-// (no s16: element-wise loads of 64 values per lane do not fit 128 registers; such rows take the three-pass kernel)
+// (no s16: element-wise loads of 64 values per lane do not fit 128 registers; such rows take the two-pass kernel)
 #define ROW_GROUP_V(OP, MODE, NV)                                                                  \
   extern "C" __global__ void __launch_bounds__(1024) row_##OP##_group_v##NV(SoftmaxParams p) {     \
     row_softmax_group_body<NV, true, MODE>(p);                                                     \
@@ -149,12 +150,25 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
   extern "C" __global__ void __launch_bounds__(1024) row_##OP##_group_s##NV(SoftmaxParams p) {     \
     row_softmax_group_body<NV, false, MODE>(p);                                                    \
   }
+// row_<op>_sub_{v,s}<G>: cols <= 4 G <= 128, G lanes per row (64 / G rows per wavefront)
+#define ROW_SUB(OP, MODE, G)                                                                       \
+  extern "C" __global__ void __launch_bounds__(256) row_##OP##_sub_v##G(SoftmaxParams p) {         \
+    row_softmax_sub_body<G, true, MODE>(p);                                                        \
+  }                                                                                                \
+  extern "C" __global__ void __launch_bounds__(256) row_##OP##_sub_s##G(SoftmaxParams p) {         \
+    row_softmax_sub_body<G, false, MODE>(p);                                                       \
+  }
 #define ROW_OP(OP, MODE)                                                                           \
   ROW_WAVE(OP, MODE, 1) ROW_WAVE(OP, MODE, 2) ROW_WAVE(OP, MODE, 4) ROW_WAVE(OP, MODE, 8)          \
   ROW_WAVE(OP, MODE, 16) ROW_WAVE(OP, MODE, 32)                                                    \
   ROW_GROUP(OP, MODE, 4) ROW_GROUP(OP, MODE, 8) ROW_GROUP_V(OP, MODE, 16)                           \
+  ROW_SUB(OP, MODE, 1) ROW_SUB(OP, MODE, 2) ROW_SUB(OP, MODE, 4) ROW_SUB(OP, MODE, 8)              \
+  ROW_SUB(OP, MODE, 16) ROW_SUB(OP, MODE, 32)                                                      \
   extern "C" __global__ void __launch_bounds__(1024) row_##OP##_block(SoftmaxParams p) {           \
-    row_softmax_block_body<MODE>(p);                                                               \
+    row_softmax_block_body<MODE, false>(p);                                                        \
+  }                                                                                                \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_block_v(SoftmaxParams p) {         \
+    row_softmax_block_body<MODE, true>(p);                                                         \
   }
 ROW_OP(softmax, 0)
 ROW_OP(shift, 1)

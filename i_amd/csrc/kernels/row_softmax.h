@@ -4,7 +4,8 @@
 // The reference's valid schedules materialise the shifted / exponentiated row
 // (three kernels, ilang-python/flash-attn.py:60-62); here the row lives in
 // registers, so HBM sees exactly one read and one write per element.
-// One wavefront owns one row; reductions use cross-lane shuffles only.  Loads and stores are non-temporal: with
+// One wavefront owns one row (a group of lanes for rows of at most 128 columns, a workgroup for rows beyond
+// 8192); reductions use cross-lane shuffles, and 16 words of LDS across wavefronts.  Loads and stores are non-temporal: with
 // ordinary loads the kernel looks 12 % faster when it is timed on one buffer over and over (the input then comes
 // partly out of the 256 MiB Infinity Cache) and is 6 % slower on inputs that really come from HBM.
 //
@@ -215,51 +216,203 @@ __device__ __forceinline__ void row_softmax_group_body(const SoftmaxParams& p) {
   for (int t = 0; t < NV; ++t) store(t, r[t] * inv);
 }
 
-// Any width: one workgroup per row, three passes over the row (max, sum, write).
-template <int MODE>
-__device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
-  __shared__ float red[16];
-  const uint32_t row = blockIdx.x;
-  const float* __restrict__ x = p.x + (size_t)row * p.cols;
-  float* __restrict__ y = p.y + (size_t)row * p.cols;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  if constexpr (MODE == 3) {  // exp(x), elementwise
-    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = fast_exp2(x[j] * I_LOG2_E32);
+// Rows of at most 128 columns: G lanes own one row (4 G >= cols, one float4 chunk per lane), so a wavefront
+// works on 64 / G rows at once and its loads cover consecutive rows; the reductions are butterflies inside the
+// groups of G lanes.  (With a wavefront per row, a row of 16 columns occupied 4 lanes of 64.)
+template <int G, bool VEC, int MODE>
+__device__ __forceinline__ void row_softmax_sub_body(const SoftmaxParams& p) {
+  const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint64_t row = gid / G;
+  const uint32_t col = 4u * (uint32_t)(gid % G);
+  const bool live = row < p.rows;  // lanes of rows past the end take part in the exchanges with neutral values
+  const float* __restrict__ x = p.x + row * p.cols;
+  float* __restrict__ y = p.y + row * p.cols;
+  const float pad = MODE == 2 ? 0.0f : -INFINITY;
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;
+  f32x4 r = {pad, pad, pad, pad};
+  if (live) {
+    if (VEC) {
+      if (col < p.cols) {
+        r = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + col));
+        if constexpr (MODE == 4) r *= sc;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (col + e < p.cols) r[e] = MODE == 4 ? x[col + e] * sc : x[col + e];
+    }
+  }
+  auto store = [&](f32x4 v) {
+    if (!live) return;
+    if (VEC) {
+      if (col < p.cols) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(y + col));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (col + e < p.cols) y[col + e] = v[e];
+    }
+  };
+  auto group_max = [](float v) {
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+  };
+  auto group_sum = [](float v) {
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+  };
+  if constexpr (MODE == 3) {
+    f32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = fast_exp2(r[e] * I_LOG2_E32);
+    store(v);
     return;
   }
-  if constexpr (MODE == 2) {  // row_normalize
-    float total = 0.0f;
-    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) total += x[j];
-    total = wave_sum(total);
-    if (lane == 0) red[wave] = total;
-    __syncthreads();
-    total = 0.0f;
-    for (int w = 0; w < nw; ++w) total += red[w];
-    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] / total;
+  if constexpr (MODE == 2) {
+    const float total = group_sum((r[0] + r[1]) + (r[2] + r[3]));
+    store(r / total);
     return;
   }
-  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;  // mode 4: softmax(scale * x)
-  float mx = -INFINITY;
-  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) mx = fmaxf(mx, x[j] * sc);
-  mx = wave_max(mx);
-  if (lane == 0) red[wave] = mx;
-  __syncthreads();
-  mx = red[0];
-  for (int w = 1; w < nw; ++w) mx = fmaxf(mx, red[w]);
-  __syncthreads();
-  if constexpr (MODE == 1) {  // row_max_shift
-    for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) y[j] = x[j] - mx;
+  const float mx = group_max(fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3])));
+  if constexpr (MODE == 1) {
+    store(r - mx);
     return;
   }
   const float mb = mx * I_LOG2_E32;
   float sum = 0.0f;
-  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x) sum += fast_exp2(__builtin_fmaf(x[j] * sc, I_LOG2_E32, -mb));
-  sum = wave_sum(sum);
-  if (lane == 0) red[wave] = sum;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    r[e] = fast_exp2(__builtin_fmaf(r[e], I_LOG2_E32, -mb));
+    sum += r[e];
+  }
+  sum = group_sum(sum);
+  store(r * (1.0f / sum));
+}
+
+// Any width (rows beyond what a workgroup's registers hold): one workgroup of 16 wavefronts per row and two
+// passes over it.  The first pass takes the row max and the row sum together: every lane keeps a running max m
+// and the sum of exp(x - m) over what it has seen, rescaling the sum when its max moves, and lanes, then
+// wavefronts, combine their (m, sum) pairs the same way; the second pass writes.  HBM sees the row twice on the
+// way in at most (the second read of a row of a few hundred KiB comes out of the caches) and once on the way out.
+// VEC: cols % 4 == 0 and 16-byte aligned rows, float4 accesses.
+template <int MODE, bool VEC>
+__device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
+  __shared__ float red[2][16];
+  const uint32_t row = blockIdx.x;
+  const float* __restrict__ x = p.x + (size_t)row * p.cols;
+  float* __restrict__ y = p.y + (size_t)row * p.cols;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  constexpr int W = VEC ? 4 : 1;                    // elements per access
+  const uint32_t chunks = VEC ? p.cols / 4 : p.cols;
+  auto load = [&](uint32_t c) {
+    f32x4 v;
+    if constexpr (VEC) v = *reinterpret_cast<const f32x4*>(x + 4 * (size_t)c);
+    else v[0] = x[c];
+    return v;
+  };
+  auto store = [&](uint32_t c, f32x4 v) {
+    if constexpr (VEC) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(y + 4 * (size_t)c));
+    else y[c] = v[0];
+  };
+  if constexpr (MODE == 3) {  // exp(x), elementwise
+#pragma unroll 4
+    for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+      f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = fast_exp2(v[e] * I_LOG2_E32);
+      store(c, v);
+    }
+    return;
+  }
+  // the reduction of a per-lane value over the workgroup (every lane gets it), wavefront partials in order
+  auto over_workgroup = [&](float v, auto combine) {
+    if (lane == 0) red[0][wave] = v;
+    __syncthreads();
+    float total = red[0][0];
+    for (int w = 1; w < nw; ++w) total = combine(total, red[0][w]);
+    return total;
+  };
+  if constexpr (MODE == 2) {  // row_normalize
+    float total = 0.0f;
+#pragma unroll 4
+    for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+      const f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) total += v[e];
+    }
+    total = over_workgroup(wave_sum(total), [](float a, float b) { return a + b; });
+#pragma unroll 4
+    for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+      f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = v[e] / total;
+      store(c, v);
+    }
+    return;
+  }
+  if constexpr (MODE == 1) {  // row_max_shift
+    float mx = -INFINITY;
+#pragma unroll 4
+    for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+      const f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) mx = fmaxf(mx, v[e]);
+    }
+    mx = over_workgroup(wave_max(mx), [](float a, float b) { return fmaxf(a, b); });
+#pragma unroll 4
+    for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+      f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] -= mx;
+      store(c, v);
+    }
+    return;
+  }
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;  // mode 4: softmax(scale * x)
+  // (m, s): the running max of t = scale * x * log2(e) and the sum of exp2(t - m) over the elements seen
+  float m = -INFINITY, s = 0.0f;
+  auto weight = [](float from, float to) { return from == to ? 1.0f : fast_exp2(from - to); };  // (-inf to -inf: nothing seen yet)
+  auto merge = [&](float& ma, float& sa, float mb, float sb) {
+    const float mn = fmaxf(ma, mb);
+    sa = sa * weight(ma, mn) + sb * weight(mb, mn);
+    ma = mn;
+  };
+#pragma unroll 4
+  for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+    f32x4 v = load(c);
+    float cm = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+      v[e] = v[e] * sc * I_LOG2_E32;
+      cm = fmaxf(cm, v[e]);
+    }
+    const float mn = fmaxf(m, cm);
+    s *= weight(m, mn);
+#pragma unroll
+    for (int e = 0; e < W; ++e) s += fast_exp2(v[e] - mn);
+    m = mn;
+  }
+  // lanes, then wavefronts
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float mo = __shfl_xor(m, o, 64), so = __shfl_xor(s, o, 64);
+    merge(m, s, mo, so);
+  }
+  if (lane == 0) {
+    red[0][wave] = m;
+    red[1][wave] = s;
+  }
   __syncthreads();
-  sum = 0.0f;
-  for (int w = 0; w < nw; ++w) sum += red[w];
-  const float inv = 1.0f / sum;
-  for (uint32_t j = threadIdx.x; j < p.cols; j += blockDim.x)
-    y[j] = fast_exp2(__builtin_fmaf(x[j] * sc, I_LOG2_E32, -mb)) * inv;
+  m = red[0][0];
+  s = red[1][0];
+  for (int w = 1; w < nw; ++w) merge(m, s, red[0][w], red[1][w]);
+  const float inv = 1.0f / s;
+#pragma unroll 4
+  for (uint32_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+    f32x4 v = load(c);
+#pragma unroll
+    for (int e = 0; e < W; ++e) v[e] = fast_exp2(v[e] * sc * I_LOG2_E32 - m) * inv;
+    store(c, v);
+  }
 }

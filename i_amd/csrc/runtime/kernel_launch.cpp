@@ -291,10 +291,21 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
   static const char* const kOps[5] = {"softmax", "shift", "norm", "exp", "scaled_softmax"};
   SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, scale_ptr, scale};
   hipFunction_t fn;
+  const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+  if (cols <= 128) {
+    // G lanes per row, one float4 chunk each: 64 / G rows per wavefront
+    size_t g = 1;
+    while (4 * g < cols) g *= 2;
+    const std::string name = std::string("row_") + kOps[mode] + "_sub_" + (vec ? "v" : "s") + std::to_string(g);
+    if (note) *note = LaunchNote{name, 0, 0};
+    if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
+    const size_t grid = (rows * g + 255) / 256;
+    if (grid > kMaxGrid) return "row_softmax kernel: grid too large";
+    return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+  }
   if (cols <= 8192) {
     int nv = 1;
     while ((size_t)256 * nv < cols) nv *= 2;
-    const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
     const std::string name = std::string("row_") + kOps[mode] + "_wave_" + (vec ? "v" : "s") + std::to_string(nv);
     if (note) *note = LaunchNote{name, 0, 0};
     if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
@@ -303,7 +314,6 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
     return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
   }
   if (rows > kMaxGrid) return "row_softmax kernel: grid too large";
-  const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
   if (cols <= 32768 || (cols <= 65536 && vec)) {
     // the row still fits the registers of one workgroup of 16 wavefronts: one read and one write per element
     const int nv = cols <= 16384 ? 4 : cols <= 32768 ? 8 : 16;
@@ -312,8 +322,10 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
     if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
     return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
   }
-  if (note) *note = LaunchNote{std::string("row_") + kOps[mode] + "_block", 0, 0};
-  if (Err e = builtin_function((std::string("row_") + kOps[mode] + "_block").c_str(), &fn); !e.empty()) return e;
+  // wider rows: two passes over the row (one for exp, elementwise)
+  const std::string name = std::string("row_") + kOps[mode] + (vec ? "_block_v" : "_block");
+  if (note) *note = LaunchNote{name, 0, 0};
+  if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)rows, 1, 1, 1024, &p, sizeof(p), stream);
 }
 

@@ -152,6 +152,10 @@ int i_hip_gemm_nt_f32(const float* a, const float* b, float* c,
 /*
  * Row softmax over the last axis of an f32 [rows, cols] matrix: the fused
  * kernel for  row_max_shift >> exp >> row_normalize  (README.md:19-25).
+ * Any cols: up to 65536 columns a row is read once and written once (it lives
+ * in the registers of a group of lanes, a wavefront or a workgroup), wider
+ * rows are read twice.  16-byte aligned operands with cols % 4 == 0 take the
+ * float4 forms.
  */
 int i_hip_row_softmax(const float* x, float* y, size_t rows, size_t cols, void* stream);
 

@@ -295,7 +295,7 @@ def test_matmul_nn_batched_and_the_demo_mm(torch):
     close(mm.exec_numpy(p_, v_), oracle.compile_component(mm.handle).run(p_, v_), RTOL_F32)
 
 
-@pytest.mark.parametrize("rows,cols", [(37, 100), (64, 4096), (5, 9000), (300, 33)])
+@pytest.mark.parametrize("rows,cols", [(37, 100), (64, 4096), (5, 9000), (300, 33), (1000, 16), (3, 70000), (2, 70002)])
 def test_row_max_shift_and_row_normalize_kernels(torch, rows, cols):
     x = rnd((rows, cols), 1)
     shift = (I & i(">ij~i|i:16,j:16|jii'j'")) >> i("ij-i~ij|i:16,j:16|1jii'j'")
