@@ -76,6 +76,29 @@ __device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_
   tile = slot % per_group;
 }
 
+// Output tile of a large-tile GEMM workgroup.  The tiles are numbered block by block (blocks of 4 x 8 tiles, the
+// blocks of one block column after the other, blocks at the far edges being as small as the tile grid leaves
+// them; inside a block the m index runs fastest), and that sequence is cut into 8 equal runs, one per XCD:
+// workgroup id (xcd = id % 8, slot = id / 8) takes tile number xcd * ceil(T / 8) + slot of it.  The 32 CUs
+// of an XCD thus work on consecutive tiles (at most 1024 rows of A and 2048 of B at a time, shared through the
+// XCD's L2), and the XCDs get the same number of tiles to within one: with whole blocks dealt out to XCDs
+// instead, 22 x 22 tiles (18 blocks) cost three rounds of workgroups where two suffice.
+// Launch with 8 * ceil(T / 8) workgroups per batch.  Returns false for a workgroup that has no tile.
+__device__ __forceinline__ bool gemm_tile_of_workgroup(uint32_t id, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm,
+                                                       uint32_t& tn) {
+  const uint32_t total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
+  const uint32_t slot = id >> 3, at = (id & 7u) * per_xcd + slot;
+  if (slot >= per_xcd || at >= total) return false;
+  const uint32_t column = tiles_m * 8;            // tiles in a full block column
+  const uint32_t bn = at / column, in_column = at - bn * column;
+  const uint32_t wn = min(8u, tiles_n - 8 * bn);  // width of this block column, in tiles
+  const uint32_t bm = in_column / (4 * wn), in_block = in_column - bm * 4 * wn;
+  const uint32_t hm = min(4u, tiles_m - 4 * bm);  // height of this block
+  tm = 4 * bm + in_block % hm;
+  tn = 8 * bn + in_block / hm;
+  return true;
+}
+
 // One 16-byte-per-lane global -> LDS transfer.  `lds_base` (wave-uniform) is where lane 0's
 // 16 bytes land; lane l lands at lds_base + 16 l.  `base` is wave-uniform, `voff` per lane.
 // The compiler is not told that LDS is written: completion is awaited explicitly with

@@ -8,7 +8,9 @@
 // 16x16x32 MFMAs per second than 32x32x16 ones under its power limit, at the same operand traffic from LDS.
 //
 //   workgroup   WM x WN waves; a wave owns (BT / WM) x (BT / WN) of the tile as TM x TN accumulators of
-//               16 x 16 (256 x 256 with 2 x 4 waves: 8 x 4 accumulators, 128 registers)
+//               16 x 16 (256 x 256 with 2 x 4 waves: 8 x 4 accumulators, 128 registers; with 2 x 2 waves, one per
+//               SIMD: 8 x 8 accumulators, the 256 registers of the accumulation file, a third fewer operand
+//               reads per matrix instruction; that form's matrix instructions are inline assembly, see kstep)
 //   operands    a lane holds 8 consecutive k of one row: row = lane % 16 of the 16-row fragment, 16-byte
 //               chunk 4 ks + lane / 16 of the 128-byte slab row (ks = 0, 1: two k-steps of 32 per slab).
 //               The 16 rows one quarter-wave reads with one ds_read_b128 fall into 16 different bank groups
@@ -97,6 +99,9 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     r += NWAVES * RPW * it;
     return (r < lim ? r : lim) * (uint32_t)row_bytes + ch_bytes;
   };
+  uint32_t voff_it[WLW];  // (k <= 2^22: 256 rows of 2 k bytes stay below 2^32)
+#pragma unroll
+  for (int it = 0; it < WLW; ++it) voff_it[it] = voff0 + (uint32_t)it * (uint32_t)it_stride;
   const char* a_tile = A + (size_t)m0 * row_bytes;
   const char* b_tile = NN ? B + (size_t)n0 * 2 : B + (size_t)n0 * row_bytes;
   // NN: wave-load w of a B slab covers slab rows (k) RPWN w .. + RPWN - 1; this lane's LDS slot is (row, chunk
@@ -141,6 +146,11 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     } else if constexpr (EDGE) {
       if (r < WLW) move(a_tile + k_byte, row_offset(it, lim_a), to_a, valid);
       else move(b_tile + k_byte, row_offset(it, lim_b), to_b, valid);
+    } else if constexpr (TM * TN > 32) {
+      // (one wave per SIMD: nothing hides the scalar address arithmetic of a request, so the wave-loads differ in
+      // a per-lane offset kept in a register each, and the base moves once per slab)
+      if (r < WLW) move(a_tile + k_byte, voff_it[it], to_a, valid);
+      else move(b_tile + k_byte, voff_it[it], to_b, valid);
     } else {
       if (r < WLW) move(a_tile + k_byte + it * it_stride, voff0, to_a, valid);
       else move(b_tile + k_byte + it * it_stride, voff0, to_b, valid);
@@ -169,6 +179,23 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  // The matrix instructions of the 256-accumulator form are inline assembly (see kstep), which the compiler's
+  // hazard handling does not look into: the wait states between an ordinary write of an accumulator register
+  // and the first matrix instruction that reads it, and between the last matrix instruction and the first
+  // ordinary read of its result, are spelled out here and after the k loop.
+  constexpr bool ASM_MFMA = TM * TN > 32;
+  auto settle = [&]() {
+    if constexpr (ASM_MFMA) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+    }
+  };
+  if constexpr (ASM_MFMA) {
+    settle();                         // the zeros are in their registers here ...
+    asm volatile("s_nop 7");          // ... and have landed before anything below reads them
+  }
 
 #pragma unroll
   for (int r = 0; r < 2 * WLW; ++r) request(0, 0, r, std::true_type{});
@@ -200,7 +227,13 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bc[j], a[i], acc[i][j], 0, 0, 0);
+        if constexpr (ASM_MFMA) {
+          // 256 accumulator registers: named as the accumulation file, the operands as the ordinary one (left to
+          // itself the register allocator moves values between the two files three times per instruction)
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bc[j]), "v"(a[i]));
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bc[j], a[i], acc[i][j], 0, 0, 0);
+        }
         const int slot = i * TN + j;
         if (refill) {
           if (i == 0) load_b(buf, ks, j, bn);
@@ -230,6 +263,16 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   for (int i = 0; i < TM; ++i) a[i] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
 #pragma unroll
   for (int j = 0; j < TN; ++j) b0[j] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+  if constexpr (ASM_MFMA) {
+    // (these zeros are written by ordinary vector instructions, and a matrix instruction may read a register two
+    // wait states after such a write at the earliest: a matrix instruction that came sooner multiplied what the
+    // registers held before, which is NaN now and then)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(a[i]));
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(b0[j]));
+    asm volatile("s_nop 3");
+  }
   uint32_t s = 0;
   // KTAIL: trip s requests slab s + 1, so the trips before nslabs - 2 request whole slabs; the two or three that
   // remain after the pairs of them are written out with the per-lane test
@@ -247,6 +290,12 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   }
   // last k-step of the last slab
   kstep(b0, b1, 0, 0, false, std::false_type{}, 0, 0, std::false_type{});
+  if constexpr (ASM_MFMA) {
+    // an 8-pass matrix instruction needs 11 wait states before its result may be read by another kind of
+    // instruction; the reads below are tied to this point
+    asm volatile("s_nop 15\n\ts_nop 15");
+    settle();
+  }
 
   // ---- store.  acc[i][j][r] is C[m0 + 16 (wm TM + i) + c16][n0 + 16 (wn TN + j) + 4 g + r]: a lane writes four
   // consecutive columns at once, a quarter-wave 16 rows of them.  Columns come in fours, so a C whose n is not
@@ -283,15 +332,9 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
 template <int BT, int WM, int WN, bool NN = false, bool KTAIL = false>
 __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
-  // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
-  constexpr uint32_t SBM = 4, SBN = 8, SB = SBM * SBN;
-  const uint32_t nsb_m = (p.tiles_m + SBM - 1) / SBM, nsb_n = (p.tiles_n + SBN - 1) / SBN;
-  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t sb = (slot / SB) * 8u + xcd, within = slot % SB;
-  if (sb >= nsb_m * nsb_n) return;
-  const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
-  const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
-  if (tm >= p.tiles_m || tn >= p.tiles_n) return;
+  // ---- tile of this workgroup
+  uint32_t tm, tn;
+  if (!gemm_tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
   if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN, KTAIL>(p, smem, tm, tn);
   else gemm_nt_mfma16_tile<BT, WM, WN, true, NN, KTAIL>(p, smem, tm, tn);
 }

@@ -19,7 +19,7 @@
 //   operands    both A rows and B rows are K-contiguous, so both MFMA operands are plain ds_read_b128 of
 //               (row, chunk 2 ks + h).  The instruction's operands are one f32 per lane with k = lane / 32: a
 //               16-byte operand read covers k = 4 (2 ks + h) .. + 3, and element e of it feeds MFMA e of the k-step.
-//   L2          the workgroup ids that land on one XCD (id % 8) fill a block of 4 x 8
+//   L2          the workgroup ids that land on one XCD (id % 8) walk blocks of 4 x 8
 //               tiles, so at any time an XCD streams 1024 rows of A and 2048 rows of B
 //   M, N edges  rows past the end re-read the last valid row and are not stored
 // Requires k % 32 == 0.
@@ -48,15 +48,9 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   static_assert(BMT == BNT && WL % NWAVES == 0 && NWAVES % 2 == 0, "slab shape");
   __shared__ __attribute__((aligned(1024))) char smem[2][2][SLAB];  // [buffer][A, B]
 
-  // ---- tile of this workgroup: super-blocks of SBM x SBN tiles, one per XCD at a time
-  constexpr uint32_t SBM = 4, SBN = 8, SB = SBM * SBN;
-  const uint32_t nsb_m = (p.tiles_m + SBM - 1) / SBM, nsb_n = (p.tiles_n + SBN - 1) / SBN;
-  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t sb = (slot / SB) * 8u + xcd, within = slot % SB;
-  if (sb >= nsb_m * nsb_n) return;
-  const uint32_t tm = (sb % nsb_m) * SBM + within % SBM;
-  const uint32_t tn = (sb / nsb_m) * SBN + within / SBM;
-  if (tm >= p.tiles_m || tn >= p.tiles_n) return;
+  // ---- tile of this workgroup
+  uint32_t tm, tn;
+  if (!gemm_tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
   const uint32_t batch = blockIdx.y;
 
   const int tid = threadIdx.x;

@@ -110,6 +110,14 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nn_bf16_128x128x64_dir
   gemm_nt_mfma16_body<128, 2, 2, true>(p);
 }
 // k a multiple of 8 but not of 64: the last slab partial
+// ..._w4: the 256 x 256 tile with four waves of 128 x 128 (one per SIMD, its 256 accumulator registers in the
+// accumulation file): a third fewer operand reads from LDS per matrix instruction than with eight waves
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_direct_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_direct_ktail_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2, false, true>(p);
+}
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct_ktail(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 4, false, true>(p);
 }

@@ -152,15 +152,17 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }
 
 // 256 x 256 tiles (one workgroup per CU, 256 at a time) or 128 x 128 tiles (two per CU, 512 at a time) for a
-// problem with enough of either?  The larger tile is about 20 % more efficient per flop (1420 against 1214 TFLOP/s
+// problem with enough of either?  The larger tile is about 20 % more efficient per flop (1442 against 1237 TFLOP/s
 // at 4096^3, whole rounds of either), but its last round of workgroups may leave most of the chip idle: 4608^3 is
-// 1.27 rounds of 256-tiles (measured 1037 TFLOP/s) and 2.53 rounds of 128-tiles (1101).  Rounds of the two-per-CU
-// kernel count in halves.  (A model, within 5 % of the better tile from 1024^3 to 8192^3: it misjudges 3072^3 and
-// 6144^3 by 4 % and 2 %.)
+// 1.27 rounds of 256-tiles (measured 1061 TFLOP/s) and 2.53 rounds of 128-tiles (1092).  Rounds of the two-per-CU
+// kernel count in halves.  A round that leaves part of the chip idle runs its tiles faster (the clock rises when
+// fewer CUs draw power): 1600 per filled CU-round against 1460 for full rounds.  (A model, within 3 % of the
+// better tile from 1024^3 to 8192^3 in steps of 512.)
 static unsigned pick_direct_tile(size_t t256, size_t t128) {
   const double r256 = (double)t256 / 256.0, r128 = (double)t128 / 512.0;
-  const double e256 = 1430.0 * r256 / std::ceil(r256);
-  const double e128 = 1144.0 * r128 / (std::ceil(2.0 * r128) / 2.0);
+  const double fill256 = r256 / std::ceil(r256);
+  const double e256 = (fill256 > 0.95 ? 1460.0 : 1600.0) * fill256;
+  const double e128 = (r128 < 1.0 ? 1250.0 : 1150.0) * r128 / (std::ceil(2.0 * r128) / 2.0);
   return e256 >= e128 ? 256 : 128;
 }
 
@@ -185,7 +187,7 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   {
     const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
     unsigned tile = 0;  // 0: register-staged kernel
-    if (k >= 512 && t256 >= 128) tile = pick_direct_tile(t256, t128);
+    if (k >= 512 && t256 >= 64) tile = pick_direct_tile(t256, t128);
     else if (k >= 256 && t128 >= 64) tile = 128;
     if (tile_m == 256 && tile_n == 256) tile = 256;
     if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
@@ -194,15 +196,18 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
     if (tile && k <= (size_t(1) << 22) && bh <= 65535) {
       p.tiles_m = (uint32_t)((m + tile - 1) / tile);
       p.tiles_n = (uint32_t)((n + tile - 1) / tile);
-      const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs
-      const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+      const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
+      // the 256 x 256 tile runs with four waves of 128 x 128 (ILANG_GEMM_WAVES=8: the form with eight of 128 x 64,
+      // kept for comparison: equal on one round of tiles, 5-10 % behind on several)
+      const char* waves = std::getenv("ILANG_GEMM_WAVES");
+      const bool w4 = tile == 256 && !(waves && std::atoi(waves) == 8);
       const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct") +
-                               (ktail ? "_ktail" : "");
+                               (ktail ? "_ktail" : "") + (w4 ? "_w4" : "");
       if (note) *note = LaunchNote{name, tile, tile};
       if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-      return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
+      return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
     }
   }
   p.tiles_m = (uint32_t)((m + 127) / 128);
@@ -243,8 +248,7 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
   p.tiles_m = (uint32_t)((m + tile - 1) / tile);
   p.tiles_n = (uint32_t)((n + tile - 1) / tile);
-  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks, dealt to the 8 XCDs
-  const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+  const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
   hipFunction_t fn;
   const std::string name = std::string(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct") +
@@ -271,8 +275,7 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = std::atoi(f) == 128 ? 128 : 256;
   p.tiles_m = (uint32_t)((m + tile - 1) / tile);
   p.tiles_n = (uint32_t)((n + tile - 1) / tile);
-  const size_t nsb = ((size_t(p.tiles_m) + 3) / 4) * ((size_t(p.tiles_n) + 7) / 8);  // 4 x 8 tile blocks
-  const size_t grid = ((nsb + 7) / 8 * 8) * 32;
+  const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
   hipFunction_t fn;
   const char* name = tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct";

@@ -481,12 +481,14 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
                                       (3, 257, 255, 320)])
-@pytest.mark.parametrize("direct", ["256", "128", "0"])
+@pytest.mark.parametrize("direct", ["256", "256w8", "128", "0"])
 def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
-    """The launcher picks between the 256 x 256 and 128 x 128 direct-to-LDS kernels and the register-staged
-    kernel by problem size; force each of them on small ragged problems with 1 to 5 k-slabs, edge tiles on
-    both axes and several batches."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
+    """The launcher picks between the 256 x 256 (four waves; "w8": the form with eight) and 128 x 128
+    direct-to-LDS kernels and the register-staged kernel by problem size; force each of them on small ragged
+    problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct[:3])
+    if direct.endswith("w8"):
+        monkeypatch.setenv("ILANG_GEMM_WAVES", "8")
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -500,11 +502,13 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, dire
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 8), (1, 300, 264, 40), (2, 600, 520, 136), (1, 1, 8, 200), (3, 257, 256, 1000),
                                       (1, 128, 128, 72)])
 @pytest.mark.parametrize("nn", [False, True])
-@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("tile", ["128", "256", "256w8"])
 def test_gemm_bf16_k_that_is_no_multiple_of_64(env, monkeypatch, bh, m, n, k, nn, tile):
     """k % 8 == 0 but k % 64 != 0: the direct kernels with a partial last slab (the lanes past k clear their LDS
-    slots), both tile sizes forced here at small sizes; NT and NN, f32 and bf16 output."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile)
+    slots), both tile sizes (and both forms of the larger) forced here at small sizes; NT and NN, f32 and bf16 output."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile[:3])
+    if tile.endswith("w8"):
+        monkeypatch.setenv("ILANG_GEMM_WAVES", "8")
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
