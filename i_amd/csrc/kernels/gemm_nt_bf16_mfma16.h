@@ -110,15 +110,21 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   constexpr int RBN = 2 * BT;         // bytes per row of an NN slab
   constexpr int CHN = RBN / 16;       // chunks per row
   constexpr int RPWN = 1024 / RBN;    // rows per wave-load
-  static_assert(!NN || NWAVES * RPWN == 16, "NN slab rounds");
+  // (with four waves a round of wave-loads is 8 rows, and f(row) of a lane alternates between two values from one
+  // round to the next: two offsets, by the parity of the round)
+  constexpr int NN_ROUND = NWAVES * RPWN;  // slab rows per round of the workgroup's wave-loads
+  static_assert(!NN || NN_ROUND == 16 || NN_ROUND == 8, "NN slab rounds");
   const size_t brow_bytes = (size_t)p.n * 2;  // NN: a row of B is n elements
-  uint32_t boff_nn = 0;
+  uint32_t boff_nn[2] = {0, 0};
   if constexpr (NN) {
-    const uint32_t r = wave * RPWN + lane / CHN;
     const uint32_t last_chunk = (p.n - n0) / 8 - 1;  // n % 8 == 0 and n0 < n
-    uint32_t ch = (lane % CHN) ^ (2 * ((r & 3) | (((r >> 3) & 1) << 2)));
-    ch = ch < last_chunk ? ch : last_chunk;
-    boff_nn = r * (uint32_t)brow_bytes + 16 * ch;
+#pragma unroll
+    for (int parity = 0; parity < 2; ++parity) {
+      const uint32_t r = wave * RPWN + lane / CHN + (NN_ROUND == 8 ? 8 * parity : 0);
+      uint32_t ch = (lane % CHN) ^ (2 * ((r & 3) | (((r >> 3) & 1) << 2)));
+      ch = ch < last_chunk ? ch : last_chunk;
+      boff_nn[parity] = (wave * RPWN + lane / CHN) * (uint32_t)brow_bytes + 16 * ch;
+    }
   }
   const uint32_t nslabs = KTAIL ? (p.k + BK - 1) / BK : p.k / BK;
   // KTAIL: what exists of the last slab: 16-byte chunks per row (rows of k for an NN slab of B)
@@ -142,7 +148,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
     const bool valid = whole || gch < tail_chunks;         // ... or this lane's chunk of a K-contiguous row does
     if (r >= WLW && NN) {
       const bool valid_row = whole || (w * RPWN + lane / CHN) < 8 * tail_chunks;
-      move(b_tile + ((size_t)s * BK + 16 * it) * brow_bytes, boff_nn, to_b, valid_row);
+      move(b_tile + ((size_t)s * BK + NN_ROUND * it) * brow_bytes, boff_nn[NN_ROUND == 8 ? it % 2 : 0], to_b, valid_row);
     } else if constexpr (EDGE) {
       if (r < WLW) move(a_tile + k_byte, row_offset(it, lim_a), to_a, valid);
       else move(b_tile + k_byte, row_offset(it, lim_b), to_b, valid);

@@ -118,6 +118,12 @@ extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_dir
 extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_direct_ktail_w4(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 2, false, true>(p);
 }
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nn_bf16_256x256x64_direct_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2, true>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nn_bf16_256x256x64_direct_ktail_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2, true, true>(p);
+}
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_bf16_256x256x64_direct_ktail(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 4, false, true>(p);
 }

@@ -251,11 +251,13 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
   hipFunction_t fn;
+  const char* waves = std::getenv("ILANG_GEMM_WAVES");  // (as for the NT kernels: four waves unless 8 is asked for)
+  const bool w4 = tile == 256 && !(waves && std::atoi(waves) == 8);
   const std::string name = std::string(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct") +
-                           (k % 64 != 0 ? "_ktail" : "");
+                           (k % 64 != 0 ? "_ktail" : "") + (w4 ? "_w4" : "");
   if (note) *note = LaunchNote{name, tile, tile};
   if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
+  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
 }
 
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 32 == 0 && k <= (size_t(1) << 21); }
