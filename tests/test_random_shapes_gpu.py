@@ -1,8 +1,8 @@
-"""Randomised parity sweep of the hand-written attention and GEMM kernels (through the C ABI of include/i_hip.h)
+"""Randomised parity sweep of the hand-written attention, GEMM and row-softmax kernels (through the C ABI of include/i_hip.h)
 against the closed forms in f64, computed on the device by torch: many ragged shapes, every workgroup size and
 tile the launcher can pick, each case run twice.  The seeds are fixed; a mismatch prints the case.
 
-Tolerance 2e-2 of max |reference| for attention (bf16 in, f32 accumulate), 1e-2 for the GEMMs.
+Tolerance 2e-2 of max |reference| for attention (bf16 in, f32 accumulate), 1e-2 for the GEMMs, 1e-4 for the softmax (f32).
 """
 import random
 
@@ -83,3 +83,35 @@ def test_gemm_bf16_random_shapes(env, monkeypatch, seed):
             t.cuda.synchronize()
             err = float((c.double() - ref).abs().max() / ref.abs().max().clamp_min(1e-6))
             assert err <= 1e-2, dict(case=case, nn=nn, bh=bh, m=m, n=n, k=k, direct=direct, rep=rep, err=err)
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_row_softmax_random_shapes(env, seed):
+    """Row widths from 1 to 300000 columns, i.e. every form of the row kernel (several rows per wavefront, a
+    wavefront, a workgroup with the row in registers, a workgroup in two passes), aligned and unaligned, with rows
+    that sit far from zero; against softmax in f64.  Each case runs twice and must repeat bit for bit."""
+    t, nat = env.torch, env.nat
+    rng = random.Random(seed)
+    for case in range(60):
+        band = rng.choice([(1, 128), (1, 128), (129, 8192), (8193, 65536), (65537, 300000)])
+        cols = rng.randint(*band)
+        if rng.random() < 0.5:
+            cols = max(4, cols // 4 * 4)
+        rows = rng.randint(1, max(1, min(700, (1 << 22) // cols)))
+        shift = rng.choice([0.0, 30.0, -80.0])
+        g = t.Generator(device="cuda").manual_seed(7000 * seed + case)
+        offset = rng.choice([0, 0, 1])  # 1: operands start 4 bytes into their allocations
+        xbuf = t.randn(rows * cols + 1, device="cuda", generator=g) * 3 + shift
+        x = xbuf[offset:offset + rows * cols].view(rows, cols)
+        ref = t.softmax(x.double(), dim=-1)
+        results = []
+        for rep in range(2):
+            ybuf = t.full((rows * cols + 2,), float("nan"), device="cuda")
+            nat.check(nat.core.i_hip_row_softmax(x.data_ptr(), ybuf.data_ptr() + 4 * offset, rows, cols, env.stream()))
+            t.cuda.synchronize()
+            y = ybuf[offset:offset + rows * cols].view(rows, cols)
+            err = float((y.double() - ref).abs().max() / ref.abs().max())
+            assert err <= 1e-4, dict(case=case, rows=rows, cols=cols, offset=offset, shift=shift, rep=rep, err=err)
+            assert bool(t.isnan(ybuf[offset + rows * cols:]).all()) and (offset == 0 or bool(t.isnan(ybuf[0])))
+            results.append(y.clone())
+        assert t.equal(results[0], results[1]), dict(case=case, rows=rows, cols=cols)
