@@ -22,7 +22,7 @@
 //   L2          the workgroup ids that land on one XCD (id % 8) walk blocks of 4 x 8
 //               tiles, so at any time an XCD streams 1024 rows of A and 2048 rows of B
 //   M, N edges  rows past the end re-read the last valid row and are not stored
-// Requires k % 32 == 0.
+// Requires k % 32 == 0, or k % 4 == 0 with KTAIL.
 #pragma once
 
 #include "common.h"
@@ -30,7 +30,9 @@
 
 // BT x BT output tile per workgroup of WM x WN waves: 256 with 2 x 4 waves (one workgroup per CU) for large
 // problems, 128 with 2 x 2 waves (two workgroups per CU) for problems with too few 256-tiles to fill the chip.
-template <int BT, int WM, int WN>
+// KTAIL: k is a multiple of 4 but not of 32, the last slab is partial: a lane whose 16-byte chunk lies past k
+// transfers nothing and clears its LDS slot instead, so the slab reads as zeros there.
+template <int BT, int WM, int WN, bool KTAIL = false>
 __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   constexpr int BMT = BT, BNT = BT;
   constexpr int ELEM = 4;            // bytes per operand element
@@ -84,13 +86,24 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   const char* a_tile = A + (size_t)m0 * row_bytes;
   const char* b_tile = B + (size_t)n0 * row_bytes;
   const size_t b_slab_step = (size_t)RB;  // bytes from one k slab of B to the next
+  const uint32_t nslabs = KTAIL ? (p.k + BK - 1) / BK : p.k / BK;
+  const uint32_t tail_chunks = (p.k - (nslabs - 1) * BK) / 4;  // KTAIL: 16-byte chunks per row of the last slab
+  // one transfer of 16 bytes per lane of slab s; KTAIL: nothing to fetch for this lane: its slot is cleared
+  auto move = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t s) {
+    if constexpr (KTAIL) {
+      if (s + 1 < nslabs || gch < tail_chunks) dma16(base, voff, lds_base);
+      else *reinterpret_cast<u32x4*>(&smem[0][0][0] + (lds_base - smem0) + 16 * lane) = u32x4{0, 0, 0, 0};
+    } else {
+      dma16(base, voff, lds_base);
+    }
+  };
   auto request_slab = [&](uint32_t s, int buf) {
     const size_t k_byte = (size_t)s * RB;
 #pragma unroll
     for (int it = 0; it < WLW; ++it) {
       const uint32_t w = wave + NWAVES * it;
-      dma16(a_tile + k_byte, aoff[it], smem0 + (2 * buf + 0) * SLAB + w * 1024);
-      dma16(b_tile + s * b_slab_step, boff[it], smem0 + (2 * buf + 1) * SLAB + w * 1024);
+      move(a_tile + k_byte, aoff[it], smem0 + (2 * buf + 0) * SLAB + w * 1024, s);
+      move(b_tile + s * b_slab_step, boff[it], smem0 + (2 * buf + 1) * SLAB + w * 1024, s);
     }
   };
 
@@ -108,7 +121,6 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  const uint32_t nslabs = p.k / BK;
   request_slab(0, 0);
   dma_wait_all();
   __syncthreads();
@@ -154,8 +166,8 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
         for (int r = slot * NREQ / (TM * TN); r < (slot + 1) * NREQ / (TM * TN); ++r) {
           const int it = r % WLW;
           const uint32_t w = wave + NWAVES * it;
-          if (r < WLW) dma16(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024);
-          else dma16(b_tile + s_req * b_slab_step, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024);
+          if (r < WLW) move(a_tile + k_byte, aoff[it], smem0 + (2 * (buf ^ 1) + 0) * SLAB + w * 1024, s_req);
+          else move(b_tile + s_req * b_slab_step, boff[it], smem0 + (2 * (buf ^ 1) + 1) * SLAB + w * 1024, s_req);
         }
         __builtin_amdgcn_sched_barrier(0);
       }

@@ -143,6 +143,13 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_dire
 extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_direct(GemmParams p) {
   gemm_nt_f32_direct_body<256, 2, 4>(p);
 }
+// k that is a multiple of 4 but not of 32: the last slab partial
+extern "C" __global__ void __launch_bounds__(256, 2) gemm_nt_f32_128x128x32_direct_ktail(GemmParams p) {
+  gemm_nt_f32_direct_body<128, 2, 2, true>(p);
+}
+extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_direct_ktail(GemmParams p) {
+  gemm_nt_f32_direct_body<256, 2, 4, true>(p);
+}
 
 // row_<op>_wave_{v,s}<NV>, row_<op>_sub_{v,s}<G>, row_<op>_group_{v,s}<NV> and row_<op>_block[_v] for op = softmax,
 // shift (x - row max), norm (x / row sum), exp, scaled_softmax

@@ -260,11 +260,13 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
 }
 
-bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 32 == 0 && k <= (size_t(1) << 21); }
+bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 4 == 0 && k <= (size_t(1) << 21); }
 
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
                        hipStream_t stream, LaunchNote* note) {
-  if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 32 (at most 2^21)";
+  if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 4 (at most 2^21)";
+  if (reinterpret_cast<uintptr_t>(a) % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0)
+    return "gemm_nt f32 kernel: operands must be 16-byte aligned";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || bh > 65535) return "gemm_nt f32 kernel: extent too large";
   if (!a || !b || !c) return "gemm_nt f32 kernel: null device pointer";
@@ -280,9 +282,10 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
   hipFunction_t fn;
-  const char* name = tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct";
+  const std::string name = std::string(tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct") +
+                           (k % 32 != 0 ? "_ktail" : "");  // (a partial last slab of 32 k)
   if (note) *note = LaunchNote{name, tile, tile};
-  if (Err e = builtin_function(name, &fn); !e.empty()) return e;
+  if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
   return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
 }
 

@@ -51,7 +51,7 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
                         DType out_dtype = F32);
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
 
-// c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 32 == 0
+// c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 4 == 0 and 16-byte aligned operands
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
                        hipStream_t stream, LaunchNote* note = nullptr);
 bool gemm_nt_f32_supported(size_t k);

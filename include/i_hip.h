@@ -144,7 +144,7 @@ int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c,
 
 /*
  * The same mm_t with f32 a, b, c and f32 products and sums (f32 MFMA), the reference's own
- * arithmetic type: what the host f32 ABI of i.h dispatches to.  Requires k % 32 == 0.
+ * arithmetic type: what the host f32 ABI of i.h dispatches to.  Requires k % 4 == 0 and 16-byte aligned a, b.
  */
 int i_hip_gemm_nt_f32(const float* a, const float* b, float* c,
                       size_t bh, size_t m, size_t n, size_t k, void* stream);

@@ -167,7 +167,7 @@ def test_head_sizes_above_128(torch):
         else:
             assert "attention in three kernels" in comp.report() and "scaled_softmax" in comp.report()
         close(out.cpu().numpy(), oracle.attention_tiled(qb, kb, vb, scale), RTOL_BF16)
-    # extents the GEMM kernels cannot take (f32 with a key count that is no multiple of 32) still run generated
+    # extents the GEMM kernels cannot take (f32 with a key count that is no multiple of 4) still run generated
     q, k, v = rnd((20, 160), 1), rnd((33, 160), 2), rnd((33, 160), 3)
     comp = flash()
     close(comp.exec_numpy(q, k, v), oracle.attention_tiled(q, k, v), RTOL_F32)
@@ -240,11 +240,13 @@ def test_config3_mm_t_bf16_device(torch):
     close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
 
 
-@pytest.mark.parametrize("k", [40, 64])  # 40: generated kernel; 64: f32 MFMA kernel
+@pytest.mark.parametrize("k", [42, 40, 64])  # 42: generated kernel; 40: f32 MFMA kernel with a partial last slab; 64: f32 MFMA kernel
 def test_mm_t_f32_small_vs_emitted_c(torch, k):
     a, b = rnd((100, k), 1), rnd((70, k), 2)
     comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     close(comp.exec_numpy(a, b), oracle.compile_component(comp.handle).run(a, b), RTOL_F32)
+    assert ("generated kernel" in comp.report()) == (k == 42)
+    assert ("_ktail" in comp.report()) == (k == 40)
 
 
 def test_config3_mm_t_through_the_host_f32_abi(torch):

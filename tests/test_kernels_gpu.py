@@ -603,7 +603,9 @@ def test_gemm_nn_bf16_rejects_what_the_direct_kernels_cannot_read(env):
 
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 32), (1, 300, 260, 96), (2, 600, 520, 160), (1, 1, 1, 64),
-                                      (3, 257, 255, 320), (1, 100, 70, 64)])
+                                      (3, 257, 255, 320), (1, 100, 70, 64),
+                                      # k a multiple of 4 but not of 32: a partial last slab
+                                      (1, 256, 256, 40), (2, 300, 260, 100), (1, 100, 70, 4), (3, 257, 255, 1004), (1, 64, 64, 28)])
 @pytest.mark.parametrize("tile", ["256", "128"])
 def test_gemm_nt_f32_vs_oracle(env, monkeypatch, bh, m, n, k, tile):
     """f32 operands, f32 MFMA: the reference's own arithmetic type, against the scalar oracle at the f32 bar."""
@@ -619,10 +621,10 @@ def test_gemm_nt_f32_vs_oracle(env, monkeypatch, bh, m, n, k, tile):
 
 def test_gemm_nt_f32_rejects_ragged_k(env):
     t = env.torch
-    x = t.zeros(64, 40, device="cuda")
+    x = t.zeros(64, 42, device="cuda")
     c = t.zeros(64, 64, device="cuda")
-    rc = env.nat.core.i_hip_gemm_nt_f32(x.data_ptr(), x.data_ptr(), c.data_ptr(), 1, 64, 64, 40, env.stream())
-    assert rc == -1 and "multiple of 32" in env.nat.last_error()
+    rc = env.nat.core.i_hip_gemm_nt_f32(x.data_ptr(), x.data_ptr(), c.data_ptr(), 1, 64, 64, 42, env.stream())
+    assert rc == -1 and "multiple of 4" in env.nat.last_error()
 
 
 def test_gemm_nt_bf16_full_size_linearity(env):
