@@ -530,6 +530,33 @@ def test_gemm_bf16_k_that_is_no_multiple_of_64(env, monkeypatch, bh, m, n, k, nn
         assert t.equal(c16, cd.bfloat16())
 
 
+def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, monkeypatch):
+    """The four-wave form of the 256 x 256 tile spells its matrix instructions as inline assembly and carries its own
+    wait states.  Its first matrix instructions multiply zeroed operands; issued too soon after the zeroing they read
+    what the registers held before, which is visible when that was NaN: products of NaN operands run first here, so
+    that the register file is full of NaN, then several small multi-batch products (many short-lived workgroups)."""
+    monkeypatch.setenv("ILANG_GEMM_DIRECT", "256")
+    t = env.torch
+    poison = t.full((2048, 512), float("nan"), device="cuda", dtype=t.bfloat16)
+    sink = t.empty(2048, 2048, device="cuda")
+    core = env.nat.core
+    for rep in range(6):
+        env.nat.check(core.i_hip_gemm_nt_bf16(poison.data_ptr(), poison.data_ptr(), sink.data_ptr(), 1, 2048, 2048, 512, env.stream()))
+        for bh, m, n, k in ((3, 677, 61, 128), (4, 512, 61, 128), (3, 677, 60, 256), (2, 300, 264, 64)):
+            g = t.Generator(device="cuda").manual_seed(100 * rep + m)
+            a = (t.rand(bh, m, k, device="cuda", generator=g) * 2 - 1).bfloat16()
+            b = (t.rand(bh, n, k, device="cuda", generator=g) * 2 - 1).bfloat16()
+            c = t.full((bh, m, n), 12345.0, device="cuda")
+            env.nat.check(core.i_hip_gemm_nt_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), bh, m, n, k, env.stream()))
+            bn = b[:, : n // 8 * 8].transpose(1, 2).contiguous()  # the same product with a row-major right operand
+            cn = t.full((bh, m, n // 8 * 8), 12345.0, device="cuda")
+            env.nat.check(core.i_hip_gemm_nn_bf16(a.data_ptr(), bn.data_ptr(), cn.data_ptr(), bh, m, n // 8 * 8, k, env.stream()))
+            t.cuda.synchronize()
+            ref = a.double() @ b.double().transpose(1, 2)
+            assert float((c.double() - ref).abs().max()) <= 1e-2 * float(ref.abs().max()), (rep, bh, m, n, k)
+            assert float((cn.double() - ref[:, :, : n // 8 * 8]).abs().max()) <= 1e-2 * float(ref.abs().max()), (rep, bh, m, n, k)
+
+
 @pytest.mark.parametrize("tile", [0, 128, 256])
 def test_gemm_nt_bf16_output_in_bf16(env, monkeypatch, tile):
     """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
