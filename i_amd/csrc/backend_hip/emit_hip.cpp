@@ -614,6 +614,7 @@ const MStmt* find_loop(const std::vector<MStmt>& stmts, const std::string& iter)
 GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const std::vector<bool>& emit) {
   const char* unchecked = std::getenv("ILANG_HIP_UNCHECKED");
   g_checked_accesses = !(unchecked && unchecked[0] == '1');
+  g_held.clear();  // (an error thrown while a loop was being printed must not leave its substitutions behind)
   GenericModule out;
   out.kernels.resize(plan.kernels.size());
   size_t rank = 1;
