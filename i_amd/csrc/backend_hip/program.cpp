@@ -145,6 +145,15 @@ bool attention_in_parts_usable(DType t, size_t bh, size_t nq, size_t nk, size_t 
   return ihip::gemm_nt_bf16_supported(d) && ihip::gemm_nt_bf16_supported(nk);
 }
 
+// A product runs on the matrix-instruction kernels whatever its contracted extent k: when k is no multiple of what
+// they need (8 in bf16, 4 in f32), or f32 operands are not 16-byte aligned, both operands are first copied into
+// temporaries whose rows are padded with zeros (padded_operands below); the padding adds nothing to the sums.
+size_t product_k_quantum(DType t) { return t == DType::BF16 ? 8 : 4; }
+bool product_extent_usable(DType t, size_t k) {
+  const size_t q = product_k_quantum(t), kp = (k + q - 1) / q * q;
+  return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(kp) : ihip::gemm_nt_f32_supported(kp);
+}
+
 // Returns true when kernel k can run on its hand-written form with these operands.
 bool hand_usable(const Run& run, const Recognized& r) {
   // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
@@ -170,14 +179,14 @@ bool hand_usable(const Run& run, const Recognized& r) {
       if (run.dtype_of(r.b.buffer) != t) return false;
       const auto a = rows_cols(r.a);
       if (a.size() < 2) return false;
-      return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
+      return product_extent_usable(t, a.back());
     }
     case Recognized::GemmNN: {
       const DType t = run.dtype_of(r.a.buffer);
       if (run.dtype_of(r.b.buffer) != t) return false;
       const auto a = rows_cols(r.a);
       if (a.size() < 2) return false;
-      return t == DType::BF16 ? ihip::gemm_nt_bf16_supported(a.back()) : ihip::gemm_nt_f32_supported(a.back());
+      return product_extent_usable(t, a.back());
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
@@ -264,6 +273,25 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
   return {};
 }
 
+// The two operands of an NT product ([rows_a, k] and [rows_b, k], dense) as the matrix-instruction kernels can
+// read them: untouched when k is a multiple of their quantum (and, for f32, both are 16-byte aligned), otherwise
+// copied into stream-ordered temporaries with every row padded with zeros up to the next multiple; *k becomes the
+// padded extent.
+ihip::Err padded_operands(Run& run, DType t, const void** a, size_t rows_a, const void** b, size_t rows_b, size_t* k) {
+  const size_t q = product_k_quantum(t), kp = (*k + q - 1) / q * q, elem = t == DType::BF16 ? 2 : 4;
+  const bool misaligned = t == DType::F32 && (reinterpret_cast<uintptr_t>(*a) % 16 != 0 || reinterpret_cast<uintptr_t>(*b) % 16 != 0);
+  if (kp == *k && !misaligned) return {};
+  void *ta = nullptr, *tb = nullptr;
+  if (ihip::Err e = run.alloc(&ta, std::max<size_t>(rows_a * kp * elem, 16)); !e.empty()) return e;
+  if (ihip::Err e = run.alloc(&tb, std::max<size_t>(rows_b * kp * elem, 16)); !e.empty()) return e;
+  if (ihip::Err e = ihip::launch_pad_rows(*a, ta, rows_a, *k, kp, elem, run.stream); !e.empty()) return e;
+  if (ihip::Err e = ihip::launch_pad_rows(*b, tb, rows_b, *k, kp, elem, run.stream); !e.empty()) return e;
+  *a = ta;
+  *b = tb;
+  *k = kp;
+  return {};
+}
+
 ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* note) {
   switch (r.kind) {
     case Recognized::Attention: {
@@ -314,12 +342,14 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
         return e;
       }
-      if (run.dtype_of(r.a.buffer) == DType::F32)
-        return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)),
-                                        static_cast<const float*>(run.raw_ptr(r.b.buffer)), static_cast<float*>(out), bh,
-                                        a[nb], b[nb], a[nb + 1], run.stream, note);
-      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), out, bh, a[nb], b[nb], a[nb + 1],
-                                       run.stream, r.tile_i, r.tile_j, note, out_dt);
+      const DType t = run.dtype_of(r.a.buffer);
+      const void *pa = run.raw_ptr(r.a.buffer), *pb = run.raw_ptr(r.b.buffer);
+      size_t k = a[nb + 1];
+      if (ihip::Err e = padded_operands(run, t, &pa, bh * a[nb], &pb, bh * b[nb], &k); !e.empty()) return e;
+      if (t == DType::F32)
+        return ihip::launch_gemm_nt_f32(static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(out), bh,
+                                        a[nb], b[nb], k, run.stream, note);
+      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, a[nb], b[nb], k, run.stream, r.tile_i, r.tile_j, note, out_dt);
     }
     case Recognized::GemmNN: {
       // b [B.., K, J]: the direct bf16 kernels read it in place; otherwise it is transposed into a stream-ordered
@@ -349,11 +379,13 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       void* bt = nullptr;
       if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;
       if (ihip::Err e = ihip::launch_transpose(run.raw_ptr(r.b.buffer), bt, bh, k, n, elem, run.stream); !e.empty()) return e;
+      const void *pa = run.raw_ptr(r.a.buffer), *pb = bt;
+      size_t kp = k;
+      if (ihip::Err e = padded_operands(run, f32 ? DType::F32 : DType::BF16, &pa, bh * m, &pb, bh * n, &kp); !e.empty()) return e;
       if (f32)
-        return ihip::launch_gemm_nt_f32(static_cast<const float*>(run.raw_ptr(r.a.buffer)), static_cast<const float*>(bt),
-                                        static_cast<float*>(out), bh, m, n, k, run.stream, note);
-      return ihip::launch_gemm_nt_bf16(run.raw_ptr(r.a.buffer), bt, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note,
-                                       out_dt);
+        return ihip::launch_gemm_nt_f32(static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(out), bh,
+                                        m, n, kp, run.stream, note);
+      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, m, n, kp, run.stream, r.tile_i, r.tile_j, note, out_dt);
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:

@@ -229,6 +229,22 @@ __device__ __forceinline__ void transpose_body(const TransposeParams& p) {
   for (uint32_t y = y0; y < 64; y += 4)
     if (c0 + y < p.cols && r0 + x < p.rows) dst[(size_t)(c0 + y) * p.rows + r0 + x] = tile[x][y];
 }
+// rows copied into rows of cols_padded elements, the tail zeroed: what gives a product whose contracted extent the
+// matrix-instruction kernels cannot take (k % 8 != 0 in bf16, k % 4 != 0 in f32) operands they can
+template <class T>
+__device__ __forceinline__ void pad_rows_body(const PadParams& p) {
+  const T* src = reinterpret_cast<const T*>(p.src);
+  T* dst = reinterpret_cast<T*>(p.dst);
+  const uint64_t total = p.rows * p.cols_padded;
+  for (uint64_t at = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; at < total; at += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t r = at / p.cols_padded;
+    const uint32_t c = (uint32_t)(at - r * p.cols_padded);
+    dst[at] = c < p.cols ? src[r * p.cols + c] : T(0);
+  }
+}
+extern "C" __global__ void __launch_bounds__(256) pad_rows_b16(PadParams p) { pad_rows_body<uint16_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) pad_rows_b32(PadParams p) { pad_rows_body<uint32_t>(p); }
+
 extern "C" __global__ void __launch_bounds__(256) transpose_b16(TransposeParams p) { transpose_body<uint16_t>(p); }
 extern "C" __global__ void __launch_bounds__(256) transpose_b32(TransposeParams p) { transpose_body<uint32_t>(p); }
 

@@ -43,6 +43,14 @@ struct ConvertParams {
 };
 
 // dst[b][c][r] = src[b][r][c] for b < bh, r < rows, c < cols; elements of 2 or 4 bytes
+// dst[r][c] = c < cols ? src[r][c] : 0 for r < rows, c < cols_padded; elements of 2 or 4 bytes
+struct PadParams {
+  const void* src;
+  void* dst;
+  uint64_t rows;
+  uint32_t cols, cols_padded;
+};
+
 struct TransposeParams {
   const void* src;
   void* dst;

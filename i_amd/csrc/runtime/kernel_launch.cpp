@@ -366,4 +366,18 @@ Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, h
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
 
+Err launch_pad_rows(const void* src, void* dst, size_t rows, size_t cols, size_t cols_padded, size_t elem_bytes,
+                    hipStream_t stream) {
+  if (elem_bytes != 2 && elem_bytes != 4) return "pad kernel: element size must be 2 or 4 bytes";
+  if (rows == 0 || cols_padded == 0) return {};
+  if (!fits_u32(cols_padded) || cols > cols_padded) return "pad kernel: bad extents";
+  if (!src || !dst) return "pad kernel: null device pointer";
+  PadParams p{src, dst, (uint64_t)rows, (uint32_t)cols, (uint32_t)cols_padded};
+  hipFunction_t fn;
+  if (Err e = builtin_function(elem_bytes == 2 ? "pad_rows_b16" : "pad_rows_b32", &fn); !e.empty()) return e;
+  size_t grid = (rows * cols_padded + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
+}
+
 }  // namespace ihip

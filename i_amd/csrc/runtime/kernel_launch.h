@@ -69,4 +69,8 @@ Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t 
 
 Err launch_convert(const void* src, void* dst, DType from, DType to, size_t n, hipStream_t stream);
 
+// dst[r][c] = c < cols ? src[r][c] : 0 for c < cols_padded; elem_bytes is 2 or 4
+Err launch_pad_rows(const void* src, void* dst, size_t rows, size_t cols, size_t cols_padded, size_t elem_bytes,
+                    hipStream_t stream);
+
 }  // namespace ihip

@@ -240,13 +240,45 @@ def test_config3_mm_t_bf16_device(torch):
     close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
 
 
-@pytest.mark.parametrize("k", [42, 40, 64])  # 42: generated kernel; 40: f32 MFMA kernel with a partial last slab; 64: f32 MFMA kernel
+@pytest.mark.parametrize("k", [42, 40, 64])  # 42: operands padded to k = 44 first; 40: a partial last slab; 64: whole slabs
 def test_mm_t_f32_small_vs_emitted_c(torch, k):
     a, b = rnd((100, k), 1), rnd((70, k), 2)
     comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     close(comp.exec_numpy(a, b), oracle.compile_component(comp.handle).run(a, b), RTOL_F32)
-    assert ("generated kernel" in comp.report()) == (k == 42)
-    assert ("_ktail" in comp.report()) == (k == 40)
+    assert "gemm_nt_f32" in comp.report() and "generated kernel" not in comp.report()
+    assert ("_ktail" in comp.report()) == (k != 64)
+
+
+def test_products_with_any_contracted_extent_run_on_the_matrix_kernels(torch):
+    """A contracted extent that is no multiple of what the matrix-instruction kernels read (4 elements in f32, 8 in
+    bf16) does not fall back to the generated kernel: the executor pads both operands with zero columns first.
+    NT and NN products, f32 and bf16, against float64."""
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    mm = i("ik*kj~ijk|i:2,k:2|ii'jkk'") >> i("+ijk~ij|i:2,k:2|ii'j!kk'0")
+    for k in (1, 7, 42, 1001):
+        a, b = rnd((150, k), 1), rnd((90, k), 2)
+        ref = a.astype(np.float64) @ b.astype(np.float64).T
+        close(mm_t.exec_numpy(a, b), ref, RTOL_F32)
+        assert "gemm_nt_f32" in mm_t.report(), mm_t.report()
+        close(mm.exec_numpy(a, np.ascontiguousarray(b.T)), ref, RTOL_F32)
+        assert "gemm_nt_f32" in mm.report(), mm.report()
+        ad, bd = torch.from_numpy(a).cuda().bfloat16(), torch.from_numpy(b).cuda().bfloat16()
+        ref16 = ad.double() @ bd.double().T
+        got = mm_t.exec_torch(ad, bd)
+        assert "gemm_nt_bf16" in mm_t.report(), mm_t.report()
+        assert float((got.double() - ref16).abs().max()) <= RTOL_BF16 * float(ref16.abs().max())
+        got = mm.exec_torch(ad, bd.T.contiguous())
+        assert float((got.double() - ref16).abs().max()) <= RTOL_BF16 * float(ref16.abs().max())
+    # batched, and an f32 operand that starts 4 bytes into its allocation (rows not 16-byte aligned)
+    ab, bb = rnd((3, 40, 30), 3), rnd((3, 50, 30), 4)
+    bmm = i("bik*bjk~bijk | i:16,j:16 | bjii'j'k") >> i("+bijk~bij | i:16,j:16 | bjii'j'k0")
+    close(bmm.exec_numpy(ab, bb), np.einsum("bik,bjk->bij", ab.astype(np.float64), bb.astype(np.float64)), RTOL_F32)
+    buf = torch.zeros(100 * 64 + 1, device="cuda")
+    x = rnd((100, 64), 5)
+    buf[1:] = torch.from_numpy(x).cuda().reshape(-1)
+    shifted = buf[1:].view(100, 64)
+    got = mm_t.exec_torch(shifted, shifted)
+    assert float((got.double().cpu() - torch.from_numpy(x.astype(np.float64) @ x.astype(np.float64).T)).abs().max()) <= 1e-4 * 64
 
 
 def test_config3_mm_t_through_the_host_f32_abi(torch):
