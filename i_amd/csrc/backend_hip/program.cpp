@@ -349,6 +349,16 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       if (t == DType::F32)
         return ihip::launch_gemm_nt_f32(static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(out), bh,
                                         a[nb], b[nb], k, run.stream, note);
+      // few output tiles under a long k loop: the loop is split over workgroups, partial products in a temporary
+      // (unless the schedule names one of the kernels' own tiles: then that kernel runs as asked)
+      const bool tile_asked = (r.tile_i == 128 && r.tile_j == 128) || (r.tile_i == 256 && r.tile_j == 256);
+      if (const unsigned splits = tile_asked ? 1u : ihip::gemm_nt_bf16_split_k(bh, a[nb], b[nb], k);
+          splits > 1 && (a[nb] * b[nb]) % 4 == 0) {
+        void* partial = nullptr;
+        if (run.alloc(&partial, bh * splits * a[nb] * b[nb] * 4).empty())  // (no room for it: the unsplit kernel)
+          return ihip::launch_gemm_nt_bf16_split_k(pa, pb, out, static_cast<float*>(partial), splits, bh, a[nb], b[nb], k, run.stream,
+                                                   note, out_dt);
+      }
       return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, a[nb], b[nb], k, run.stream, r.tile_i, r.tile_j, note, out_dt);
     }
     case Recognized::GemmNN: {

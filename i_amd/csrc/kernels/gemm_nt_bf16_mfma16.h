@@ -66,7 +66,11 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   constexpr int WLW = WL / NWAVES;
   static_assert(WL % NWAVES == 0 && NWAVES % 2 == 0 && TM >= 2 && TN >= 2, "slab shape");
   char (*smem)[2][SLAB] = reinterpret_cast<char (*)[2][SLAB]>(smem_base);  // [buffer][A, B]
-  const uint32_t batch = blockIdx.y;
+  // (the k loop split over workgroups: blockIdx.y counts (batch, split) pairs)
+  const uint32_t nsplit = (!NN && p.splits > 1) ? p.splits : 1u;
+  const uint32_t batch = blockIdx.y / nsplit, split = blockIdx.y - batch * nsplit;
+  const uint32_t k_first = split * p.k_chunk;                                            // first k of this split
+  const uint32_t kk = nsplit > 1 ? (p.k - k_first < p.k_chunk ? p.k - k_first : p.k_chunk) : p.k;  // its extent
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -75,9 +79,9 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   const uint32_t c16 = lane & 15, g = lane >> 4;
 
   const size_t row_bytes = (size_t)p.k * 2;
-  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
-  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;
-  char* __restrict__ C = reinterpret_cast<char*>(p.c) + (size_t)batch * p.m * p.n * (p.out_bf16 ? 2 : 4);
+  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes + (size_t)k_first * 2;
+  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes + (size_t)k_first * 2;
+  char* __restrict__ C = reinterpret_cast<char*>(p.c) + (size_t)blockIdx.y * p.m * p.n * (p.out_bf16 ? 2 : 4);
   const uint32_t m0 = tm * BT, n0 = tn * BT;
 
   // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
@@ -126,9 +130,9 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
       boff_nn[parity] = (wave * RPWN + lane / CHN) * (uint32_t)brow_bytes + 16 * ch;
     }
   }
-  const uint32_t nslabs = KTAIL ? (p.k + BK - 1) / BK : p.k / BK;
+  const uint32_t nslabs = KTAIL ? (kk + BK - 1) / BK : kk / BK;
   // KTAIL: what exists of the last slab: 16-byte chunks per row (rows of k for an NN slab of B)
-  const uint32_t tail_chunks = (p.k - (nslabs - 1) * BK) / 8;
+  const uint32_t tail_chunks = (kk - (nslabs - 1) * BK) / 8;
   // a transfer of 16 bytes per lane; KTAIL: a lane that has nothing to fetch (`valid` false) clears its slot
   auto move = [&](const void* base, uint32_t voff, uint32_t lds_base, bool valid) {
     if constexpr (KTAIL) {

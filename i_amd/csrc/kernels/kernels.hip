@@ -229,6 +229,25 @@ __device__ __forceinline__ void transpose_body(const TransposeParams& p) {
   for (uint32_t y = y0; y < 64; y += 4)
     if (c0 + y < p.cols && r0 + x < p.rows) dst[(size_t)(c0 + y) * p.rows + r0 + x] = tile[x][y];
 }
+// the partial products of a GEMM whose k loop was split over workgroups, added up in split order
+extern "C" __global__ void __launch_bounds__(256) splitk_reduce(SplitReduceParams p) {
+  const uint64_t quads = p.count / 4, total = (uint64_t)p.batches * quads;
+  for (uint64_t at = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; at < total; at += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t b = at / quads, i = at - b * quads;
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)b * p.splits * p.count) + i;
+    f32x4 sum = src[0];
+    for (uint32_t s = 1; s < p.splits; ++s) sum += src[(size_t)s * quads];
+    if (p.out_bf16) {
+      bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (bf16_t)sum[e];
+      reinterpret_cast<bf16x4*>(p.out)[at] = v;
+    } else {
+      reinterpret_cast<f32x4*>(p.out)[at] = sum;
+    }
+  }
+}
+
 // rows copied into rows of cols_padded elements, the tail zeroed: what gives a product whose contracted extent the
 // matrix-instruction kernels cannot take (k % 8 != 0 in bf16, k % 4 != 0 in f32) operands they can
 template <class T>

@@ -25,6 +25,20 @@ struct GemmParams {
   uint32_t bh, m, n, k;
   uint32_t tiles_m, tiles_n;
   uint32_t out_bf16;  // 0: f32 output, 1: the f32 sums are rounded to bf16 on the way out
+  // The k loop split over workgroups (direct NT kernels only; 0 or 1: not split).  blockIdx.y then counts
+  // (batch, split) pairs; split s contracts k_chunk * s .. + k_chunk (what is left of k for the last one) and
+  // writes its f32 partial products to c[(batch * splits + s)][m][n], a temporary that splitk_reduce adds up.
+  uint32_t splits;
+  uint32_t k_chunk;   // a multiple of 64
+};
+
+// out[b][i] = sum over s < splits of partial[b][s][i], i < count (count a multiple of 4); out f32 or bf16
+struct SplitReduceParams {
+  const float* partial;
+  void* out;
+  uint32_t batches, splits;
+  uint64_t count;
+  uint32_t out_bf16;
 };
 
 struct SoftmaxParams {

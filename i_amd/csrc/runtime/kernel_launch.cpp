@@ -223,6 +223,57 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
 
 // NN product on the direct kernels: 64-wide k slabs (the last one may be partial), 16-byte chunks along n, 32-bit byte
 // offsets inside a slab
+// Tile of a split product: the large tile needs both extents to fill most of it
+static unsigned split_k_tile(size_t m, size_t n) { return m >= 192 && n >= 192 ? 256 : 128; }
+
+unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k) {
+  if (bh == 0 || m == 0 || n == 0 || k % 8 != 0 || std::getenv("ILANG_GEMM_NO_SPLIT")) return 1;
+  const unsigned tile = split_k_tile(m, n);
+  // The split costs a second launch, a temporary and a pass over the partial products: about 15 us of host time
+  // and 10 us on the device.  It pays when the unsplit loop is long (measured: 128 x 16384 x 8192 317 -> 457
+  // TFLOP/s, 64 x 8192 x 8192 108 -> 212, 512 x 512 x 16384 41 -> 164; 256 x 4096 x 4096 203 -> 163, 1024^3 118 -> 58).
+  if (k < (tile == 256 ? 8192u : 4096u)) return 1;
+  const size_t tiles = ((m + tile - 1) / tile) * ((n + tile - 1) / tile) * bh;
+  const size_t fill = tile == 256 ? 256 : 512;  // workgroups the chip holds at once
+  if (4 * tiles > fill) return 1;               // at least a quarter full as it is
+  size_t splits = std::min<size_t>(std::min<size_t>(fill / tiles, k / 512), 32);
+  if (splits < 2 || bh * splits > 65535) return 1;
+  const size_t chunk = (k / splits + 63) / 64 * 64;  // what one split contracts: whole 64-wide slabs
+  return (unsigned)((k + chunk - 1) / chunk);
+}
+
+Err launch_gemm_nt_bf16_split_k(const void* a, const void* b, void* c, float* partial, unsigned splits, size_t bh, size_t m,
+                                size_t n, size_t k, hipStream_t stream, LaunchNote* note, DType out_dtype) {
+  if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
+  if (splits < 2 || bh * splits > 65535 || !fits_u32(m) || !fits_u32(n) || k > (size_t(1) << 22)) return "gemm_nt kernel: bad split";
+  if (!a || !b || !c || !partial) return "gemm_nt kernel: null device pointer";
+  if ((m * n) % 4 != 0) return "gemm_nt kernel: a split product needs m * n to be a multiple of 4";
+  GemmParams p{};
+  p.a = a; p.b = b; p.c = partial;
+  p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
+  p.k_chunk = (uint32_t)(((k + splits - 1) / splits + 63) / 64 * 64);
+  splits = (unsigned)((k + p.k_chunk - 1) / p.k_chunk);  // (rounding the parts up to whole slabs may leave fewer of them)
+  if (splits < 2) return "gemm_nt kernel: bad split";
+  p.splits = splits;
+  const unsigned tile = split_k_tile(m, n);
+  p.tiles_m = (uint32_t)((m + tile - 1) / tile);
+  p.tiles_n = (uint32_t)((n + tile - 1) / tile);
+  const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;
+  if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
+  const bool ktail = k % 64 != 0;  // (only the last split is partial; the others run whole slabs through the same code)
+  const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct") +
+                           (ktail ? "_ktail" : "") + (tile == 256 ? "_w4" : "");
+  if (note) *note = LaunchNote{name + " (k in " + std::to_string(splits) + " parts)", tile, tile};
+  hipFunction_t fn;
+  if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
+  if (Err e = launch(fn, (unsigned)grid, (unsigned)(bh * splits), 1, 256, &p, sizeof(p), stream); !e.empty()) return e;
+  SplitReduceParams r{partial, c, (uint32_t)bh, splits, (uint64_t)m * n, out_dtype == BF16 ? 1u : 0u};
+  if (Err e = builtin_function("splitk_reduce", &fn); !e.empty()) return e;
+  size_t rgrid = (bh * m * n / 4 + 255) / 256;
+  if (rgrid > 65536) rgrid = 65536;
+  return launch(fn, (unsigned)rgrid, 1, 1, 256, &r, sizeof(r), stream);
+}
+
 static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n) {
   if (k == 0 || k % 8 != 0 || n % 8 != 0 || k > (size_t(1) << 22) || n > (size_t(1) << 24) || bh > 65535) return 0;
   if (!fits_u32(m) || !fits_u32(n)) return 0;

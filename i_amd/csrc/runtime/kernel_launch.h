@@ -44,6 +44,14 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
                         DType out_dtype = F32);
 bool gemm_nt_bf16_supported(size_t k);
 
+// The same product with its k loop split over workgroups, for products that have few output tiles and a long k loop
+// (one small extent against two large ones), which would leave most of the chip idle.  gemm_nt_bf16_split_k says
+// into how many parts (1: do not split); the caller provides `partial`, room for bh * splits * m * n floats, which
+// the GEMM kernels fill with the partial products of each split and splitk_reduce adds up into c.
+unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k);
+Err launch_gemm_nt_bf16_split_k(const void* a, const void* b, void* c, float* partial, unsigned splits, size_t bh, size_t m,
+                                size_t n, size_t k, hipStream_t stream, LaunchNote* note = nullptr, DType out_dtype = F32);
+
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
 // Needs k % 8 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,

@@ -281,6 +281,36 @@ def test_products_with_any_contracted_extent_run_on_the_matrix_kernels(torch):
     assert float((got.double().cpu() - torch.from_numpy(x.astype(np.float64) @ x.astype(np.float64).T)).abs().max()) <= 1e-4 * 64
 
 
+def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(torch, monkeypatch):
+    """One small extent against a long contraction leaves most CUs without an output tile: the executor then splits
+    the k loop over workgroups (partial products in a temporary, added up by a second kernel).  Against float64,
+    with whole and partial last slabs, several batches, f32 and bf16 results; ILANG_GEMM_NO_SPLIT=1 gives the
+    unsplit kernel and the same numbers to within the order of the sums."""
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    bmm = i("bik*bjk~bijk | i:16,j:16 | bjii'j'k") >> i("+bijk~bij | i:16,j:16 | bjii'j'k0")
+    for shape_a, shape_b, comp in (((64, 8192), (1000, 8192), mm_t), ((100, 5000), (1000, 5000), mm_t),
+                                   ((300, 16424), (260, 16424), mm_t), ((2, 64, 8192), (2, 512, 8192), bmm)):
+        g = torch.Generator(device="cuda").manual_seed(shape_a[-1])
+        a = (torch.rand(*shape_a, device="cuda", generator=g) * 2 - 1).bfloat16()
+        b = (torch.rand(*shape_b, device="cuda", generator=g) * 2 - 1).bfloat16()
+        ref = a.double() @ b.double().transpose(-1, -2)
+        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        got = comp.exec_torch(a, b)
+        assert "parts)" in comp.report(), comp.report()
+        assert float((got.double() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
+        got16 = comp.exec_torch(a, b, out_dtype=torch.bfloat16)
+        assert float((got16.double() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        plain = comp.exec_torch(a, b)
+        assert "parts)" not in comp.report()
+        assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
+    # a product that fills the chip is left alone
+    monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+    a = torch.randn(2048, 4096, device="cuda").bfloat16()
+    mm_t.exec_torch(a, a)
+    assert "parts)" not in mm_t.report()
+
+
 def test_config3_mm_t_through_the_host_f32_abi(torch):
     """BASELINE configs[2] the way the unchanged reference frontend would run it: host f32 arrays holding
     bf16-representable values through i_exec_into (upload, f32 MFMA kernel, download)."""
