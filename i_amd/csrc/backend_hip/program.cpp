@@ -93,6 +93,13 @@ struct Run {
     return {};
   }
 
+  // A temporary that a launch can do without (the parts of a split loop): with a workspace, which is small and whose
+  // sizing pass only adds up, at most 16 MiB are taken for one, so that what fits unsplit still fits.
+  bool alloc_optional(void** ptr, size_t bytes) {
+    if (workspace && bytes > (size_t(16) << 20)) return false;
+    return alloc(ptr, bytes).empty();
+  }
+
   // Device pointer to f32 data of a buffer some f32 kernel reads.
   ihip::Err read_f32(BufferRef r, void** ptr) {
     if (dtype_of(r) == DType::F32) {
@@ -321,9 +328,21 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
         return e;
       }
+      ihip::AttentionOptions options{r.tile_i, r.tile_j, run.p.attention_f32_scale.load()};
+      // few workgroups under a long key loop (a single head, a few long sequences): the keys of a head in parts
+      // over workgroups, each part's result in a temporary (no room for it: the unsplit kernel)
+      if (const unsigned splits = ihip::attention_kv_splits(bf16 ? ihip::BF16 : ihip::F32, bh, nq, nk, dq, dv, options); splits > 1) {
+        void* partial = nullptr;  // the parts' results, then their row sums' logarithms
+        const size_t rows = bh * splits * nq;
+        if (run.alloc_optional(&partial, rows * dv * 4 + rows * 4)) {
+          options.kv_splits = splits;
+          options.partial_o = static_cast<float*>(partial);
+          options.partial_lse = static_cast<float*>(partial) + rows * dv;
+        }
+      }
       return ihip::launch_attention(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), run.raw_ptr(r.c.buffer), out,
                                     bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream,
-                                    ihip::AttentionOptions{r.tile_i, r.tile_j, run.p.attention_f32_scale.load()}, note);
+                                    options, note);
     }
     case Recognized::GemmNT: {
       const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
@@ -355,7 +374,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       if (const unsigned splits = tile_asked ? 1u : ihip::gemm_nt_bf16_split_k(bh, a[nb], b[nb], k);
           splits > 1 && (a[nb] * b[nb]) % 4 == 0) {
         void* partial = nullptr;
-        if (run.alloc(&partial, bh * splits * a[nb] * b[nb] * 4).empty())  // (no room for it: the unsplit kernel)
+        if (run.alloc_optional(&partial, bh * splits * a[nb] * b[nb] * 4))  // (no room for it: the unsplit kernel)
           return ihip::launch_gemm_nt_bf16_split_k(pa, pb, out, static_cast<float*>(partial), splits, bh, a[nb], b[nb], k, run.stream,
                                                    note, out_dt);
       }

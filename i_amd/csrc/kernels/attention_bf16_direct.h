@@ -93,7 +93,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[2][2][TILE_BYTES];  // [buffer][K, V]
 
   uint32_t head, qt;
-  xcd_map(blockIdx.x, p.nqt, head, qt);
+  xcd_map(blockIdx.x, p.nqt, p.bh, head, qt);
   if (head >= p.bh) return;
 
   const int tid = threadIdx.x;
@@ -106,9 +106,19 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const uint32_t RBG = 2 * d, RBGV = 2 * dv;            // bytes per global row of K, of V (RB when not PADDED)
   const uint32_t chunks = d / 8, chunks_v = dv / 8;     // 16-byte chunks per global row
 
-  const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)head * p.nq * d;
-  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBGV;
+  // The keys of a head split over workgroups (p.kv_splits > 1): `head` then counts (head, part) pairs.  A part runs
+  // the keys key0 .. key0 + nk of its head as if they were all there are and leaves its normalised result in
+  // o[head] (a temporary) and, per query row, the base-2 logarithm of its sum of exponentials in p.lse[head];
+  // attn_kv_merge puts the parts together.
+  uint32_t qhead = head, key0 = 0, nk = p.nk;
+  if (p.kv_splits > 1) {
+    qhead = head / p.kv_splits;
+    key0 = (head - qhead * p.kv_splits) * p.kv_chunk;
+    nk = p.nk - key0 < p.kv_chunk ? p.nk - key0 : p.kv_chunk;
+  }
+  const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)qhead * p.nq * d;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + ((size_t)qhead * p.nk + key0) * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + ((size_t)qhead * p.nk + key0) * RBGV;
 
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).
@@ -164,7 +174,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   float l_run = 0.0f;       // running sum over this half-wave's keys
   float mb_run = 0.0f;      // m_run * scale_log2, kept while the steady-state loop runs
 
-  const uint32_t nfull_tiles = p.nk / BN;  // tiles that lie entirely inside nk
+  const uint32_t nfull_tiles = nk / BN;  // tiles that lie entirely inside nk
   // ---- global -> LDS: this lane's slot in wave-load w is tile row w*RPW + lane/CH, chunk lane%CH
   const uint32_t lrow = lane / CH, lch = lane % CH;
   const uint32_t smem0 = lds_address(&smem[0][0][0]);
@@ -214,11 +224,11 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const uint32_t w = wave + NWAVES * it;
       dma16_chunk(K + (PADDED ? ((size_t)tile * BN + w * RPW) * RBG : (size_t)tile * TILE_BYTES + w * 1024),
                   koff_of(it), smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch_lane ^ ((uint32_t)(KSTRIDE * it) % KMOD), chunks);
-    } else if (tile * BN < p.nk) {
+    } else if (tile * BN < nk) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;
       uint32_t key = tile * BN + row;
-      key = key < p.nk ? key : p.nk - 1;
+      key = key < nk ? key : nk - 1;
       const uint32_t kch = lch ^ ((row / RPB) % KMOD);
       dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch, chunks);
     }
@@ -234,7 +244,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
       const uint32_t kch = lch ^ ((row / RPB) % KMOD);
       const uint32_t vch = lch ^ (4 * ((row / RPB) % VMOD));
       uint32_t key = key0 + row;
-      if constexpr (PARTIAL) key = key < p.nk ? key : p.nk - 1;
+      if constexpr (PARTIAL) key = key < nk ? key : nk - 1;
       if constexpr (decltype(want_k)::value) dma16_chunk(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024, kch, chunks);
       if constexpr (decltype(want_v)::value) dma16_chunk(V, key * RBGV + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024, vch, chunks_v);
     }
@@ -287,7 +297,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const uint32_t key = j * BN + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
-          if (key >= p.nk) s[kt][i] = -INFINITY;
+          if (key >= nk) s[kt][i] = -INFINITY;
         }
     }
     float mx = s[0][0];
@@ -314,7 +324,7 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
         if (masked) {
           // spelled out rather than left to exp(-inf): a zero scale turns the masked score into 0 * inf
           const uint32_t key = j * BN + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
-          if (key >= p.nk) e = 0.0f;
+          if (key >= nk) e = 0.0f;
         }
         pb[kt][i >> 3][i & 7] = (bf16_t)e;
       }
@@ -355,8 +365,8 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
 
   using No = std::integral_constant<bool, false>;
   using Yes = std::integral_constant<bool, true>;
-  const uint32_t ntiles = (p.nk + BN - 1) / BN;
-  const uint32_t nfull = p.nk / BN;  // tiles that lie entirely inside nk
+  const uint32_t ntiles = (nk + BN - 1) / BN;
+  const uint32_t nfull = nk / BN;  // tiles that lie entirely inside nk
 
   // Software pipeline: the scores of tile j+1 are computed (matrix pipe) in the same iteration as the
   // softmax of tile j (vector pipe).  K is therefore consumed one iteration before V: K(j+2) and V(j+1)
@@ -691,7 +701,9 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   }
 
   // ---- epilogue: normalise and store.  Lane (c, h) holds O[q = c][32 t + 8 g + 4 h + e].
-  const float inv = 1.0f / half_sum(l_run);
+  const float row_total = half_sum(l_run);
+  const float inv = 1.0f / row_total;
+  if (p.kv_splits > 1 && qrow < p.nq && h == 0) p.lse[(size_t)head * p.nq + qrow] = m_run * scale_log2 + log2f(row_total);
   if (qrow < p.nq) {
     if (p.out_bf16) {
       bf16_t* O = reinterpret_cast<bf16_t*>(p.o) + ((size_t)head * p.nq + qrow) * dv;

@@ -43,7 +43,7 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[2][2][TILE_BYTES];  // [buffer][K, V]
 
   uint32_t head, qt;
-  xcd_map(blockIdx.x, p.nqt, head, qt);
+  xcd_map(blockIdx.x, p.nqt, p.bh, head, qt);
   if (head >= p.bh) return;
 
   const int tid = threadIdx.x;

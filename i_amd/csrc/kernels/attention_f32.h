@@ -28,7 +28,7 @@ __device__ __forceinline__ void attn_fwd_f32_body(const AttnParams& p) {
   __shared__ __attribute__((aligned(16))) Smem sm;
 
   uint32_t head, qt;
-  xcd_map(blockIdx.x, p.nqt, head, qt);
+  xcd_map(blockIdx.x, p.nqt, p.bh, head, qt);
   if (head >= p.bh) return;
 
   const int tid = threadIdx.x;

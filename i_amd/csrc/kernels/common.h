@@ -65,15 +65,22 @@ __device__ __forceinline__ float load_scale(const float* ptr, float value) {
   return (ptr ? *ptr : 1.0f) * value;
 }
 
-// Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.
-// Map the linear workgroup id so that ids sharing an XCD walk consecutive
-// tiles of one `group` (e.g. one attention head, whose K/V then stay in that
-// XCD's L2).  `per_group` tiles per group; groups are padded to a multiple of 8.
-__device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_t& group, uint32_t& tile) {
-  uint32_t xcd = id & 7u;
-  uint32_t slot = id >> 3;
-  group = (slot / per_group) * 8u + xcd;
-  tile = slot % per_group;
+// Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.  The tiles of all groups in sequence
+// (`per_group` tiles per group, e.g. the query tiles of one attention head after those of the one before) are cut
+// into 8 equal runs, one per XCD: workgroup id (xcd = id % 8, slot = id / 8) takes number xcd * ceil(T / 8) + slot
+// of the sequence.  The workgroups of an XCD thus walk consecutive tiles of one group after the other (a head's K/V
+// stay in that XCD's L2) and every XCD has work whatever the number of groups: a single head is spread over all
+// eight.  Launch with at least 8 * ceil(T / 8) workgroups; one without a tile gets group == groups.
+__device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_t groups, uint32_t& group, uint32_t& tile) {
+  const uint32_t total = groups * per_group, per_xcd = (total + 7u) / 8u;
+  const uint32_t slot = id >> 3, at = (id & 7u) * per_xcd + slot;
+  if (slot >= per_xcd || at >= total) {
+    group = groups;
+    tile = 0;
+    return;
+  }
+  group = at / per_group;
+  tile = at - group * per_group;
 }
 
 // Output tile of a large-tile GEMM workgroup.  The tiles are numbered block by block (blocks of 4 x 8 tiles, the

@@ -248,6 +248,39 @@ extern "C" __global__ void __launch_bounds__(256) splitk_reduce(SplitReduceParam
   }
 }
 
+// the parts of an attention whose keys were split over workgroups, put together: each part's rows are normalised
+// by their own sum of exponentials, whose base-2 logarithm weighs them here (relative to the largest of the row)
+extern "C" __global__ void __launch_bounds__(256) attn_kv_merge(AttnMergeParams p) {
+  const uint32_t quads = p.dv / 4;
+  const uint64_t rows = (uint64_t)p.heads * p.nq, total = rows * quads;
+  for (uint64_t at = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; at < total; at += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t row = at / quads;
+    const uint32_t quad = (uint32_t)(at - row * quads);
+    const uint64_t head = row / p.nq;
+    const uint32_t r = (uint32_t)(row - head * p.nq);
+    const float* lse = p.lse + (size_t)head * p.splits * p.nq + r;
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + ((size_t)head * p.splits * p.nq + r) * p.dv) + quad;
+    float top = lse[0];
+    for (uint32_t s = 1; s < p.splits; ++s) top = fmaxf(top, lse[(size_t)s * p.nq]);
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    float weights = 0.0f;
+    for (uint32_t s = 0; s < p.splits; ++s) {
+      const float w = exp2f(lse[(size_t)s * p.nq] - top);
+      weights += w;
+      sum += w * src[(size_t)s * p.nq * quads];
+    }
+    sum *= 1.0f / weights;
+    if (p.out_bf16) {
+      bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (bf16_t)sum[e];
+      reinterpret_cast<bf16x4*>(p.out)[at] = v;
+    } else {
+      reinterpret_cast<f32x4*>(p.out)[at] = sum;
+    }
+  }
+}
+
 // rows copied into rows of cols_padded elements, the tail zeroed: what gives a product whose contracted extent the
 // matrix-instruction kernels cannot take (k % 8 != 0 in bf16, k % 4 != 0 in f32) operands they can
 template <class T>

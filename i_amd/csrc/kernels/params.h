@@ -16,6 +16,22 @@ struct AttnParams {
   // score scale = scale_value * (scale_ptr ? *scale_ptr : 1), any finite value
   const float* scale_ptr;  // optional rank-0 f32 operand in device memory
   float scale_value;
+  // The keys of a head split over workgroups (direct bf16 kernels only; 0 or 1: not split).  bh then counts
+  // (head, part) pairs: part s attends the keys kv_chunk * s .. + kv_chunk (what is left of nk for the last one)
+  // and writes its normalised f32 result to o[head * kv_splits + s][nq][dv] and log2 of its sum of exponentials
+  // (relative to nothing: reference included) to lse[head * kv_splits + s][nq]; attn_kv_merge combines them.
+  uint32_t kv_splits;
+  uint32_t kv_chunk;  // a multiple of 64
+  float* lse;
+};
+
+// out[b][r][:] = sum_s w_s partial[b * splits + s][r][:],  w_s = 2^lse[b * splits + s][r] / sum_t 2^lse[b * splits + t][r]
+struct AttnMergeParams {
+  const float* partial;  // [heads * splits, nq, dv]
+  const float* lse;      // [heads * splits, nq]
+  void* out;             // [heads, nq, dv] f32 or bf16
+  uint32_t heads, splits, nq, dv;  // dv a multiple of 4
+  uint32_t out_bf16;
 };
 
 struct GemmParams {

@@ -108,6 +108,23 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
   p.scale_ptr = scale_ptr;
   p.scale_value = scale;
+  // the keys of a head in several parts: the direct kernels take (head, part) pairs for heads and write to the
+  // caller's temporaries; attn_kv_merge follows
+  unsigned splits = 1;
+  if (options.kv_splits > 1) {
+    if (!direct || q64 || in_dtype != BF16) return "attention kernel: only the direct bf16 kernels split the keys of a head";
+    if (!options.partial_o || !options.partial_lse) return "attention kernel: a split needs its temporaries";
+    p.kv_chunk = (uint32_t)(((nk + options.kv_splits - 1) / options.kv_splits + 63) / 64 * 64);
+    splits = (unsigned)((nk + p.kv_chunk - 1) / p.kv_chunk);  // (rounding the parts up to whole tiles may leave fewer)
+    if (splits > 1) {
+      if (!fits_u32(bh * splits)) return "attention kernel: extent exceeds 32 bits";
+      p.kv_splits = splits;
+      p.bh = (uint32_t)(bh * splits);
+      p.o = options.partial_o;
+      p.lse = options.partial_lse;
+      p.out_bf16 = 0;
+    }
+  }
 
   std::string name;
   unsigned threads = 2 * bm;  // one query per lane of a half-wave: 32 queries per wave
@@ -139,14 +156,48 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     else name = dmax <= 32 ? "attn_fwd_f32_d32_bn32" : dmax <= 64 ? "attn_fwd_f32_d64_bn32" : "attn_fwd_f32_d128_bn32";
     bn = 32;
   }
-  if (note) *note = LaunchNote{name, bm, bn};
+  if (note) *note = LaunchNote{splits > 1 ? name + " (keys in " + std::to_string(splits) + " parts)" : name, bm, bn};
 
-  const size_t groups = (bh + 7) / 8 * 8;  // heads padded to the XCD count
-  const size_t grid = groups * p.nqt;
+  const size_t grid = (size_t(p.bh) * p.nqt + 7) / 8 * 8;  // the query tiles of all heads in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "attention kernel: grid too large";
   hipFunction_t fn;
   if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, 1, 1, threads, &p, sizeof(p), stream);
+  if (Err e = launch(fn, (unsigned)grid, 1, 1, threads, &p, sizeof(p), stream); !e.empty() || splits == 1) return e;
+  AttnMergeParams m{options.partial_o, options.partial_lse, o, (uint32_t)bh, splits, (uint32_t)nq, (uint32_t)dv, out_dtype == BF16 ? 1u : 0u};
+  if (Err e = builtin_function("attn_kv_merge", &fn); !e.empty()) return e;
+  size_t mgrid = (bh * nq * (dv / 4) + 255) / 256;
+  if (mgrid > 65536) mgrid = 65536;
+  return launch(fn, (unsigned)mgrid, 1, 1, 256, &m, sizeof(m), stream);
+}
+
+// Into how many parts to split the keys of each head (1: do not).  A grid of bh * ceil(nq / 128) workgroups that
+// leaves most of the 256 CUs without one (a single head, a few sequences) finishes sooner when parts of the key
+// loop run side by side: 94 -> 67 us for one head of 8192 x 128, 177 -> 131 us for 16384.  The temporaries and the
+// merge kernel cost the host about 25 us a call, so only key loops of 2^20 elements (8192 keys of 128) and more are
+// split, into parts of at least a quarter of that, and into no more parts than fill the CUs once.  Only where the
+// direct bf16 kernels run (launch_attention's own conditions).
+unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, size_t d, size_t dv, const AttentionOptions& options) {
+  if (in_dtype != BF16 || bh == 0 || nq == 0 || d == 0 || dv == 0) return 1;
+  if (d % 8 != 0 || dv % 8 != 0 || d > 256 || dv > 256) return 1;
+  const size_t dmax = d > dv ? d : dv;
+  if (!(nk * dmax * 2 < (size_t(1) << 32)) || std::getenv("ILANG_ATTN_NO_DIRECT") != nullptr) return 1;
+  if (const char* w = std::getenv("ILANG_ATTN_WAVES"); w && std::atoi(w) == 64) return 1;
+  if (options.query_tile == 512) return 1;  // (may select the 64-queries-per-wave kernel)
+  size_t want;
+  if (const char* f = std::getenv("ILANG_ATTN_KV_SPLITS")) {
+    want = (size_t)std::atoi(f);  // forced (0 or 1: never split), still bounded by whole 64-key tiles below
+  } else {
+    if (nk * dmax < (size_t(1) << 20)) return 1;
+    const size_t bm = options.query_tile == 64 || options.query_tile == 256 ? options.query_tile : 128;
+    const size_t groups = bh * ((nq + bm - 1) / bm);
+    const size_t least = (size_t(1) << 18) / dmax;
+    want = std::min<size_t>(std::min<size_t>(256 / groups, nk / least), 16);
+  }
+  if (want < 2 || nk < 128) return 1;
+  want = std::min<size_t>(want, nk / 64);
+  if (want < 2) return 1;
+  const size_t chunk = ((nk + want - 1) / want + 63) / 64 * 64;
+  return (unsigned)((nk + chunk - 1) / chunk);
 }
 
 bool gemm_nt_bf16_supported(size_t k) { return k > 0 && k % 8 == 0; }

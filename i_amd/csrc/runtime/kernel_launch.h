@@ -27,10 +27,17 @@ struct LaunchNote {
 // d = 64 (64 queries per wave); any other request leaves the choice to the launcher's size heuristic.
 // f32_scale: apply the score scale in f32 to every score, as the reference does, instead of folding it into Q
 // with one more bf16 rounding (direct kernels only; the other kernels always multiply in f32).
+// kv_splits > 1: the keys of each head in that many parts over workgroups (direct bf16 kernels only; ask
+// attention_kv_splits, which also says when it pays: grids that leave most CUs without a workgroup).  The caller
+// provides partial_o, room for bh * kv_splits * nq * dv floats, and partial_lse, for bh * kv_splits * nq.
 struct AttentionOptions {
   size_t query_tile = 0, key_tile = 0;
   bool f32_scale = false;
+  unsigned kv_splits = 0;
+  float* partial_o = nullptr;
+  float* partial_lse = nullptr;
 };
+unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, size_t d, size_t dv, const AttentionOptions& options = {});
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options = {}, LaunchNote* note = nullptr);

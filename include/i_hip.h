@@ -81,7 +81,8 @@ int i_exec_into_device_noalloc(const i_program* program,
  * (f32), 0 < d,dv <= 256 and multiples of 8 (bf16).  bf16 runs the direct-to-LDS kernels
  * at every such head size (d = dv = 64, 128, 256 exactly, the others with zero-padded LDS
  * rows); f32 with d and dv multiples of 4, the larger from 36 to 128, and 16-byte aligned
- * operands runs the f32 kernel of the same design.
+ * operands runs the f32 kernel of the same design.  One kernel launch, no temporaries: the key loop
+ * of a head is split over workgroups (few heads, long loops) only by programs run through i_exec*.
  */
 int i_hip_attention(const void* q, const void* k, const void* v, void* o,
                     int in_dtype, int out_dtype,

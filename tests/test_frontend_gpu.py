@@ -451,6 +451,48 @@ def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
     assert (c256 - ref).abs().max() <= 1e-3 * ref.abs().max()
 
 
+def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroups(torch, monkeypatch):
+    """A single head (or a few sequences) leaves most CUs without a query tile: the executor then runs parts of the
+    key loop side by side (each part's normalised rows and the logarithm of its row sums in a temporary) and a
+    second kernel merges them.  ILANG_ATTN_KV_SPLITS forces a number of parts, so that small operands reach the
+    path: every direct bf16 kernel family (d = 128 without a reference, d = 64 with prescaled scores, padded head
+    sizes, d = 256), ragged query and key counts, f32 and bf16 results, against the oracle and against the
+    unsplit kernel; then the launcher's own choice for one long head."""
+    comp = flash(prefix="b", scaled=True)
+    for BH, NQ, NK, D, DV in ((1, 300, 4100, 128, 128), (2, 200, 2500, 72, 40), (1, 130, 3000, 256, 256), (3, 257, 2111, 64, 64)):
+        q, k, v = (oracle.to_bf16_f32(rnd(shape, s)) for s, shape in ((1, (BH, NQ, D)), (2, (BH, NK, D)), (3, (BH, NK, DV))))
+        scale = np.float32(1.0 / np.sqrt(D))
+        qd, kd, vd = (torch.from_numpy(a).cuda().bfloat16() for a in (q, k, v))
+        sd = torch.tensor(scale, device="cuda")
+        rows = np.r_[0:8, NQ - 8:NQ]
+        ref = oracle.attention_tiled(q[:, rows], k, v, scale)
+        monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "1")
+        plain = comp.exec_torch(qd, kd, sd, vd)
+        assert "keys in" not in comp.report()
+        for parts in ("2", "3", "16"):
+            monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", parts)
+            got = comp.exec_torch(qd, kd, sd, vd)
+            assert "(keys in " in comp.report(), comp.report()
+            close(got.cpu().numpy()[:, rows], ref, RTOL_BF16)
+            assert float((got - plain).abs().max()) <= 2e-3
+            got16 = comp.exec_torch(qd, kd, sd, vd, out_dtype=torch.bfloat16)
+            close(got16.float().cpu().numpy()[:, rows], ref, RTOL_BF16)
+    monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
+    # the launcher's choice: one head of 8192 x 128 in 4 parts; short key loops and grids that fill the chip as they are
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = (torch.randn(1, 8192, 128, device="cuda", generator=g).bfloat16() for _ in range(3))
+    sd = torch.tensor(128 ** -0.5, device="cuda")
+    got = comp.exec_torch(q, k, sd, v)
+    assert "(keys in 4 parts)" in comp.report(), comp.report()
+    ref = torch.softmax((q[:, :64].double() @ k.double().transpose(1, 2)) * 128 ** -0.5, -1) @ v.double()
+    assert float((got[:, :64].double() - ref).abs().max()) <= 2e-3
+    comp.exec_torch(q[:, :2048], k[:, :2048], sd, v[:, :2048])
+    assert "keys in" not in comp.report()
+    q, k, v = (torch.randn(64, 8192, 128, device="cuda", generator=g).bfloat16() for _ in range(3))
+    comp.exec_torch(q, k, sd, v)
+    assert "keys in" not in comp.report()
+
+
 def test_config4_full_size_properties(torch):
     B, H, N, D = 8, 32, 4096, 128
     g = torch.Generator(device="cuda").manual_seed(1)

@@ -87,6 +87,27 @@ def test_transposed_operand_and_generated_kernels(torch):
         assert float((c2.double() - ref).abs().max() / ref.abs().max()) <= 1e-4
 
 
+def test_split_loops_keep_their_partial_results_in_the_workspace(torch, monkeypatch):
+    """A product whose k loop and an attention whose key loop are split over workgroups: the parts' results are
+    temporaries like any other (up to 16 MiB of the fixed array; above that the unsplit kernel runs)."""
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    for m, n, k in ((64, 1000, 8192), (40, 300, 4104)):
+        print("case split product", (m, n, k), flush=True)
+        both(mm_t, [randn(torch, (m, k), 7, torch.bfloat16), randn(torch, (n, k), 8, torch.bfloat16)], torch)
+        assert "parts)" in mm_t.report(), mm_t.report()
+    s = "i:16,j:16"
+    attention = ((i(f"ik*jk~ijk | {s} | jii'j'k") >> i(f"+ijk~ij | {s} | jii'j'k0"))
+                 >> ((I & i(f">ij~i | {s} | ji0i'j'")) >> i(f"ij-i~ij | {s} | ji01i'j'")) >> i(f"^ij~ij | {s} | ji0i'j'")
+                 >> ((I & i(f"+ij~i | {s} | ji0i'j'")) >> i(f"ij/i~ij | {s} | ji01i'j'"))
+                 >> (i(f"ij*jk~ikj | {s} | ji0i'kj'") >> i(f"+ikj~ik | {s} | jii'kj'0")))
+    monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "3")
+    for nq, nk, d in ((300, 2500, 128), (70, 1000, 64)):
+        print("case split attention", (nq, nk, d), flush=True)
+        q, k, v = (randn(torch, shape, seed, torch.bfloat16) for seed, shape in ((9, (nq, d)), (10, (nk, d)), (11, (nk, d))))
+        both(attention, [q * d ** -0.25, k * d ** -0.25, v], torch)
+        assert "(keys in 3 parts)" in attention.report(), attention.report()
+
+
 def test_operands_beyond_the_workspace_are_refused_before_anything_runs(torch):
     comp = softmax_naive()
     x = randn(torch, (8192, 4096), 5)  # two 128 MiB intermediates
