@@ -5,6 +5,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <map>
+#include <memory>
+#include <mutex>
 #include <set>
 #include <sstream>
 
@@ -30,6 +33,39 @@ std::string ref_name(BufferRef r) {
   return (r.kind == BufferRef::Input ? "in" : r.kind == BufferRef::Intermediate ? "s" : "out") + std::to_string(r.id);
 }
 
+// The temporaries of the calls on one stream of one device share a block that the library keeps: kernels on a
+// stream run one after the other, so a call may overwrite what the call before it on the same stream left there,
+// and after the first call of a program no call allocates or frees anything (a stream-ordered allocation and its
+// release cost the host 20 to 45 us a call here, several times the rest of the executor).  A call carves its
+// temporaries off the block; what does not fit is allocated as before, and at its end the call replaces the block
+// by one large enough for all it needed, up to ILANG_HIP_ARENA_MB (default 256; 0: no such block) per stream,
+// held until the process ends.  A stream under capture, a second call in flight on the same stream from another
+// thread, and the emulated runtime (whose allocations are guarded one by one) take the allocating path.
+struct Arena {
+  void* base = nullptr;
+  size_t capacity = 0;
+  std::mutex busy;  // held by the call that carves from it
+};
+
+Arena* arena_of(hipStream_t stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, std::unique_ptr<Arena>> arenas;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  auto& arena = arenas[{device, stream}];
+  if (!arena) arena = std::make_unique<Arena>();
+  return arena.get();
+}
+
+size_t arena_limit() {
+  static const size_t limit = [] {
+    const char* mb = std::getenv("ILANG_HIP_ARENA_MB");
+    return (mb ? (size_t)std::max(0, std::atoi(mb)) : size_t(256)) << 20;
+  }();
+  return limit;
+}
+
 // Everything the executor needs to know about one invocation.
 struct Run {
   Program& p;
@@ -43,6 +79,8 @@ struct Run {
   std::map<size_t, void*> output_f32;        // f32 staging for bf16 outputs
   Workspace* workspace = nullptr;            // when set, temporaries are carved out of it and nothing is allocated
   std::vector<std::string> notes;            // one line per dispatched kernel: what ran, on which tile
+  Arena* arena = nullptr;                    // when set (and locked by this call), temporaries come off it while they fit
+  size_t arena_used = 0, arena_needed = 0;
 
   size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
   size_t extent(const Extent<size_t>& e) const {
@@ -88,15 +126,24 @@ struct Run {
       workspace->used += step;
       return {};
     }
-    if (ihip::Err e = ihip::check(hipMallocAsync(ptr, bytes, stream), "hipMallocAsync"); !e.empty()) return e;
+    if (arena) {
+      const size_t step = (bytes + 255) / 256 * 256;
+      arena_needed += step;
+      if (step <= arena->capacity - arena_used) {
+        *ptr = static_cast<char*>(arena->base) + arena_used;
+        arena_used += step;
+        return {};
+      }
+    }
+    if (ihip::Err e = ihip::temp_alloc(ptr, bytes, stream); !e.empty()) return e;
     temps.push_back(*ptr);
     return {};
   }
 
   // A temporary that a launch can do without (the parts of a split loop): with a workspace, which is small and whose
-  // sizing pass only adds up, at most 16 MiB are taken for one, so that what fits unsplit still fits.
+  // sizing pass only adds up, at most 20 MiB are taken for one, so that most of what fits unsplit still fits.
   bool alloc_optional(void** ptr, size_t bytes) {
-    if (workspace && bytes > (size_t(16) << 20)) return false;
+    if (workspace && bytes > (size_t(20) << 20)) return false;
     return alloc(ptr, bytes).empty();
   }
 
@@ -771,9 +818,30 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
     }
   }
 
-  ihip::Err err;
+  std::unique_lock<std::mutex> arena_lock;
+  if (!workspace && arena_limit() > 0 && !ihip::runtime_is_emulated()) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+      (void)hipGetLastError();
+    } else if (capture == hipStreamCaptureStatusNone) {
+      if (Arena* arena = arena_of(stream)) {
+        arena_lock = std::unique_lock<std::mutex>(arena->busy, std::try_to_lock);
+        if (arena_lock.owns_lock()) run.arena = arena;
+      }
+    }
+  }
   auto finish = [&](ihip::Err e) {
     for (auto it = run.temps.rbegin(); it != run.temps.rend(); ++it) (void)hipFreeAsync(*it, stream);
+    if (run.arena && run.arena_needed > run.arena->capacity && run.arena_needed <= arena_limit()) {
+      // the next call on this stream finds room for everything this one needed
+      const size_t bytes = (run.arena_needed + (size_t(1) << 20) - 1) >> 20 << 20;
+      void* bigger = nullptr;
+      if (ihip::temp_alloc(&bigger, bytes, stream).empty()) {
+        if (run.arena->base) (void)hipFreeAsync(run.arena->base, stream);
+        run.arena->base = bigger;
+        run.arena->capacity = bytes;
+      }
+    }
     return e;
   };
   for (const Step& step : plan.exec) {

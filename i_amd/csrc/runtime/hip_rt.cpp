@@ -24,6 +24,8 @@ namespace {
 struct DeviceModule {
   hipModule_t mod = nullptr;
   std::map<std::string, hipFunction_t> fns;
+  bool pool_tried = false;
+  hipMemPool_t pool = nullptr;  // stream-ordered temporaries (temp_alloc)
 };
 
 thread_local int g_dry_run = 0;
@@ -106,6 +108,41 @@ bool runtime_is_emulated() {
 
 DryRun::DryRun() { ++g_dry_run; }
 DryRun::~DryRun() { --g_dry_run; }
+
+// Stream-ordered temporaries come from a pool of the library's own, one per device, that keeps up to 1 GiB of
+// freed memory instead of handing it back to the system when the stream runs dry, which is what makes a
+// temporary cost tens of microseconds from the device's default pool.  The default pool and its settings, which
+// belong to the application, are left alone; without a pool of its own (the emulated runtime, a failed creation)
+// the library allocates from the default one.
+Err temp_alloc(void** p, size_t bytes, hipStream_t stream) {
+  *p = nullptr;
+  if (bytes == 0) bytes = 4;
+  hipMemPool_t pool = nullptr;
+  if (!runtime_is_emulated()) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    int dev = 0;
+    if (Err e = check(hipGetDevice(&dev), "hipGetDevice"); !e.empty()) return e;
+    DeviceModule& dm = g_builtin[dev];
+    if (!dm.pool_tried) {
+      dm.pool_tried = true;
+      hipMemPoolProps props{};
+      props.allocType = hipMemAllocationTypePinned;
+      props.handleTypes = hipMemHandleTypeNone;
+      props.location.type = hipMemLocationTypeDevice;
+      props.location.id = dev;
+      uint64_t keep = uint64_t(1) << 30;
+      if (hipMemPoolCreate(&dm.pool, &props) != hipSuccess ||
+          hipMemPoolSetAttribute(dm.pool, hipMemPoolAttrReleaseThreshold, &keep) != hipSuccess) {
+        if (dm.pool) (void)hipMemPoolDestroy(dm.pool);
+        dm.pool = nullptr;
+        (void)hipGetLastError();
+      }
+    }
+    pool = dm.pool;
+  }
+  if (pool) return check(hipMallocFromPoolAsync(p, bytes, pool, stream), "hipMallocFromPoolAsync");
+  return check(hipMallocAsync(p, bytes, stream), "hipMallocAsync");
+}
 
 Err dev_alloc(void** p, size_t bytes) {
   *p = nullptr;

@@ -42,6 +42,8 @@ struct DryRun {
 };
 
 Err dev_alloc(void** p, size_t bytes);
+// a temporary that hipFreeAsync(p, stream) gives back, from the library's own pool of the current device
+Err temp_alloc(void** p, size_t bytes, hipStream_t stream);
 void dev_free(void* p);
 Err h2d(void* dst, const void* src, size_t bytes, hipStream_t stream);
 Err d2h(void* dst, const void* src, size_t bytes, hipStream_t stream);

@@ -171,11 +171,13 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 }
 
 // Into how many parts to split the keys of each head (1: do not).  A grid of bh * ceil(nq / 128) workgroups that
-// leaves most of the 256 CUs without one (a single head, a few sequences) finishes sooner when parts of the key
-// loop run side by side: 94 -> 67 us for one head of 8192 x 128, 177 -> 131 us for 16384.  The temporaries and the
-// merge kernel cost the host about 25 us a call, so only key loops of 2^20 elements (8192 keys of 128) and more are
-// split, into parts of at least a quarter of that, and into no more parts than fill the CUs once.  Only where the
-// direct bf16 kernels run (launch_attention's own conditions).
+// leaves most of the 256 CUs without one (a single head, a few sequences, a few queries against many keys)
+// finishes sooner when parts of the key loop run side by side: as many parts as fill the CUs once, of at least 512
+// keys each, at most 32, and only for loops of 2048 keys and more (below that the second launch takes what the
+// split gains).  Measured, enqueued back to back, d = 128: one head of 8192 x 8192 92 -> 46 us (4 parts), of
+// 4096 x 4096 48 -> 27, 128 queries x 8192 keys 91 -> 23 (16 parts), 8 heads of 128 x 16384 176 -> 32; from 256
+// workgroups on nothing is gained (16 heads of 4096: 127 -> 146 us with 2 parts).  Only where the direct bf16
+// kernels run (launch_attention's own conditions).
 unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, size_t d, size_t dv, const AttentionOptions& options) {
   if (in_dtype != BF16 || bh == 0 || nq == 0 || d == 0 || dv == 0) return 1;
   if (d % 8 != 0 || dv % 8 != 0 || d > 256 || dv > 256) return 1;
@@ -187,11 +189,10 @@ unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, si
   if (const char* f = std::getenv("ILANG_ATTN_KV_SPLITS")) {
     want = (size_t)std::atoi(f);  // forced (0 or 1: never split), still bounded by whole 64-key tiles below
   } else {
-    if (nk * dmax < (size_t(1) << 20)) return 1;
     const size_t bm = options.query_tile == 64 || options.query_tile == 256 ? options.query_tile : 128;
     const size_t groups = bh * ((nq + bm - 1) / bm);
-    const size_t least = (size_t(1) << 18) / dmax;
-    want = std::min<size_t>(std::min<size_t>(256 / groups, nk / least), 16);
+    if (nk < 2048 || nk < 32 * groups) return 1;  // (half the CUs busy: two parts pay from 4096 keys on)
+    want = std::min<size_t>(std::min<size_t>(256 / groups, nk / 512), 32);
   }
   if (want < 2 || nk < 128) return 1;
   want = std::min<size_t>(want, nk / 64);

@@ -41,7 +41,9 @@ typedef struct {
 /*
  * i_exec_into for operands that already live on the GPU (reference host form:
  * core/src/lib.rs:200-225).  Enqueues the whole program on `stream` and returns
- * without waiting; temporaries are stream-ordered allocations.  Rank-0 operands
+ * without waiting; temporaries are stream-ordered (a block per stream that the
+ * library keeps from call to call, at most ILANG_HIP_ARENA_MB, default 256, and
+ * stream-ordered allocations beyond it).  Rank-0 operands
  * (scalars) must be f32.  bf16 operands select the bf16-in / f32-accumulate
  * kernels where a kernel has one and are widened on the device otherwise;
  * each output is written in its own dtype.  Output shapes, when given

@@ -96,6 +96,16 @@ hipError_t hipMalloc(void** p, size_t bytes) { return guarded_alloc(p, bytes); }
 hipError_t hipFree(void* p) { return guarded_free(p); }
 hipError_t hipMallocAsync(void** p, size_t bytes, hipStream_t) { return guarded_alloc(p, bytes); }
 hipError_t hipFreeAsync(void* p, hipStream_t) { return guarded_free(p); }
+// (the library asks ilang_hip_runtime_is_emulated first and creates no pool here; these only satisfy the linker)
+hipError_t hipGetLastError() { return hipSuccess; }
+hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* status) {
+  *status = hipStreamCaptureStatusNone;
+  return hipSuccess;
+}
+hipError_t hipMemPoolCreate(hipMemPool_t*, const hipMemPoolProps*) { return hipErrorNotSupported; }
+hipError_t hipMemPoolDestroy(hipMemPool_t) { return hipErrorNotSupported; }
+hipError_t hipMemPoolSetAttribute(hipMemPool_t, hipMemPoolAttr, void*) { return hipErrorNotSupported; }
+hipError_t hipMallocFromPoolAsync(void** p, size_t bytes, hipMemPool_t, hipStream_t) { return guarded_alloc(p, bytes); }
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t) {
   std::memcpy(dst, src, bytes);
   return hipSuccess;

@@ -478,7 +478,8 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
             got16 = comp.exec_torch(qd, kd, sd, vd, out_dtype=torch.bfloat16)
             close(got16.float().cpu().numpy()[:, rows], ref, RTOL_BF16)
     monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
-    # the launcher's choice: one head of 8192 x 128 in 4 parts; short key loops and grids that fill the chip as they are
+    # the launcher's choice: one head of 8192 x 128 in 4 parts (64 query tiles for 256 CUs); short key loops and grids that fill
+    # the chip as they are
     g = torch.Generator(device="cuda").manual_seed(5)
     q, k, v = (torch.randn(1, 8192, 128, device="cuda", generator=g).bfloat16() for _ in range(3))
     sd = torch.tensor(128 ** -0.5, device="cuda")
@@ -486,11 +487,37 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
     assert "(keys in 4 parts)" in comp.report(), comp.report()
     ref = torch.softmax((q[:, :64].double() @ k.double().transpose(1, 2)) * 128 ** -0.5, -1) @ v.double()
     assert float((got[:, :64].double() - ref).abs().max()) <= 2e-3
-    comp.exec_torch(q[:, :2048], k[:, :2048], sd, v[:, :2048])
+    comp.exec_torch(q[:, :1024].contiguous(), k[:, :1024].contiguous(), sd, v[:, :1024].contiguous())
     assert "keys in" not in comp.report()
+    comp.exec_torch(q[:, :100].contiguous(), k, sd, v)  # a few queries against many keys: 16 parts of 512
+    assert "(keys in 16 parts)" in comp.report(), comp.report()
     q, k, v = (torch.randn(64, 8192, 128, device="cuda", generator=g).bfloat16() for _ in range(3))
     comp.exec_torch(q, k, sd, v)
     assert "keys in" not in comp.report()
+
+
+def test_temporaries_are_kept_from_call_to_call_on_a_stream(torch):
+    """Calls enqueued back to back on one stream carve their temporaries (here the two [rows, cols] intermediates
+    of the naive softmax) from one block that the library keeps and replaces when a call needs more: operands that
+    grow and shrink from call to call without a synchronisation in between, then two streams interleaved, each
+    with a block of its own."""
+    comp = softmax_naive()
+    g = torch.Generator(device="cuda").manual_seed(11)
+    xs = [torch.randn(*shape, device="cuda", generator=g) for shape in ((64, 100), (2048, 3000), (300, 77), (2048, 3000), (5, 9), (4096, 2000))]
+    torch.cuda.synchronize()
+    outs = [comp.exec_torch(x) for x in xs]
+    torch.cuda.synchronize()
+    for x, y in zip(xs, outs):
+        assert float((y.double() - torch.softmax(x.double(), -1)).abs().max()) <= 1e-6
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    results = []
+    for rep in range(3):
+        for stream, x in zip(streams, (xs[1], xs[5])):
+            with torch.cuda.stream(stream):
+                results.append((x, comp.exec_torch(x)))
+    torch.cuda.synchronize()
+    for x, y in results:
+        assert float((y.double() - torch.softmax(x.double(), -1)).abs().max()) <= 1e-6
 
 
 def test_config4_full_size_properties(torch):

@@ -89,7 +89,7 @@ def test_transposed_operand_and_generated_kernels(torch):
 
 def test_split_loops_keep_their_partial_results_in_the_workspace(torch, monkeypatch):
     """A product whose k loop and an attention whose key loop are split over workgroups: the parts' results are
-    temporaries like any other (up to 16 MiB of the fixed array; above that the unsplit kernel runs)."""
+    temporaries like any other (up to 20 MiB of the fixed array; above that the unsplit kernel runs)."""
     mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     for m, n, k in ((64, 1000, 8192), (40, 300, 4104)):
         print("case split product", (m, n, k), flush=True)
