@@ -90,11 +90,14 @@ __device__ __forceinline__ void xcd_map(uint32_t id, uint32_t per_group, uint32_
 // of an XCD thus work on consecutive tiles (at most 1024 rows of A and 2048 of B at a time, shared through the
 // XCD's L2), and the XCDs get the same number of tiles to within one: with whole blocks dealt out to XCDs
 // instead, 22 x 22 tiles (18 blocks) cost three rounds of workgroups where two suffice.
-// Launch with 8 * ceil(T / 8) workgroups per batch.  Returns false for a workgroup that has no tile.
-__device__ __forceinline__ bool gemm_tile_of_workgroup(uint32_t id, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm,
-                                                       uint32_t& tn) {
+// Launch with 8 * ceil(T / 8) workgroups per batch (so that id % 8 is the XCD in every batch).  `batch` rotates
+// which XCD takes which run: when T is not a multiple of 8 the short and the empty runs then fall on a different
+// XCD in every batch (one tile per batch: batch b runs on XCD (8 - b) % 8 instead of all of them on XCD 0).
+// Returns false for a workgroup that has no tile.
+__device__ __forceinline__ bool gemm_tile_of_workgroup(uint32_t id, uint32_t batch, uint32_t tiles_m, uint32_t tiles_n,
+                                                       uint32_t& tm, uint32_t& tn) {
   const uint32_t total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-  const uint32_t slot = id >> 3, at = (id & 7u) * per_xcd + slot;
+  const uint32_t slot = id >> 3, at = ((id + batch) & 7u) * per_xcd + slot;
   if (slot >= per_xcd || at >= total) return false;
   const uint32_t column = tiles_m * 8;            // tiles in a full block column
   const uint32_t bn = at / column, in_column = at - bn * column;

@@ -35,7 +35,7 @@ __device__ __forceinline__ void gemm_nt_bf16_body(const GemmParams& p) {
   const uint32_t batch = lin / (((tiles + 7) / 8) * 8);
   lin -= batch * (((tiles + 7) / 8) * 8);
   const uint32_t per_xcd = (tiles + 7) / 8;
-  const uint32_t tile = (lin & 7u) * per_xcd + (lin >> 3);
+  const uint32_t tile = ((lin + batch) & 7u) * per_xcd + (lin >> 3);  // (the runs rotate over the XCDs from batch to batch)
   if (tile >= tiles) return;
   const uint32_t tn = tile / p.tiles_m;
   const uint32_t tm = tile % p.tiles_m;

@@ -344,7 +344,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
   __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
   // ---- tile of this workgroup
   uint32_t tm, tn;
-  if (!gemm_tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
+  if (!gemm_tile_of_workgroup(blockIdx.x, blockIdx.y, p.tiles_m, p.tiles_n, tm, tn)) return;
   if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN, KTAIL>(p, smem, tm, tn);
   else gemm_nt_mfma16_tile<BT, WM, WN, true, NN, KTAIL>(p, smem, tm, tn);
 }

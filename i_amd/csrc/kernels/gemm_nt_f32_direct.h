@@ -52,7 +52,7 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
 
   // ---- tile of this workgroup
   uint32_t tm, tn;
-  if (!gemm_tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
+  if (!gemm_tile_of_workgroup(blockIdx.x, blockIdx.y, p.tiles_m, p.tiles_n, tm, tn)) return;
   const uint32_t batch = blockIdx.y;
 
   const int tid = threadIdx.x;

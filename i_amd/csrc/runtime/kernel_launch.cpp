@@ -273,23 +273,45 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   return launch(fn, (unsigned)grid, 1, 1, 256, &p, sizeof(p), stream);
 }
 
-// NN product on the direct kernels: 64-wide k slabs (the last one may be partial), 16-byte chunks along n, 32-bit byte
-// offsets inside a slab
 // Tile of a split product: the large tile needs both extents to fill most of it
 static unsigned split_k_tile(size_t m, size_t n) { return m >= 192 && n >= 192 ? 256 : 128; }
 
 unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k) {
   if (bh == 0 || m == 0 || n == 0 || k % 8 != 0 || std::getenv("ILANG_GEMM_NO_SPLIT")) return 1;
   const unsigned tile = split_k_tile(m, n);
-  // The split costs a second launch, a temporary and a pass over the partial products: about 15 us of host time
-  // and 10 us on the device.  It pays when the unsplit loop is long (measured: 128 x 16384 x 8192 317 -> 457
-  // TFLOP/s, 64 x 8192 x 8192 108 -> 212, 512 x 512 x 16384 41 -> 164; 256 x 4096 x 4096 203 -> 163, 1024^3 118 -> 58).
-  if (k < (tile == 256 ? 8192u : 4096u)) return 1;
-  const size_t tiles = ((m + tile - 1) / tile) * ((n + tile - 1) / tile) * bh;
-  const size_t fill = tile == 256 ? 256 : 512;  // workgroups the chip holds at once
-  if (4 * tiles > fill) return 1;               // at least a quarter full as it is
-  size_t splits = std::min<size_t>(std::min<size_t>(fill / tiles, k / 512), 32);
-  if (splits < 2 || bh * splits > 65535) return 1;
+  if (const char* forced = std::getenv("ILANG_GEMM_SPLITS")) {  // (tests and measurements: that many parts, whole slabs each)
+    const size_t want = std::min<size_t>((size_t)std::max(0, std::atoi(forced)), k / 64);
+    if (want < 2 || bh * want > 65535) return 1;
+    const size_t chunk = (k / want + 63) / 64 * 64;
+    return (unsigned)((k + chunk - 1) / chunk);
+  }
+  // A model of the time in us, fitted to products from 32 x 4096 x 4096 to 2048 x 2048 x 8192 enqueued back to back
+  // (it picks the measured best number of parts, or one within a few per cent of it, on 14 of 16 of them): a
+  // workgroup spends 0.7 us per 64-wide slab on a 128 x 128 tile (1.1 us when two share a CU), 1.3 us on a
+  // 256 x 256 tile, plus two slabs' worth before and after its loop; the chip holds 512 / 256 of them at a time;
+  // the second launch costs 4 us and the pass over the partial products runs at 3 TB/s.  Examples (unsplit ->
+  // split): 64 x 8192 x 8192 79 -> 30 us in 8 parts, 512 x 512 x 4096 52 -> 27 in 8, 256 x 4096 x 4096 41 -> 29
+  // in 8, 256 x 256 x 65536 812 -> 73 in 32; left whole: 1024^3 (10 us; 25 in 2 parts), 2048^3 (28; 40).
+  if (k > (size_t(1) << 22)) return 1;
+  const size_t slabs = (k + 63) / 64;
+  const size_t t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh, t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
+  auto time_of = [](unsigned tile_, size_t workgroups, size_t slabs_) {
+    const double rounds = (double)((workgroups + (tile_ == 128 ? 511 : 255)) / (tile_ == 128 ? 512 : 256));
+    return rounds * (double)(slabs_ + 2) * (tile_ == 128 ? (workgroups <= 256 ? 0.7 : 1.1) : 1.3);
+  };
+  double best = time_of(128, t128, slabs);
+  if (t256 >= 64) best = std::min(best, time_of(256, t256, slabs));
+  best *= 0.85;  // a split has to gain at least 15 %
+  const size_t tiles = tile == 256 ? t256 : t128;
+  size_t splits = 1;
+  for (size_t s = 2; s <= 32 && k / s >= (s == 32 ? 2048u : 512u) && bh * s <= 65535; s *= 2) {
+    const double t = time_of(tile, tiles * s, (slabs + s - 1) / s) + 4.0 + (double)(bh * s * m * n * 4) / 3e6;
+    if (t < best) {
+      best = t;
+      splits = s;
+    }
+  }
+  if (splits < 2) return 1;
   const size_t chunk = (k / splits + 63) / 64 * 64;  // what one split contracts: whole 64-wide slabs
   return (unsigned)((k + chunk - 1) / chunk);
 }
