@@ -477,6 +477,26 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
             assert float((got - plain).abs().max()) <= 2e-3
             got16 = comp.exec_torch(qd, kd, sd, vd, out_dtype=torch.bfloat16)
             close(got16.float().cpu().numpy()[:, rows], ref, RTOL_BF16)
+    # parts whose scores lie far apart: the first third of the keys adds `offset` nats to the scores of rows 0..95, which
+    # sends that part of the d = 128 kernel (exponentials without a reference) through its second pass with the
+    # running max, and the merge then weighs parts whose sums differ by 2^115 or 2^-430
+    plain_flash = flash(prefix="b")
+    monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "3")
+    for d in (128, 64):
+        for offset in (80.0, -300.0):
+            nq, nk = 300, 1500
+            q = oracle.to_bf16_f32(rnd((2, nq, d), 1) * 0.5)
+            k = oracle.to_bf16_f32(rnd((2, nk, d), 2) * 0.5)
+            q[:, :, 0] = 0.0
+            q[:, :96, 0] = 1.0
+            k[:, :, 0] = 0.0
+            k[:, :nk // 3, 0] = oracle.to_bf16_f32(np.full((2, nk // 3), offset, np.float32))
+            v = oracle.to_bf16_f32(rnd((2, nk, d), 3))
+            ref = oracle.attention_tiled(q, k, v)
+            assert np.isfinite(ref).all()
+            got = plain_flash.exec_torch(*(torch.from_numpy(a).cuda().bfloat16() for a in (q, k, v)))
+            assert "(keys in 3 parts)" in plain_flash.report(), plain_flash.report()
+            close(got.cpu().numpy(), ref, RTOL_BF16)
     monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
     # the launcher's choice: one head of 8192 x 128 in 4 parts (64 query tiles for 256 CUs); short key loops and grids that fill
     # the chip as they are
