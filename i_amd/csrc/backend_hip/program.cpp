@@ -39,8 +39,9 @@ std::string ref_name(BufferRef r) {
 // release cost the host 20 to 45 us a call here, several times the rest of the executor).  A call carves its
 // temporaries off the block; what does not fit is allocated as before, and at its end the call replaces the block
 // by one large enough for all it needed, up to ILANG_HIP_ARENA_MB (default 256; 0: no such block) per stream,
-// held until the process ends.  A stream under capture, a second call in flight on the same stream from another
-// thread, and the emulated runtime (whose allocations are guarded one by one) take the allocating path.
+// held until the process ends, for the first 16 streams that run programs.  A stream under capture, a second
+// call in flight on the same stream from another thread, and the emulated runtime (whose allocations are guarded
+// one by one) take the allocating path.
 struct Arena {
   void* base = nullptr;
   size_t capacity = 0;
@@ -53,9 +54,10 @@ Arena* arena_of(hipStream_t stream) {
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(mu);
-  auto& arena = arenas[{device, stream}];
-  if (!arena) arena = std::make_unique<Arena>();
-  return arena.get();
+  const auto found = arenas.find({device, stream});
+  if (found != arenas.end()) return found->second.get();
+  if (arenas.size() >= 16) return nullptr;  // (an application with a stream per request: the later streams allocate)
+  return (arenas[{device, stream}] = std::make_unique<Arena>()).get();
 }
 
 size_t arena_limit() {
