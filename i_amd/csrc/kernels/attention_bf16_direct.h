@@ -107,18 +107,18 @@ __device__ __forceinline__ void attn_fwd_bf16_direct_body(const AttnParams& p) {
   const uint32_t chunks = d / 8, chunks_v = dv / 8;     // 16-byte chunks per global row
 
   // The keys of a head split over workgroups (p.kv_splits > 1): `head` then counts (head, part) pairs.  A part runs
-  // the keys key0 .. key0 + nk of its head as if they were all there are and leaves its normalised result in
+  // the keys first_key .. first_key + nk of its head as if they were all there are and leaves its normalised result in
   // o[head] (a temporary) and, per query row, the base-2 logarithm of its sum of exponentials in p.lse[head];
   // attn_kv_merge puts the parts together.
-  uint32_t qhead = head, key0 = 0, nk = p.nk;
+  uint32_t qhead = head, first_key = 0, nk = p.nk;
   if (p.kv_splits > 1) {
     qhead = head / p.kv_splits;
-    key0 = (head - qhead * p.kv_splits) * p.kv_chunk;
-    nk = p.nk - key0 < p.kv_chunk ? p.nk - key0 : p.kv_chunk;
+    first_key = (head - qhead * p.kv_splits) * p.kv_chunk;
+    nk = p.nk - first_key < p.kv_chunk ? p.nk - first_key : p.kv_chunk;
   }
   const bf16_t* __restrict__ Q = reinterpret_cast<const bf16_t*>(p.q) + (size_t)qhead * p.nq * d;
-  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + ((size_t)qhead * p.nk + key0) * RBG;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + ((size_t)qhead * p.nk + key0) * RBGV;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + ((size_t)qhead * p.nk + first_key) * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + ((size_t)qhead * p.nk + first_key) * RBGV;
 
   // A negative scale is folded into Q (sign flip is exact), so the running max
   // can be tracked on the raw scores: max_j(s_j * scale) == scale * max_j(s_j).

@@ -69,9 +69,18 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   const uint32_t RBG = 4 * d, RBGV = 4 * dv;            // bytes per global row of K, of V (RB when not PADDED)
   const uint32_t chunks = d / 4, chunks_v = dv / 4;     // 16-byte chunks per global row
 
-  const float* __restrict__ Q = reinterpret_cast<const float*>(p.q) + (size_t)head * p.nq * d;
-  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + (size_t)head * p.nk * RBG;
-  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + (size_t)head * p.nk * RBGV;
+  // The keys of a head split over workgroups (p.kv_splits > 1), as in the bf16 kernels: `head` counts (head, part)
+  // pairs, a part runs the keys first_key .. first_key + nk of its head and leaves its normalised result in o[head] (a
+  // temporary) and log2 of its row sums of exponentials in p.lse[head] for attn_kv_merge.
+  uint32_t qhead = head, first_key = 0, nk = p.nk;
+  if (p.kv_splits > 1) {
+    qhead = head / p.kv_splits;
+    first_key = (head - qhead * p.kv_splits) * p.kv_chunk;
+    nk = p.nk - first_key < p.kv_chunk ? p.nk - first_key : p.kv_chunk;
+  }
+  const float* __restrict__ Q = reinterpret_cast<const float*>(p.q) + (size_t)qhead * p.nq * d;
+  const char* __restrict__ K = reinterpret_cast<const char*>(p.k) + ((size_t)qhead * p.nk + first_key) * RBG;
+  const char* __restrict__ V = reinterpret_cast<const char*>(p.v) + ((size_t)qhead * p.nk + first_key) * RBGV;
 
   const float scale_raw = load_scale(p.scale_ptr, p.scale_value);
   const float qsign = scale_raw < 0.0f ? -1.0f : 1.0f;  // negative scale folded into Q (exact)
@@ -79,7 +88,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
 
   // ---- global -> LDS: this lane's slot in wave-load w is tile row w*RPW + lane/CH, chunk lane%CH; rows past nk
   // re-read the last row (their scores are masked)
-  const uint32_t ntiles = (p.nk + BN - 1) / BN;
+  const uint32_t ntiles = (nk + BN - 1) / BN;
   const uint32_t lrow = lane / CH, lch = lane % CH;
   const uint32_t smem0 = lds_address(&smem[0][0][0]);
   auto request_tile = [&](uint32_t tile, int buf) {
@@ -88,7 +97,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       const uint32_t w = wave + NWAVES * it;
       const uint32_t row = w * RPW + lrow;  // row within the tile
       uint32_t key = tile * BN + row;
-      key = key < p.nk ? key : p.nk - 1;
+      key = key < nk ? key : nk - 1;
       const uint32_t kch = lch ^ (row % 16), vch = lch ^ (8 * ((row >> 2) & 1));
       if (!PADDED || kch < chunks) dma16(K, key * RBG + 16 * kch, smem0 + (2 * buf + 0) * TILE_BYTES + w * 1024);
       if (!PADDED || vch < chunks_v) dma16(V, key * RBGV + 16 * vch, smem0 + (2 * buf + 1) * TILE_BYTES + w * 1024);
@@ -151,12 +160,12 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[g][e], s, 0, 0, 0);
     }
 
-    const bool masked = key0 + BN > p.nk;
+    const bool masked = key0 + BN > nk;
     if (masked) {  // tail guard: keys past nk do not take part in the max
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const uint32_t key = key0 + 8 * (i >> 2) + 4 * h + (i & 3);
-        if (key >= p.nk) s[i] = -INFINITY;
+        if (key >= nk) s[i] = -INFINITY;
       }
     }
     float mx = s[0];
@@ -175,7 +184,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
       if (masked) {
         // spelled out rather than left to exp(-inf): a zero scale turns the masked score into 0 * inf
         const uint32_t key = key0 + 8 * (i >> 2) + 4 * h + (i & 3);
-        if (key >= p.nk) e = 0.0f;
+        if (key >= nk) e = 0.0f;
       }
       s[i] = e;
       psum += e;
@@ -206,6 +215,7 @@ __device__ __forceinline__ void attn_fwd_f32_direct_body(const AttnParams& p) {
   // ---- epilogue: normalise and store.  Lane (c, h) holds O[q = c][32 t + 8 g + 4 h + e].
   const float l_tot = l_run + xhalf(l_run);
   const float inv = 1.0f / l_tot;
+  if (p.kv_splits > 1 && qrow < p.nq && h == 0) p.lse[(size_t)head * p.nq + qrow] = m_run * scale_log2 + log2f(l_tot);
   if (qrow < p.nq) {
     float* O = reinterpret_cast<float*>(p.o) + ((size_t)head * p.nq + qrow) * dv;
 #pragma unroll

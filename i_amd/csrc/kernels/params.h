@@ -16,7 +16,7 @@ struct AttnParams {
   // score scale = scale_value * (scale_ptr ? *scale_ptr : 1), any finite value
   const float* scale_ptr;  // optional rank-0 f32 operand in device memory
   float scale_value;
-  // The keys of a head split over workgroups (direct bf16 kernels only; 0 or 1: not split).  bh then counts
+  // The keys of a head split over workgroups (the direct kernels, bf16 and f32; 0 or 1: not split).  bh then counts
   // (head, part) pairs: part s attends the keys kv_chunk * s .. + kv_chunk (what is left of nk for the last one)
   // and writes its normalised f32 result to o[head * kv_splits + s][nq][dv] and log2 of its sum of exponentials
   // (relative to nothing: reference included) to lse[head * kv_splits + s][nq]; attn_kv_merge combines them.

@@ -101,6 +101,13 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     }
     if (q64) { bm = 512; bn = 32; }
   }
+  // f32: the direct-to-LDS kernel for d, dv multiples of 4 up to 128, the larger above 32 (16-byte aligned operands,
+  // 32-bit byte offsets inside a head; up to 32 the register-staged kernel with 32-column tiles is the faster one), the
+  // register-staged kernel with guarded columns otherwise (and under ILANG_ATTN_NO_DIRECT=1)
+  auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  const bool f32_direct = in_dtype == F32 && d % 4 == 0 && dv % 4 == 0 && dmax > 32 && dmax <= 128 &&
+                          nk * dmax * 4 < (size_t(1) << 32) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) &&
+                          std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o;
   p.bh = (uint32_t)bh; p.nq = (uint32_t)nq; p.nk = (uint32_t)nk; p.d = (uint32_t)d; p.dv = (uint32_t)dv;
@@ -109,10 +116,10 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.scale_ptr = scale_ptr;
   p.scale_value = scale;
   // the keys of a head in several parts: the direct kernels take (head, part) pairs for heads and write to the
-  // caller's temporaries; attn_kv_merge follows
+  // caller's temporaries; attn_kv_merge follows.  (A request that the kernel chosen above cannot honour, the
+  // register-staged ones and the 64-queries-per-wave kernel, is ignored: the result is the same.)
   unsigned splits = 1;
-  if (options.kv_splits > 1) {
-    if (!direct || q64 || in_dtype != BF16) return "attention kernel: only the direct bf16 kernels split the keys of a head";
+  if (options.kv_splits > 1 && ((in_dtype == BF16 && direct && !q64) || f32_direct)) {
     if (!options.partial_o || !options.partial_lse) return "attention kernel: a split needs its temporaries";
     p.kv_chunk = (uint32_t)(((nk + options.kv_splits - 1) / options.kv_splits + 63) / 64 * 64);
     splits = (unsigned)((nk + p.kv_chunk - 1) / p.kv_chunk);  // (rounding the parts up to whole tiles may leave fewer)
@@ -141,13 +148,6 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
   } else {
-    // f32: the direct-to-LDS kernel for d, dv multiples of 4 up to 128, the larger above 32 (16-byte aligned operands,
-    // 32-bit byte offsets inside a head; up to 32 the register-staged kernel with 32-column tiles is the faster one), the
-    // register-staged kernel with guarded columns otherwise (and under ILANG_ATTN_NO_DIRECT=1)
-    auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
-    const bool f32_direct = d % 4 == 0 && dv % 4 == 0 && dmax > 32 && dmax <= 128 && nk * dmax * 4 < (size_t(1) << 32) &&
-                            aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) &&
-                            std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
     if (f32_direct) {
       // (head sizes other than d == dv in {64, 128}: the same kernel with its LDS rows padded to 64 or 128 columns)
       name = dmax <= 64 ? "attn_fwd_f32_d64_bn32_direct" : "attn_fwd_f32_d128_bn32_direct";
@@ -176,23 +176,30 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 // keys each, at most 32, and only for loops of 2048 keys and more (below that the second launch takes what the
 // split gains).  Measured, enqueued back to back, d = 128: one head of 8192 x 8192 92 -> 46 us (4 parts), of
 // 4096 x 4096 48 -> 27, 128 queries x 8192 keys 91 -> 23 (16 parts), 8 heads of 128 x 16384 176 -> 32; from 256
-// workgroups on nothing is gained (16 heads of 4096: 127 -> 146 us with 2 parts).  Only where the direct bf16
-// kernels run (launch_attention's own conditions).
+// workgroups on nothing is gained (16 heads of 4096: 127 -> 146 us with 2 parts).  An f32 workgroup spends four times
+// as long on half the keys, so f32 loops are split from 256 keys on, into parts of at least 64: the reference's
+// demo, one head of 512 x 64, 45 -> 16 us in 8 parts; 2 heads of 128 queries x 8192 keys of 128, 1136 -> 64 in 32.  Only where the direct kernels run (launch_attention's own
+// conditions).
 unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, size_t d, size_t dv, const AttentionOptions& options) {
-  if (in_dtype != BF16 || bh == 0 || nq == 0 || d == 0 || dv == 0) return 1;
-  if (d % 8 != 0 || dv % 8 != 0 || d > 256 || dv > 256) return 1;
+  if (bh == 0 || nq == 0 || d == 0 || dv == 0 || std::getenv("ILANG_ATTN_NO_DIRECT") != nullptr) return 1;
   const size_t dmax = d > dv ? d : dv;
-  if (!(nk * dmax * 2 < (size_t(1) << 32)) || std::getenv("ILANG_ATTN_NO_DIRECT") != nullptr) return 1;
-  if (const char* w = std::getenv("ILANG_ATTN_WAVES"); w && std::atoi(w) == 64) return 1;
-  if (options.query_tile == 512) return 1;  // (may select the 64-queries-per-wave kernel)
+  if (in_dtype == BF16) {
+    if (d % 8 != 0 || dv % 8 != 0 || d > 256 || dv > 256 || !(nk * dmax * 2 < (size_t(1) << 32))) return 1;
+    if (const char* w = std::getenv("ILANG_ATTN_WAVES"); w && std::atoi(w) == 64) return 1;
+    if (options.query_tile == 512) return 1;  // (may select the 64-queries-per-wave kernel)
+  } else if (d % 4 != 0 || dv % 4 != 0 || dmax <= 32 || dmax > 128 || !(nk * dmax * 4 < (size_t(1) << 32))) {
+    return 1;  // (f32: the direct kernel's head sizes; operands it cannot take for their alignment run unsplit)
+  }
+  // an f32 workgroup takes about 2.8 us per 32 keys (a bf16 one 0.7 us per 64): much shorter loops are worth parts
+  const size_t least_loop = in_dtype == BF16 ? 2048 : 256, least_part = in_dtype == BF16 ? 512 : 64;
   size_t want;
   if (const char* f = std::getenv("ILANG_ATTN_KV_SPLITS")) {
     want = (size_t)std::atoi(f);  // forced (0 or 1: never split), still bounded by whole 64-key tiles below
   } else {
-    const size_t bm = options.query_tile == 64 || options.query_tile == 256 ? options.query_tile : 128;
+    const size_t bm = in_dtype == BF16 && (options.query_tile == 64 || options.query_tile == 256) ? options.query_tile : 128;
     const size_t groups = bh * ((nq + bm - 1) / bm);
-    if (nk < 2048 || nk < 32 * groups) return 1;  // (half the CUs busy: two parts pay from 4096 keys on)
-    want = std::min<size_t>(std::min<size_t>(256 / groups, nk / 512), 32);
+    if (nk < least_loop || nk < least_loop / 64 * groups) return 1;  // (half the CUs busy: two parts pay from twice the least loop on)
+    want = std::min<size_t>(std::min<size_t>(256 / groups, nk / least_part), 32);
   }
   if (want < 2 || nk < 128) return 1;
   want = std::min<size_t>(want, nk / 64);

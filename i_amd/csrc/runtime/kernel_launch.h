@@ -27,7 +27,7 @@ struct LaunchNote {
 // d = 64 (64 queries per wave); any other request leaves the choice to the launcher's size heuristic.
 // f32_scale: apply the score scale in f32 to every score, as the reference does, instead of folding it into Q
 // with one more bf16 rounding (direct kernels only; the other kernels always multiply in f32).
-// kv_splits > 1: the keys of each head in that many parts over workgroups (direct bf16 kernels only; ask
+// kv_splits > 1: the keys of each head in that many parts over workgroups (the direct kernels, bf16 and f32; ask
 // attention_kv_splits, which also says when it pays: grids that leave most CUs without a workgroup).  The caller
 // provides partial_o, room for bh * kv_splits * nq * dv floats, and partial_lse, for bh * kv_splits * nq.
 struct AttentionOptions {

@@ -497,7 +497,21 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
             got = plain_flash.exec_torch(*(torch.from_numpy(a).cuda().bfloat16() for a in (q, k, v)))
             assert "(keys in 3 parts)" in plain_flash.report(), plain_flash.report()
             close(got.cpu().numpy(), ref, RTOL_BF16)
+    # f32 operands (the f32 direct kernel, plain and with padded rows), to the f32 bar
+    for BH, NQ, NK, D in ((1, 300, 1000, 96), (2, 130, 777, 64), (1, 64, 2100, 128)):
+        q, k, v = (rnd(shape, s) for s, shape in ((1, (BH, NQ, D)), (2, (BH, NK, D)), (3, (BH, NK, D))))
+        scale = np.float32(1.0 / np.sqrt(D))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        got = comp.exec_torch(*(torch.from_numpy(a).cuda() for a in (q, k)), torch.tensor(scale, device="cuda"), torch.from_numpy(v).cuda())
+        assert "_f32_" in comp.report() and "(keys in 3 parts)" in comp.report(), comp.report()
+        close(got.cpu().numpy(), ref, RTOL_F32)
     monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
+    # the reference's demo (one f32 head of 512 x 64, 4 workgroups as it is): 8 parts of 64 keys
+    q, k, v = (np.random.default_rng(s).uniform(-1, 1, (512, 64)).astype(np.float32) for s in (1, 2, 3))
+    demo = flash()
+    got = demo.exec_torch(*(torch.from_numpy(a).cuda() for a in (q, k, v)))
+    assert "(keys in 8 parts)" in demo.report(), demo.report()
+    close(got.cpu().numpy(), oracle.attention_tiled(q, k, v), RTOL_F32)
     # the launcher's choice: one head of 8192 x 128 in 4 parts (64 query tiles for 256 CUs); short key loops and grids that fill
     # the chip as they are
     g = torch.Generator(device="cuda").manual_seed(5)
