@@ -14,6 +14,7 @@ device pointer to ``i_exec_into_device`` and never leave the GPU.
 import array
 import ctypes
 import numbers
+import sys
 
 from . import _native as nat
 
@@ -75,13 +76,16 @@ class _Operand:
 
     def __init__(self, address, extents, dtype, device, anchor):
         self.address = address              # integer address of the first element (0 for an empty operand is fine)
-        self.extents = tuple(int(n) for n in extents)
+        self.extents = tuple(extents) if type(extents).__name__ == "Size" else tuple(int(n) for n in extents)
         self.dtype = dtype                  # nat.F32 or nat.BF16
         self.device = device                # None: host memory; otherwise the torch device the address belongs to
         self.anchor = anchor                # whatever must stay alive while the address is in use
 
 
 def _torch_like(x):
+    torch = sys.modules.get("torch")
+    if torch is not None and isinstance(x, torch.Tensor):
+        return True
     return all(hasattr(x, name) for name in ("data_ptr", "device", "is_contiguous", "dtype"))
 
 
@@ -151,6 +155,14 @@ def _pack(operands, on_device):
             records.append(_CTensor(ctypes.cast(op.address, _f32p), dims, len(op.extents)))
     kind = _CDeviceTensor if on_device else _CTensor
     return (kind * max(len(records), 1))(*records), keep
+
+
+def _current_stream(torch, device):
+    """The raw handle of torch's current stream on `device` (the device is current when this is called)."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        return raw(torch.cuda.current_device() if device.index is None else device.index)
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _placement(operands, what):
@@ -382,9 +394,11 @@ class Component:
             import torch
 
             entry = core.i_exec_into_device_noalloc if static_workspace else core.i_exec_into_device
-            with torch.cuda.device(device):
-                stream = torch.cuda.current_stream().cuda_stream
-                nat.check(entry(program, in_records, len(operands), out_records, len(targets), stream))
+            if device.index is None or device.index == torch.cuda.current_device():
+                nat.check(entry(program, in_records, len(operands), out_records, len(targets), _current_stream(torch, device)))
+            else:
+                with torch.cuda.device(device):
+                    nat.check(entry(program, in_records, len(operands), out_records, len(targets), _current_stream(torch, device)))
         del keep_in, keep_out
 
 
