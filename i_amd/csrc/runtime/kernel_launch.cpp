@@ -238,16 +238,16 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   // Direct global -> LDS kernels (64-wide k slabs, 32-bit byte offsets inside a tile's rows):
   //   256 x 256 tiles  long k loops on grids that fill at least half of the CUs (its prologue and its
   //                    unoverlapped store only pay off there)
-  //   128 x 128 tiles  problems with too few 256-tiles, two workgroups per CU
+  //   128 x 128 tiles  everything else, two workgroups per CU (down to one tile and one slab it is the faster
+  //                    128-tile kernel: 4.3 against 5.9 us at 128 x 128 x 64, 9.4 against 17.0 at 128 x 128 x 1024)
   // (k that is no multiple of 64: their _ktail forms, the last slab partial)
-  // and the register-staged 128 x 128 kernel for everything else (k % 8 == 0, short k, tiny grids).
+  // and the register-staged 128 x 128 kernel beyond their offset ranges (k > 2^22, more than 65535 batches).
   // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; ILANG_GEMM_DIRECT=256 | 128 | 0
   // forces a kernel so that tests can reach each of them at small sizes (1 is read as 256).
   {
     const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
-    unsigned tile = 0;  // 0: register-staged kernel
+    unsigned tile = 128;  // (0: register-staged kernel)
     if (k >= 512 && t256 >= 64) tile = pick_direct_tile(t256, t128);
-    else if (k >= 256 && t128 >= 64) tile = 128;
     if (tile_m == 256 && tile_n == 256) tile = 256;
     if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
     if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
