@@ -211,6 +211,12 @@ bool product_extent_usable(DType t, size_t k) {
 }
 
 // Returns true when kernel k can run on its hand-written form with these operands.
+// The arithmetic of a product: bf16 operands on the bf16 kernels; an f32 operand (say the probabilities of the naive
+// attention, an f32 intermediate, against bf16 values) makes it an f32 product, the other operand widened first.
+DType product_dtype(const Run& run, const Recognized& r) {
+  return run.dtype_of(r.a.buffer) == DType::BF16 && run.dtype_of(r.b.buffer) == DType::BF16 ? DType::BF16 : DType::F32;
+}
+
 bool hand_usable(const Run& run, const Recognized& r) {
   // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
   if (const char* v = std::getenv("ILANG_HIP_GENERATED_ONLY"))
@@ -230,19 +236,11 @@ bool hand_usable(const Run& run, const Recognized& r) {
       for (size_t d = 0; d + 2 < q.size(); ++d) bh *= q[d];
       return attention_in_parts_usable(t, bh, q[q.size() - 2], k[k.size() - 2], q.back(), v.back());
     }
-    case Recognized::GemmNT: {
-      const DType t = run.dtype_of(r.a.buffer);
-      if (run.dtype_of(r.b.buffer) != t) return false;
-      const auto a = rows_cols(r.a);
-      if (a.size() < 2) return false;
-      return product_extent_usable(t, a.back());
-    }
+    case Recognized::GemmNT:
     case Recognized::GemmNN: {
-      const DType t = run.dtype_of(r.a.buffer);
-      if (run.dtype_of(r.b.buffer) != t) return false;
       const auto a = rows_cols(r.a);
       if (a.size() < 2) return false;
-      return product_extent_usable(t, a.back());
+      return product_extent_usable(product_dtype(run, r), a.back());
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
@@ -282,7 +280,7 @@ std::string describe_launch(const ihip::LaunchNote& note, const Recognized& r) {
 
 // A product of bf16 operands whose result is a bf16 program output: the GEMM kernels write it themselves.
 bool bf16_result_in_place(const Run& run, const Recognized& r) {
-  return run.dtype_of(r.a.buffer) == DType::BF16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16;
+  return product_dtype(run, r) == DType::BF16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16;
 }
 
 ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
@@ -348,6 +346,21 @@ ihip::Err padded_operands(Run& run, DType t, const void** a, size_t rows_a, cons
   return {};
 }
 
+// The operands of a product in its arithmetic type: as they are, or widened to f32 where the other one is f32.
+ihip::Err product_operands(Run& run, const Recognized& r, DType t, const void** a, const void** b) {
+  if (t == DType::BF16) {
+    *a = run.raw_ptr(r.a.buffer);
+    *b = run.raw_ptr(r.b.buffer);
+    return {};
+  }
+  void *pa = nullptr, *pb = nullptr;
+  if (ihip::Err e = run.read_f32(r.a.buffer, &pa); !e.empty()) return e;
+  if (ihip::Err e = run.read_f32(r.b.buffer, &pb); !e.empty()) return e;
+  *a = pa;
+  *b = pb;
+  return {};
+}
+
 ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* note) {
   switch (r.kind) {
     case Recognized::Attention: {
@@ -410,8 +423,9 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
         return e;
       }
-      const DType t = run.dtype_of(r.a.buffer);
-      const void *pa = run.raw_ptr(r.a.buffer), *pb = run.raw_ptr(r.b.buffer);
+      const DType t = product_dtype(run, r);
+      const void *pa = nullptr, *pb = nullptr;
+      if (ihip::Err e = product_operands(run, r, t, &pa, &pb); !e.empty()) return e;
       size_t k = a[nb + 1];
       if (ihip::Err e = padded_operands(run, t, &pa, bh * a[nb], &pb, bh * b[nb], &k); !e.empty()) return e;
       if (t == DType::F32)
@@ -441,7 +455,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       }
       const size_t m = a[nb], k = a[nb + 1], n = b[nb + 1];
       if (b[nb] != k) return "gemm operands disagree on the contracted extent";
-      const bool f32 = run.dtype_of(r.a.buffer) == DType::F32;
+      const bool f32 = product_dtype(run, r) == DType::F32;
       void* out = nullptr;
       ihip::DType out_dt = ihip::F32;
       if (bf16_result_in_place(run, r)) {
@@ -450,14 +464,15 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
         return e;
       }
+      const void *pa = nullptr, *pb_rows = nullptr;
+      if (ihip::Err e = product_operands(run, r, f32 ? DType::F32 : DType::BF16, &pa, &pb_rows); !e.empty()) return e;
       if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k))  // the direct kernels read a row-major right operand themselves
-        return ihip::launch_gemm_nn_bf16(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), out, bh, m, n, k, run.stream,
-                                         r.tile_i, r.tile_j, note, out_dt);
+        return ihip::launch_gemm_nn_bf16(pa, pb_rows, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note, out_dt);
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
       if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;
-      if (ihip::Err e = ihip::launch_transpose(run.raw_ptr(r.b.buffer), bt, bh, k, n, elem, run.stream); !e.empty()) return e;
-      const void *pa = run.raw_ptr(r.a.buffer), *pb = bt;
+      if (ihip::Err e = ihip::launch_transpose(pb_rows, bt, bh, k, n, elem, run.stream); !e.empty()) return e;
+      const void* pb = bt;
       size_t kp = k;
       if (ihip::Err e = padded_operands(run, f32 ? DType::F32 : DType::BF16, &pa, bh * m, &pb, bh * n, &kp); !e.empty()) return e;
       if (f32)

@@ -414,6 +414,17 @@ def test_naive_attention_uses_both_gemm_forms(torch):
     code = comp._code()
     assert "transposed right operand" in code and "row-major right operand" in code
     assert np.allclose(comp.exec_numpy(q, k, v), oracle.np_attention64(q, k, v), rtol=3e-4, atol=5e-5)
+    # bf16 operands: S = Q K^T on the bf16 kernel; the probabilities are an f32 intermediate, so P V is an f32 product
+    # with V widened on the device (not a generated kernel), sums in f32 as the emitted C has them
+    for n, d in ((96, 64), (300, 72), (1000, 128)):
+        q, k, v = (oracle.to_bf16_f32(rnd((n, d), s) * 0.5) for s in (1, 2, 3))
+        qd, kd, vd = (torch.from_numpy(a).cuda().bfloat16() for a in (q, k, v))
+        got = comp.exec_torch(qd, kd, vd)
+        lines = comp.report().splitlines()
+        assert lines[0].startswith("f0: gemm_nt_bf16") and "gemm_nt_f32" in lines[-1], comp.report()
+        close(got.cpu().numpy(), oracle.np_attention64(q, k, v), 3e-4)
+        got16 = comp.exec_torch(qd, kd, vd, out_dtype=torch.bfloat16)
+        close(got16.float().cpu().numpy(), oracle.np_attention64(q, k, v), 1e-2)
 
 
 # ------------------------------------------------------------------ BASELINE configs 4 and 5 (bf16 in, f32 accumulate)
