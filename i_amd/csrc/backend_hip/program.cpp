@@ -283,6 +283,17 @@ bool bf16_result_in_place(const Run& run, const Recognized& r) {
   return product_dtype(run, r) == DType::BF16 && r.out.kind == BufferRef::Output && run.outputs[r.out.id].dtype == DType::BF16;
 }
 
+// An f32 product through the executor: with few output tiles under a long k loop, the loop in parts over
+// workgroups, the partial products in a temporary (no room for it: the unsplit kernel).
+ihip::Err launch_product_f32(Run& run, const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
+                             ihip::LaunchNote* note) {
+  void* partial = nullptr;
+  unsigned splits = ihip::gemm_nt_f32_split_k(bh, m, n, k);
+  if (splits > 1 && ((m * n) % 4 != 0 || !run.alloc_optional(&partial, bh * splits * m * n * 4))) splits = 1;
+  return ihip::launch_gemm_nt_f32(static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(c), bh, m, n, k,
+                                  run.stream, note, static_cast<float*>(partial), splits);
+}
+
 ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
                              const float* scale_ptr, ihip::LaunchNote* note) {
   void* out = nullptr;
@@ -318,10 +329,7 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
     void* vt = nullptr;
     if (ihip::Err e = run.alloc(&vt, bh * dv * nk * 4); !e.empty()) return e;
     if (ihip::Err e = ihip::launch_transpose(v, vt, bh, nk, dv, 4, run.stream); !e.empty()) return e;
-    if (ihip::Err e = ihip::launch_gemm_nt_f32(s, static_cast<const float*>(vt), static_cast<float*>(out), bh, nq, dv, nk,
-                                               run.stream, &last);
-        !e.empty())
-      return e;
+    if (ihip::Err e = launch_product_f32(run, s, vt, out, bh, nq, dv, nk, &last); !e.empty()) return e;
   }
   if (note) *note = ihip::LaunchNote{"attention in three kernels (head size beyond the fused kernels): " + first.kernel + ", " + middle.kernel + ", " + last.kernel, 0, 0};
   return {};
@@ -428,9 +436,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       if (ihip::Err e = product_operands(run, r, t, &pa, &pb); !e.empty()) return e;
       size_t k = a[nb + 1];
       if (ihip::Err e = padded_operands(run, t, &pa, bh * a[nb], &pb, bh * b[nb], &k); !e.empty()) return e;
-      if (t == DType::F32)
-        return ihip::launch_gemm_nt_f32(static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(out), bh,
-                                        a[nb], b[nb], k, run.stream, note);
+      if (t == DType::F32) return launch_product_f32(run, pa, pb, out, bh, a[nb], b[nb], k, note);
       // few output tiles under a long k loop: the loop is split over workgroups, partial products in a temporary
       // (unless the schedule names one of the kernels' own tiles: then that kernel runs as asked)
       const bool tile_asked = (r.tile_i == 128 && r.tile_j == 128) || (r.tile_i == 256 && r.tile_j == 256);
@@ -475,9 +481,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       const void* pb = bt;
       size_t kp = k;
       if (ihip::Err e = padded_operands(run, f32 ? DType::F32 : DType::BF16, &pa, bh * m, &pb, bh * n, &kp); !e.empty()) return e;
-      if (f32)
-        return ihip::launch_gemm_nt_f32(static_cast<const float*>(pa), static_cast<const float*>(pb), static_cast<float*>(out), bh,
-                                        m, n, kp, run.stream, note);
+      if (f32) return launch_product_f32(run, pa, pb, out, bh, m, n, kp, note);
       return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, m, n, kp, run.stream, r.tile_i, r.tile_j, note, out_dt);
     }
     case Recognized::RowSoftmax:

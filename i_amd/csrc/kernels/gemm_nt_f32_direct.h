@@ -53,7 +53,12 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   // ---- tile of this workgroup
   uint32_t tm, tn;
   if (!gemm_tile_of_workgroup(blockIdx.x, blockIdx.y, p.tiles_m, p.tiles_n, tm, tn)) return;
-  const uint32_t batch = blockIdx.y;
+  // (the k loop split over workgroups, as in the bf16 kernels: blockIdx.y counts (batch, split) pairs, split s
+  // contracts k_chunk * s .. + kk and writes its partial products to c[blockIdx.y])
+  const uint32_t nsplit = p.splits > 1 ? p.splits : 1;
+  const uint32_t batch = blockIdx.y / nsplit, split = blockIdx.y - batch * nsplit;
+  const uint32_t k_first = split * p.k_chunk;
+  const uint32_t kk = nsplit > 1 ? (p.k - k_first < p.k_chunk ? p.k - k_first : p.k_chunk) : p.k;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -62,9 +67,9 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   const int c = lane & 31, h = lane >> 5;
 
   const size_t row_bytes = (size_t)p.k * ELEM;
-  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes;
-  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes;  // n k = k n elements
-  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)batch * p.m * p.n;
+  const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes + (size_t)k_first * ELEM;
+  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes + (size_t)k_first * ELEM;
+  float* __restrict__ C = reinterpret_cast<float*>(p.c) + (size_t)blockIdx.y * p.m * p.n;
   const uint32_t m0 = tm * BMT, n0 = tn * BNT;
 
   // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
@@ -86,8 +91,8 @@ __device__ __forceinline__ void gemm_nt_f32_direct_body(const GemmParams& p) {
   const char* a_tile = A + (size_t)m0 * row_bytes;
   const char* b_tile = B + (size_t)n0 * row_bytes;
   const size_t b_slab_step = (size_t)RB;  // bytes from one k slab of B to the next
-  const uint32_t nslabs = KTAIL ? (p.k + BK - 1) / BK : p.k / BK;
-  const uint32_t tail_chunks = (p.k - (nslabs - 1) * BK) / 4;  // KTAIL: 16-byte chunks per row of the last slab
+  const uint32_t nslabs = KTAIL ? (kk + BK - 1) / BK : kk / BK;
+  const uint32_t tail_chunks = (kk - (nslabs - 1) * BK) / 4;  // KTAIL: 16-byte chunks per row of the last slab
   // one transfer of 16 bytes per lane of slab s; KTAIL: nothing to fetch for this lane: its slot is cleared
   auto move = [&](const void* base, uint32_t voff, uint32_t lds_base, uint32_t s) {
     if constexpr (KTAIL) {

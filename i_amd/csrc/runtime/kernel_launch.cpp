@@ -394,8 +394,37 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
 
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 4 == 0 && k <= (size_t(1) << 21); }
 
+unsigned gemm_nt_f32_split_k(size_t bh, size_t m, size_t n, size_t k) {
+  if (bh == 0 || m == 0 || n == 0 || !gemm_nt_f32_supported(k) || std::getenv("ILANG_GEMM_NO_SPLIT")) return 1;
+  auto parts_of = [&](size_t want) -> unsigned {
+    if (want < 2 || bh * want > 65535) return 1;
+    const size_t chunk = (k / want + 63) / 64 * 64;  // what one split contracts: whole slabs
+    return (unsigned)((k + chunk - 1) / chunk);
+  };
+  if (const char* forced = std::getenv("ILANG_GEMM_SPLITS")) return parts_of(std::min<size_t>((size_t)std::max(0, std::atoi(forced)), k / 64));
+  // The model of gemm_nt_bf16_split_k with this kernel's figures: 1.7 us per 32-wide slab for a workgroup on a
+  // 128 x 128 tile, 256 of them at a time (the 256 x 256 tile only takes grids that fill the chip), parts of at
+  // least 64 of k.  Unsplit -> split, us: 128 x 128 x 8192 444 -> 36 (32 parts), 512 x 512 x 4096 227 -> 31 (16),
+  // 1024 x 1024 x 1024 60 -> 27 (4), 8192 x 128 x 8192 (the probabilities times the values of a naive attention)
+  // 451 -> 128 (4), 512 x 64 x 512 34 -> 15 (8); left whole: 2048^3 (120 us; 130 in two parts).
+  const size_t t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh, t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
+  if (t256 >= 128) return 1;  // (the large tile's grids fill the chip)
+  const size_t slabs = (k + 31) / 32;
+  auto time_of = [](size_t workgroups, size_t slabs_) { return (double)((workgroups + 255) / 256) * (double)(slabs_ + 2) * 1.7; };
+  double best = 0.85 * time_of(t128, slabs);
+  size_t splits = 1;
+  for (size_t s = 2; s <= 32 && k / s >= 64 && bh * s <= 65535; s *= 2) {
+    const double t = time_of(t128 * s, (slabs + s - 1) / s) + 4.0 + (double)(bh * s * m * n * 4) / 3e6;
+    if (t < best) {
+      best = t;
+      splits = s;
+    }
+  }
+  return parts_of(splits);
+}
+
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                       hipStream_t stream, LaunchNote* note) {
+                       hipStream_t stream, LaunchNote* note, float* partial, unsigned splits) {
   if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 4 (at most 2^21)";
   if (reinterpret_cast<uintptr_t>(a) % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0)
     return "gemm_nt f32 kernel: operands must be 16-byte aligned";
@@ -409,16 +438,35 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
   unsigned tile = t256 >= 128 ? 256 : 128;
   if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = std::atoi(f) == 128 ? 128 : 256;
+  // the k loop in parts over workgroups (gemm_nt_f32_split_k says when): partial products in the caller's temporary
+  if (splits > 1) {
+    if (!partial) return "gemm_nt f32 kernel: a split needs its temporary";
+    if ((m * n) % 4 != 0) return "gemm_nt f32 kernel: a split product needs m * n to be a multiple of 4";
+    p.k_chunk = (uint32_t)(((k + splits - 1) / splits + 63) / 64 * 64);
+    splits = (unsigned)((k + p.k_chunk - 1) / p.k_chunk);  // (rounding the parts up to whole slabs may leave fewer of them)
+    if (bh * splits > 65535) return "gemm_nt f32 kernel: extent too large";
+  }
+  if (splits > 1) {
+    p.splits = splits;
+    p.c = partial;
+  }
   p.tiles_m = (uint32_t)((m + tile - 1) / tile);
   p.tiles_n = (uint32_t)((n + tile - 1) / tile);
   const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nt f32 kernel: grid too large";
   hipFunction_t fn;
   const std::string name = std::string(tile == 256 ? "gemm_nt_f32_256x256x32_direct" : "gemm_nt_f32_128x128x32_direct") +
-                           (k % 32 != 0 ? "_ktail" : "");  // (a partial last slab of 32 k)
-  if (note) *note = LaunchNote{name, tile, tile};
+                           (k % 32 != 0 ? "_ktail" : "");  // (a partial last slab of 32 k; of the last part, when split)
+  if (note) *note = LaunchNote{splits > 1 ? name + " (k in " + std::to_string(splits) + " parts)" : name, tile, tile};
   if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
+  if (Err e = launch(fn, (unsigned)grid, (unsigned)(bh * (splits > 1 ? splits : 1)), 1, tile == 256 ? 512 : 256, &p, sizeof(p), stream);
+      !e.empty() || splits <= 1)
+    return e;
+  SplitReduceParams r{partial, c, (uint32_t)bh, splits, (uint64_t)m * n, 0u};
+  if (Err e = builtin_function("splitk_reduce", &fn); !e.empty()) return e;
+  size_t rgrid = (bh * m * n / 4 + 255) / 256;
+  if (rgrid > 65536) rgrid = 65536;
+  return launch(fn, (unsigned)rgrid, 1, 1, 256, &r, sizeof(r), stream);
 }
 
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode,

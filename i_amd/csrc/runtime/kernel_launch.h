@@ -68,7 +68,10 @@ bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
 
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 4 == 0 and 16-byte aligned operands
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                       hipStream_t stream, LaunchNote* note = nullptr);
+                       hipStream_t stream, LaunchNote* note = nullptr, float* partial = nullptr, unsigned splits = 1);
+// (splits > 1: the k loop in that many parts over workgroups, as launch_gemm_nt_bf16_split_k does it; `partial` is
+// room for bh * splits * m * n floats, and gemm_nt_f32_split_k says into how many parts, 1: do not split)
+unsigned gemm_nt_f32_split_k(size_t bh, size_t m, size_t n, size_t k);
 bool gemm_nt_f32_supported(size_t k);
 
 // y[rows,cols] = row softmax of x, f32

@@ -304,6 +304,20 @@ def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(tor
         plain = comp.exec_torch(a, b)
         assert "parts)" not in comp.report()
         assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
+    # f32 operands: the same through the f32 kernels, to the f32 bar
+    for shape_a, shape_b, comp in (((64, 2048), (300, 2048), mm_t), ((100, 1000), (100, 1000), mm_t), ((2, 128, 4100), (2, 64, 4100), bmm)):
+        g = torch.Generator(device="cuda").manual_seed(shape_a[-1] + 1)
+        a = torch.rand(*shape_a, device="cuda", generator=g) * 2 - 1
+        b = torch.rand(*shape_b, device="cuda", generator=g) * 2 - 1
+        ref = a.double() @ b.double().transpose(-1, -2)
+        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        got = comp.exec_torch(a, b)
+        assert "_f32_" in comp.report() and "parts)" in comp.report(), comp.report()
+        assert float((got.double() - ref).abs().max()) <= RTOL_F32 * float(ref.abs().max())
+        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        plain = comp.exec_torch(a, b)
+        assert "parts)" not in comp.report()
+        assert float((plain - got).abs().max()) <= 1e-5 * float(ref.abs().max())
     # a product that fills the chip is left alone
     monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
     a = torch.randn(2048, 4096, device="cuda").bfloat16()
