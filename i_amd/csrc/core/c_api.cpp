@@ -5,6 +5,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <algorithm>
+#include <map>
+#include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -67,6 +70,40 @@ std::vector<std::vector<size_t>> host_shapes(const ihipc::Program& p, const i_te
   return out;
 }
 
+// Device memory for the operands of host calls: one block per device that the library keeps from call to call
+// (a host call returns after the GPU has finished, so the block is free again), as large as the largest call needed,
+// at most ILANG_HIP_STAGING_MB (default 1024; 0: every operand is allocated, copied and freed on its own).  Calls
+// whose operands fit 8 MiB go through a page-locked host mirror of the block as well: the inputs are gathered
+// there and cross in one asynchronous copy, the outputs come back in one, instead of a blocking copy from pageable
+// memory per operand.  A call that finds the block in use by another thread, or needs more, allocates as before;
+// so does the emulated runtime, whose allocations are guarded one by one.
+struct Staging {
+  void* base = nullptr;
+  size_t capacity = 0;
+  void* pinned = nullptr;  // a page-locked host mirror of the first kPinnedBytes of the block (small calls)
+  std::mutex busy;
+};
+constexpr size_t kPinnedBytes = size_t(8) << 20;
+
+Staging* staging_of_current_device() {
+  static std::mutex mu;
+  static std::map<int, std::unique_ptr<Staging>> blocks;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  auto& block = blocks[device];
+  if (!block) block = std::make_unique<Staging>();
+  return block.get();
+}
+
+size_t staging_limit() {
+  static const size_t limit = [] {
+    const char* mb = std::getenv("ILANG_HIP_STAGING_MB");
+    return (mb ? (size_t)std::max(0, std::atoi(mb)) : size_t(1024)) << 20;
+  }();
+  return limit;
+}
+
 // Host entry: upload f32 operands, run, download, wait.  Mirrors the
 // blocking behaviour of the reference's exec (core/src/lib.rs:200-225).
 std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_count, const std::vector<float*>& out_ptrs) {
@@ -74,11 +111,62 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
   std::vector<std::vector<size_t>> out_shapes;
   if (std::string e = ihipc::output_shapes(p, in_shapes, &out_shapes); !e.empty()) return e;
   std::vector<void*> owned;
+  hipStream_t stream = nullptr;
+  bool staged = false;
   auto cleanup = [&] {
+    if (staged) (void)ihip::sync(stream);  // (an early return: nothing may still be using the kept block)
     for (void* ptr : owned) ihip::dev_free(ptr);
   };
+  // the operands' device copies: carved from the kept block when it is free and large enough (or can be made so)
+  auto bytes_of = [](const std::vector<size_t>& shape) {
+    size_t n = 4;
+    for (size_t d : shape) n *= d;
+    return (std::max<size_t>(n, 4) + 255) / 256 * 256;
+  };
+  size_t wanted = 0;
+  for (size_t i = 0; i < input_count; ++i) wanted += bytes_of(in_shapes[i]);
+  for (const auto& shape : out_shapes) wanted += bytes_of(shape);
+  std::unique_lock<std::mutex> staging_lock;
+  char* carve = nullptr;
+  char *mirror = nullptr, *block_base = nullptr;  // mirror != nullptr: host data passes through the page-locked mirror
+  if (wanted <= staging_limit() && !ihip::runtime_is_emulated()) {
+    if (Staging* block = staging_of_current_device()) {
+      staging_lock = std::unique_lock<std::mutex>(block->busy, std::try_to_lock);
+      if (staging_lock.owns_lock()) {
+        if (block->capacity < wanted) {
+          ihip::dev_free(block->base);
+          block->base = nullptr;
+          block->capacity = 0;
+          if (ihip::dev_alloc(&block->base, wanted).empty()) block->capacity = wanted;
+        }
+        if (block->capacity >= wanted) {
+          carve = static_cast<char*>(block->base);
+          staged = true;
+          if (wanted <= kPinnedBytes) {
+            if (!block->pinned && hipHostMalloc(&block->pinned, kPinnedBytes, hipHostMallocDefault) != hipSuccess) {
+              block->pinned = nullptr;
+              (void)hipGetLastError();
+            }
+            mirror = static_cast<char*>(block->pinned);
+          }
+          block_base = carve;
+        }
+      }
+    }
+  }
+  auto device_copy = [&](void** ptr, const std::vector<size_t>& shape) -> ihip::Err {
+    if (carve) {
+      *ptr = carve;
+      carve += bytes_of(shape);
+      return {};
+    }
+    size_t n = 1;
+    for (size_t d : shape) n *= d;
+    if (ihip::Err e = ihip::dev_alloc(ptr, n * 4); !e.empty()) return e;
+    owned.push_back(*ptr);
+    return {};
+  };
   std::vector<ihipc::DeviceTensor> in, out;
-  hipStream_t stream = nullptr;
   for (size_t i = 0; i < input_count; ++i) {
     size_t n = 1;
     for (size_t d : in_shapes[i]) n *= d;
@@ -88,27 +176,34 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
       cleanup();
       return "input " + std::to_string(i) + " has no data";
     }
-    if (ihip::Err e = ihip::dev_alloc(&t.data, n * 4); !e.empty()) {
+    if (ihip::Err e = device_copy(&t.data, in_shapes[i]); !e.empty()) {
       cleanup();
       return e;
     }
-    owned.push_back(t.data);
-    if (ihip::Err e = ihip::h2d(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
+    if (mirror) {
+      if (n) std::memcpy(mirror + (static_cast<char*>(t.data) - block_base), inputs[i].data, n * 4);
+    } else if (ihip::Err e = ihip::h2d(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
       cleanup();
       return e;
     }
     in.push_back(std::move(t));
+  }
+  const size_t input_bytes = carve ? (size_t)(carve - block_base) : 0;  // (the inputs lie first in the block)
+  if (mirror && input_bytes) {
+    if (ihip::Err e = ihip::h2d(block_base, mirror, input_bytes, stream); !e.empty()) {
+      cleanup();
+      return e;
+    }
   }
   for (size_t o = 0; o < out_shapes.size(); ++o) {
     size_t n = 1;
     for (size_t d : out_shapes[o]) n *= d;
     ihipc::DeviceTensor t;
     t.shape = out_shapes[o];
-    if (ihip::Err e = ihip::dev_alloc(&t.data, n * 4); !e.empty()) {
+    if (ihip::Err e = device_copy(&t.data, out_shapes[o]); !e.empty()) {
       cleanup();
       return e;
     }
-    owned.push_back(t.data);
     out.push_back(std::move(t));
   }
   std::string err;
@@ -121,10 +216,17 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
     size_t n = 1;
     for (size_t d : out_shapes[o]) n *= d;
     if (n && !out_ptrs[o]) err = "output " + std::to_string(o) + " has no data";
-    else err = ihip::d2h(out_ptrs[o], out[o].data, n * 4, stream);
+    else if (!mirror) err = ihip::d2h(out_ptrs[o], out[o].data, n * 4, stream);
   }
+  if (mirror && err.empty() && carve - block_base > (ptrdiff_t)input_bytes)
+    err = ihip::d2h(mirror + input_bytes, block_base + input_bytes, (size_t)(carve - block_base) - input_bytes, stream);
   const ihip::Err sync_err = ihip::sync(stream);
   if (err.empty()) err = sync_err;
+  for (size_t o = 0; mirror && err.empty() && o < out.size(); ++o) {
+    size_t n = 1;
+    for (size_t d : out_shapes[o]) n *= d;
+    if (n) std::memcpy(out_ptrs[o], mirror + (static_cast<char*>(out[o].data) - block_base), n * 4);
+  }
   cleanup();
   return err;
 }

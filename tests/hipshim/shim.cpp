@@ -98,6 +98,7 @@ hipError_t hipMallocAsync(void** p, size_t bytes, hipStream_t) { return guarded_
 hipError_t hipFreeAsync(void* p, hipStream_t) { return guarded_free(p); }
 // (the library asks ilang_hip_runtime_is_emulated first and creates no pool here; these only satisfy the linker)
 hipError_t hipGetLastError() { return hipSuccess; }
+hipError_t hipHostMalloc(void**, size_t, unsigned int) { return hipErrorNotSupported; }
 hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* status) {
   *status = hipStreamCaptureStatusNone;
   return hipSuccess;
