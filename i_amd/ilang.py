@@ -247,6 +247,7 @@ class Component:
     def __init__(self, src=None, *, _handle=None):
         self._ptr = None
         self._program = None
+        self._extents_seen = {}  # output extents by input extents
         if _handle is None:
             if not isinstance(src, str):
                 raise TypeError("Component takes the source text of one expression")
@@ -322,6 +323,17 @@ class Component:
             core.i_string_free(text)
 
     def _result_extents(self, program, operands):
+        # (asked of the library once per combination of input shapes: a serving loop calls with the same ones)
+        key = tuple(op.extents for op in operands)
+        cache = self._extents_seen
+        found = cache.get(key)
+        if found is None:
+            if len(cache) >= 64:
+                cache.clear()
+            found = cache[key] = self._ask_result_extents(program, operands)
+        return list(found)
+
+    def _ask_result_extents(self, program, operands):
         count = core.i_output_count(program)
         ranks = (_sz * max(count, 1))()
         nat.check(core.i_output_ranks(program, ranks))
