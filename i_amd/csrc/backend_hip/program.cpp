@@ -83,6 +83,7 @@ struct Run {
   std::vector<std::string> notes;            // one line per dispatched kernel: what ran, on which tile
   Arena* arena = nullptr;                    // when set (and locked by this call), temporaries come off it while they fit
   size_t arena_used = 0, arena_needed = 0;
+  bool capturing = false;                    // the stream is being captured into a graph
 
   size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
   size_t extent(const Extent<size_t>& e) const {
@@ -137,7 +138,10 @@ struct Run {
         return {};
       }
     }
-    if (ihip::Err e = ihip::temp_alloc(ptr, bytes, stream); !e.empty()) return e;
+    // (a stream under capture: the plain stream-ordered allocation, which a graph records as a node of its own)
+    if (ihip::Err e = capturing ? ihip::check(hipMallocAsync(ptr, bytes, stream), "hipMallocAsync") : ihip::temp_alloc(ptr, bytes, stream);
+        !e.empty())
+      return e;
     temps.push_back(*ptr);
     return {};
   }
@@ -840,11 +844,13 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
   }
 
   std::unique_lock<std::mutex> arena_lock;
-  if (!workspace && arena_limit() > 0 && !ihip::runtime_is_emulated()) {
+  if (!workspace && !ihip::runtime_is_emulated()) {
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
       (void)hipGetLastError();
-    } else if (capture == hipStreamCaptureStatusNone) {
+    } else if (capture != hipStreamCaptureStatusNone) {
+      run.capturing = true;
+    } else if (arena_limit() > 0) {
       if (Arena* arena = arena_of(stream)) {
         arena_lock = std::unique_lock<std::mutex>(arena->busy, std::try_to_lock);
         if (arena_lock.owns_lock()) run.arena = arena;

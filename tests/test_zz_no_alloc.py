@@ -108,6 +108,42 @@ def test_split_loops_keep_their_partial_results_in_the_workspace(torch, monkeypa
         assert "(keys in 3 parts)" in attention.report(), attention.report()
 
 
+def test_both_device_entry_points_under_graph_capture(torch):
+    """What the entry point that allocates nothing is for: captured into a HIP graph (after one eager call, which
+    loads the code object and compiles the generated kernels) and replayed three times, with new input values,
+    eager work and a synchronisation between the replays, every replay checked.  The allocating entry point is
+    captured too: under capture its temporaries are plain stream-ordered allocations, which the graph records."""
+    sm = softmax_naive()
+    s = "i:16,j:16"
+    attention = ((i(f"bik*bjk~bijk | {s} | bjii'j'k") >> i(f"+bijk~bij | {s} | bjii'j'k0"))
+                 >> ((I & i(f">bij~bi | {s} | bji0i'j'")) >> i(f"bij-bi~bij | {s} | bji01i'j'")) >> i(f"^bij~bij | {s} | bji0i'j'")
+                 >> ((I & i(f"+bij~bi | {s} | bji0i'j'")) >> i(f"bij/bi~bij | {s} | bji01i'j'"))
+                 >> (i(f"bij*bjk~bikj | {s} | bji0i'kj'") >> i(f"+bikj~bik | {s} | bjii'kj'0")))
+    x, y = randn(torch, (512, 777), 12), torch.empty(512, 777, device="cuda")
+    q, k, v = (randn(torch, (2, 300, 128), seed, torch.bfloat16) * 0.3 for seed in (13, 14, 15))
+    o = torch.empty(2, 300, 128, device="cuda")
+    for static in (True, False):
+        print("case graph capture, static workspace", static, flush=True)
+        sm.into(y, x, static_workspace=static)
+        attention.into(o, q, k, v, static_workspace=static)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            sm.into(y, x, static_workspace=static)
+            attention.into(o, q, k, v, static_workspace=static)
+        for rep in range(3):
+            x.copy_(randn(torch, (512, 777), 20 + rep))
+            q.copy_(randn(torch, (2, 300, 128), 30 + rep, torch.bfloat16) * 0.3)
+            y.fill_(float("nan"))
+            o.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert float((y.double() - torch.softmax(x.double(), -1)).abs().max()) <= 1e-6
+            ref = torch.softmax(q.double() @ k.double().transpose(1, 2), -1) @ v.double()
+            assert float((o.double() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+
+
 def test_operands_beyond_the_workspace_are_refused_before_anything_runs(torch):
     comp = softmax_naive()
     x = randn(torch, (8192, 4096), 5)  # two 128 MiB intermediates
