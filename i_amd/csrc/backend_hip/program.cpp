@@ -476,8 +476,14 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       }
       const void *pa = nullptr, *pb_rows = nullptr;
       if (ihip::Err e = product_operands(run, r, f32 ? DType::F32 : DType::BF16, &pa, &pb_rows); !e.empty()) return e;
-      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k))  // the direct kernels read a row-major right operand themselves
-        return ihip::launch_gemm_nn_bf16(pa, pb_rows, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note, out_dt);
+      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k)) {  // the direct kernels read a row-major right operand themselves
+        const bool tile_asked = (r.tile_i == 128 && r.tile_j == 128) || (r.tile_i == 256 && r.tile_j == 256);
+        unsigned splits = tile_asked ? 1u : ihip::gemm_nt_bf16_split_k(bh, m, n, k);
+        void* partial = nullptr;
+        if (splits > 1 && ((m * n) % 4 != 0 || !run.alloc_optional(&partial, bh * splits * m * n * 4))) splits = 1;
+        return ihip::launch_gemm_nn_bf16(pa, pb_rows, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note, out_dt,
+                                         static_cast<float*>(partial), splits);
+      }
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
       if (ihip::Err e = run.alloc(&bt, bh * n * k * elem); !e.empty()) return e;

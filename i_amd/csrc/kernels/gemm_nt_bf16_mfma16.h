@@ -67,7 +67,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   static_assert(WL % NWAVES == 0 && NWAVES % 2 == 0 && TM >= 2 && TN >= 2, "slab shape");
   char (*smem)[2][SLAB] = reinterpret_cast<char (*)[2][SLAB]>(smem_base);  // [buffer][A, B]
   // (the k loop split over workgroups: blockIdx.y counts (batch, split) pairs)
-  const uint32_t nsplit = (!NN && p.splits > 1) ? p.splits : 1u;
+  const uint32_t nsplit = p.splits > 1 ? p.splits : 1u;
   const uint32_t batch = blockIdx.y / nsplit, split = blockIdx.y - batch * nsplit;
   const uint32_t k_first = split * p.k_chunk;                                            // first k of this split
   const uint32_t kk = nsplit > 1 ? (p.k - k_first < p.k_chunk ? p.k - k_first : p.k_chunk) : p.k;  // its extent
@@ -80,7 +80,8 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
 
   const size_t row_bytes = (size_t)p.k * 2;
   const char* __restrict__ A = reinterpret_cast<const char*>(p.a) + (size_t)batch * p.m * row_bytes + (size_t)k_first * 2;
-  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes + (size_t)k_first * 2;
+  const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes +
+                               (NN ? (size_t)k_first * p.n * 2 : (size_t)k_first * 2);  // (NN: rows of B are k)
   char* __restrict__ C = reinterpret_cast<char*>(p.c) + (size_t)blockIdx.y * p.m * p.n * (p.out_bf16 ? 2 : 4);
   const uint32_t m0 = tm * BT, n0 = tn * BT;
 

@@ -41,7 +41,7 @@ struct GemmParams {
   uint32_t bh, m, n, k;
   uint32_t tiles_m, tiles_n;
   uint32_t out_bf16;  // 0: f32 output, 1: the f32 sums are rounded to bf16 on the way out
-  // The k loop split over workgroups (direct NT kernels only; 0 or 1: not split).  blockIdx.y then counts
+  // The k loop split over workgroups (the direct kernels, NT and NN; 0 or 1: not split).  blockIdx.y then counts
   // (batch, split) pairs; split s contracts k_chunk * s .. + k_chunk (what is left of k for the last one) and
   // writes its f32 partial products to c[(batch * splits + s)][m][n], a temporary that splitk_reduce adds up.
   uint32_t splits;

@@ -369,8 +369,9 @@ static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t til
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return gemm_nn_tile(bh, m, n, k, 0, 0) != 0; }
 
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype) {
-  const unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype, float* partial,
+                        unsigned splits) {
+  unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
   if (tile == 0) return "gemm_nn kernel: needs k % 8 == 0 and n % 8 == 0 (and extents within its offset range)";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!a || !b || !c) return "gemm_nn kernel: null device pointer";
@@ -378,6 +379,21 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
+  // the k loop in parts over workgroups (gemm_nt_bf16_split_k says when, for this form too): f32 partial products
+  // in the caller's temporary, added up by splitk_reduce
+  if (splits > 1) {
+    if (!partial) return "gemm_nn kernel: a split needs its temporary";
+    if ((m * n) % 4 != 0) return "gemm_nn kernel: a split product needs m * n to be a multiple of 4";
+    p.k_chunk = (uint32_t)(((k + splits - 1) / splits + 63) / 64 * 64);
+    splits = (unsigned)((k + p.k_chunk - 1) / p.k_chunk);  // (rounding the parts up to whole slabs may leave fewer of them)
+    if (bh * splits > 65535) return "gemm_nn kernel: extent too large";
+  }
+  if (splits > 1) {
+    p.splits = splits;
+    p.c = partial;
+    p.out_bf16 = 0;
+    tile = split_k_tile(m, n);
+  }
   p.tiles_m = (uint32_t)((m + tile - 1) / tile);
   p.tiles_n = (uint32_t)((n + tile - 1) / tile);
   const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
@@ -387,9 +403,16 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   const bool w4 = tile == 256 && !(waves && std::atoi(waves) == 8);
   const std::string name = std::string(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct") +
                            (k % 64 != 0 ? "_ktail" : "") + (w4 ? "_w4" : "");
-  if (note) *note = LaunchNote{name, tile, tile};
+  if (note) *note = LaunchNote{splits > 1 ? name + " (k in " + std::to_string(splits) + " parts)" : name, tile, tile};
   if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-  return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
+  if (Err e = launch(fn, (unsigned)grid, (unsigned)(bh * (splits > 1 ? splits : 1)), 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
+      !e.empty() || splits <= 1)
+    return e;
+  SplitReduceParams r{partial, c, (uint32_t)bh, splits, (uint64_t)m * n, out_dtype == BF16 ? 1u : 0u};
+  if (Err e = builtin_function("splitk_reduce", &fn); !e.empty()) return e;
+  size_t rgrid = (bh * m * n / 4 + 255) / 256;
+  if (rgrid > 65536) rgrid = 65536;
+  return launch(fn, (unsigned)rgrid, 1, 1, 256, &r, sizeof(r), stream);
 }
 
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 4 == 0 && k <= (size_t(1) << 21); }

@@ -61,9 +61,11 @@ Err launch_gemm_nt_bf16_split_k(const void* a, const void* b, void* c, float* pa
 
 // c[bh,m,n] (f32) = a[bh,m,k] b[bh,k,n], a and b bf16, on the direct kernels with a row-major right operand.
 // Needs k % 8 == 0 and n % 8 == 0 (gemm_nn_bf16_supported); callers transpose b and use the NT kernels otherwise.
+// (splits > 1: the k loop in that many parts, as launch_gemm_nt_bf16_split_k does it, gemm_nt_bf16_split_k deciding;
+// `partial` is room for bh * splits * m * n floats)
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                         hipStream_t stream, size_t tile_m = 0, size_t tile_n = 0, LaunchNote* note = nullptr,
-                        DType out_dtype = F32);
+                        DType out_dtype = F32, float* partial = nullptr, unsigned splits = 1);
 bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k);
 
 // c[bh,m,n] = a[bh,m,k] b[bh,n,k]^T, all f32, products and sums in f32 (f32 MFMA); needs k % 4 == 0 and 16-byte aligned operands

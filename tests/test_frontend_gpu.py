@@ -304,6 +304,23 @@ def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(tor
         plain = comp.exec_torch(a, b)
         assert "parts)" not in comp.report()
         assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
+    # a row-major right operand (c = a b): the same kernels' NN forms split the same way
+    mm = i("ik*kj~ijk|i:16,k:16|ii'jkk'") >> i("+ijk~ij|i:16,k:16|ii'j!kk'0")
+    for m, k, n in ((64, 8192, 1000), (300, 5000, 264), (40, 4104, 72)):
+        g = torch.Generator(device="cuda").manual_seed(k + 2)
+        a = (torch.rand(m, k, device="cuda", generator=g) * 2 - 1).bfloat16()
+        b = (torch.rand(k, n, device="cuda", generator=g) * 2 - 1).bfloat16()
+        ref = a.double() @ b.double()
+        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        got = mm.exec_torch(a, b)
+        assert "gemm_nn_bf16" in mm.report() and "parts)" in mm.report(), mm.report()
+        assert float((got.double() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
+        got16 = mm.exec_torch(a, b, out_dtype=torch.bfloat16)
+        assert float((got16.double() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        plain = mm.exec_torch(a, b)
+        assert "parts)" not in mm.report()
+        assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
     # f32 operands: the same through the f32 kernels, to the f32 bar
     for shape_a, shape_b, comp in (((64, 2048), (300, 2048), mm_t), ((100, 1000), (100, 1000), mm_t), ((2, 128, 4100), (2, 64, 4100), bmm)):
         g = torch.Generator(device="cuda").manual_seed(shape_a[-1] + 1)
