@@ -572,6 +572,57 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
     assert "keys in" not in comp.report()
 
 
+def test_random_shapes_through_the_split_loops(torch, monkeypatch):
+    """Forty random attentions (bf16 and f32, head sizes of every kernel family, 1 to 400 queries, 130 to 3000 keys)
+    with their keys in 2 to 32 parts, and forty random products (NT and NN, bf16 and f32, every extent ragged) with
+    their k loop in 2 to 32 parts, against float64."""
+    import random
+
+    rng = random.Random(7)
+    fa = flash(prefix="b", scaled=True)
+    mm_t = i("bik*bjk~bijk | i:16,j:16 | bjii'j'k") >> i("+bijk~bij | i:16,j:16 | bjii'j'k0")
+    mm = i("bik*bkj~bijk|i:16,k:16|bii'jkk'") >> i("+bijk~bij|i:16,k:16|bii'j!kk'0")
+    split = 0
+    for case in range(40):
+        bf16 = rng.random() < 0.6
+        bh, nq, nk = rng.choice([1, 1, 2, 3]), rng.randint(1, 400), rng.randint(130, 3000)
+        d = rng.choice([64, 128, 72, 40, 256, 96] if bf16 else [64, 128, 96, 40])
+        dv = d if rng.random() < 0.7 else rng.choice([64, 128, 32 + 8 * rng.randint(0, 8)])
+        if not bf16 and dv > 128:
+            dv = d
+        dt = torch.bfloat16 if bf16 else torch.float32
+        g = torch.Generator(device="cuda").manual_seed(case)
+        q, k, v = ((torch.randn(bh, n, w, device="cuda", generator=g) * 0.7).to(dt) for n, w in ((nq, d), (nk, d), (nk, dv)))
+        ref = torch.softmax((q.double() @ k.double().transpose(1, 2)) * d ** -0.5, -1) @ v.double()
+        monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", str(rng.choice([2, 3, 5, 8, 13, 32])))
+        print("case attention", case, bf16, bh, nq, nk, d, dv, flush=True)
+        got = fa.exec_torch(q, k, torch.tensor(d ** -0.5, device="cuda"), v)
+        split += "(keys in" in fa.report()
+        assert float((got.double() - ref).abs().max()) <= (RTOL_BF16 if bf16 else RTOL_F32) * float(ref.abs().max()), fa.report()
+    monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
+    assert split >= 30  # (head sizes no direct kernel has run unsplit)
+    split = 0
+    for case in range(40):
+        kind = rng.choice(["nt16", "nn16", "nt32", "nn32"])
+        bh, m, n, k = rng.choice([1, 1, 2, 5]), rng.randint(1, 500), rng.randint(1, 500), rng.randint(64, 6000)
+        k = k // 8 * 8 if kind.endswith("16") else k // 4 * 4
+        if kind == "nn16":
+            n = max(8, n // 8 * 8)
+        dt = torch.bfloat16 if kind.endswith("16") else torch.float32
+        g = torch.Generator(device="cuda").manual_seed(100 + case)
+        a = (torch.rand(bh, m, k, device="cuda", generator=g) * 2 - 1).to(dt)
+        b = (torch.rand(*((bh, n, k) if kind.startswith("nt") else (bh, k, n)), device="cuda", generator=g) * 2 - 1).to(dt)
+        ref = a.double() @ (b.double().transpose(1, 2) if kind.startswith("nt") else b.double())
+        monkeypatch.setenv("ILANG_GEMM_SPLITS", str(rng.choice([2, 3, 4, 7, 16, 32])))
+        print("case product", case, kind, bh, m, n, k, flush=True)
+        comp = mm_t if kind.startswith("nt") else mm
+        got = comp.exec_torch(a, b)
+        split += "(k in" in comp.report()
+        bar = 1e-2 if kind.endswith("16") else RTOL_F32
+        assert float((got.double() - ref).abs().max()) <= bar * max(float(ref.abs().max()), 1e-30), comp.report()
+    assert split >= 25  # (m * n that is no multiple of 4 runs unsplit)
+
+
 def test_temporaries_are_kept_from_call_to_call_on_a_stream(torch):
     """Calls enqueued back to back on one stream carve their temporaries (here the two [rows, cols] intermediates
     of the naive softmax) from one block that the library keeps and replaces when a call needs more: operands that
