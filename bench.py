@@ -29,6 +29,7 @@ from the committed summary under profiles/ and is null when that is missing.
 """
 import argparse
 import json
+import os
 import re
 import sys
 import time
@@ -290,6 +291,23 @@ def main():
     c1_kernel = demo.report().split()[1]
     _, c1_ms = time_steps(torch, lambda: demo.into(dout, dq, dk, dv_), short_steps, short_warmup)
     c1_flop = 4.0 * 512 * 512 * 64
+    c1_launches = demo.report().strip()
+
+    # ------------------------------------------------------------------ one head of the headline's size class on its own
+    # (bf16 [1, 8192, 128]: 32 query tiles of 256 rows for 256 CUs): the keys of the head in parts over workgroups, and the same
+    # call with the split switched off
+    q1, k1, v1 = (t_[0:1, 0:1].repeat(1, 1, 2, 1).contiguous() for t_ in (q, k, v))
+    one_out = torch.empty(1, 1, 2 * N, D, dtype=torch.float32, device=dev)
+    attn.into(one_out, q1, k1, scale, v1)
+    one_launches = attn.report().strip()
+    _, one_ms = time_steps(torch, lambda: attn.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
+    os.environ["ILANG_ATTN_KV_SPLITS"] = "1"
+    try:
+        attn.into(one_out, q1, k1, scale, v1)
+        _, one_whole_ms = time_steps(torch, lambda: attn.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
+    finally:
+        del os.environ["ILANG_ATTN_KV_SPLITS"]
+    one_flop = 4.0 * (2 * N) * (2 * N) * D
 
     # ------------------------------------------------------------------ the attention workload in f32 (the reference's
     # arithmetic type): batches 2 and 3 of the headline operands as f32, through the same compiled component
@@ -421,8 +439,12 @@ def main():
              "cpu_baseline": cpu5, "rel_err": err5},
             {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,
-             "steps": short_steps, "warmup": short_warmup,
+             "steps": short_steps, "warmup": short_warmup, "launches": c1_launches,
              "cpu_baseline": cpu1, "rel_err": err1},
+            {"workload": f"flash_attention_fwd of one head, bf16 [1,{2 * N},{D}] (not a BASELINE configuration): 32 query "
+                         "tiles of 256 rows for 256 CUs, so the keys of the head run in parts over workgroups",
+             "value": one_flop / (one_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_call": one_ms, "launches": one_launches,
+             "ms_per_call_unsplit": one_whole_ms, "steps": short_steps, "warmup": short_warmup},
             {"workload": f"flash_attention_fwd B{BF} H32 N4096 d128 with f32 operands (batches 2 and 3 of the headline "
                          "operands as f32, full f32 arithmetic: the reference's own type; not a BASELINE configuration)",
              "value": f32_tflops, "unit": "TFLOP/s", "dtype": "f32",
