@@ -301,9 +301,11 @@ def main():
     attn.into(one_out, q1, k1, scale, v1)
     one_launches = attn.report().strip()
     _, one_ms = time_steps(torch, lambda: attn.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
+    one_split = one_out.clone()
     os.environ["ILANG_ATTN_KV_SPLITS"] = "1"
     try:
         attn.into(one_out, q1, k1, scale, v1)
+        one_err = float((one_split - one_out).abs().max() / one_out.abs().max())
         _, one_whole_ms = time_steps(torch, lambda: attn.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
     finally:
         del os.environ["ILANG_ATTN_KV_SPLITS"]
@@ -441,16 +443,16 @@ def main():
              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,
              "steps": short_steps, "warmup": short_warmup, "launches": c1_launches,
              "cpu_baseline": cpu1, "rel_err": err1},
-            {"workload": f"flash_attention_fwd of one head, bf16 [1,{2 * N},{D}] (not a BASELINE configuration): 32 query "
-                         "tiles of 256 rows for 256 CUs, so the keys of the head run in parts over workgroups",
-             "value": one_flop / (one_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_call": one_ms, "launches": one_launches,
-             "ms_per_call_unsplit": one_whole_ms, "steps": short_steps, "warmup": short_warmup},
             {"workload": f"flash_attention_fwd B{BF} H32 N4096 d128 with f32 operands (batches 2 and 3 of the headline "
                          "operands as f32, full f32 arithmetic: the reference's own type; not a BASELINE configuration)",
              "value": f32_tflops, "unit": "TFLOP/s", "dtype": "f32",
              "roofline": roof("mfma", f32_tflops, PEAK_F32_TFLOPS, "TFLOP/s", "flash_attention_B2_H32_N4096_d128_f32.md",
                               f32_kernel, f32_ms),
              "cpu_baseline": cpuf, "rel_err": errf},
+            {"workload": f"flash_attention_fwd of one head, bf16 [1,{2 * N},{D}] (not a BASELINE configuration): 32 query "
+                         "tiles of 256 rows for 256 CUs, so the keys of the head run in parts over workgroups",
+             "value": one_flop / (one_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_call": one_ms, "launches": one_launches,
+             "ms_per_call_unsplit": one_whole_ms, "rel_err_against_unsplit": one_err, "steps": short_steps, "warmup": short_warmup},
         ],
     }
     print(json.dumps(line))

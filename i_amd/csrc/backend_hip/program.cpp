@@ -505,7 +505,12 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       if (ihip::Err e = run.read_f32(r.a.buffer, &in); !e.empty()) return e;
       if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) return e;
       const int mode = r.kind == Recognized::RowSoftmax ? 0 : r.kind == Recognized::RowMaxShift ? 1 : r.kind == Recognized::RowNormalize ? 2 : 3;
-      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode, note);
+      // a few very long rows: every row in parts over workgroups, the parts' (max, sum) pairs in a small temporary
+      unsigned parts = ihip::row_softmax_parts(rows, x.back(), mode);
+      void* stats = nullptr;
+      if (parts > 1 && !run.alloc(&stats, rows * parts * 8).empty()) parts = 1;
+      return ihip::launch_row_softmax(static_cast<const float*>(in), static_cast<float*>(out), rows, x.back(), run.stream, mode, note,
+                                      nullptr, 1.0f, static_cast<float*>(stats), parts);
     }
     default: return "no hand-written kernel";
   }

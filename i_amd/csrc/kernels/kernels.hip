@@ -191,7 +191,22 @@ extern "C" __global__ void __launch_bounds__(512, 1) gemm_nt_f32_256x256x32_dire
   extern "C" __global__ void __launch_bounds__(1024) row_##OP##_block_v(SoftmaxParams p) {         \
     row_softmax_block_body<MODE, true>(p);                                                         \
   }
+#define ROW_PARTS(OP, MODE)                                                                                   \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_parts_stats(SoftmaxParams p) {                \
+    row_softmax_parts_body<MODE, false, 0>(p);                                                                \
+  }                                                                                                           \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_parts_stats_v(SoftmaxParams p) {              \
+    row_softmax_parts_body<MODE, true, 0>(p);                                                                 \
+  }                                                                                                           \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_parts_apply(SoftmaxParams p) {                \
+    row_softmax_parts_body<MODE, false, 1>(p);                                                                \
+  }                                                                                                           \
+  extern "C" __global__ void __launch_bounds__(1024) row_##OP##_parts_apply_v(SoftmaxParams p) {              \
+    row_softmax_parts_body<MODE, true, 1>(p);                                                                 \
+  }
 ROW_OP(softmax, 0)
+ROW_PARTS(softmax, 0)
+ROW_PARTS(scaled_softmax, 4)
 ROW_OP(shift, 1)
 ROW_OP(norm, 2)
 ROW_OP(exp, 3)

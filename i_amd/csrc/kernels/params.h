@@ -64,6 +64,11 @@ struct SoftmaxParams {
   // the "softmax of scale * x" kernels only: scale = scale_value * (scale_ptr ? *scale_ptr : 1)
   const float* scale_ptr;
   float scale_value;
+  // A row in parts over workgroups (row_*_parts_* kernels: fewer rows than CUs, very long rows): blockIdx.x counts
+  // (row, part) pairs, part s covers the accesses part_chunks * s .. + part_chunks of its row; the first kernel
+  // leaves each part's running max and sum of exponentials in stats[row][part][2], the second combines them.
+  float* stats;
+  uint32_t parts, part_chunks;
 };
 
 struct ConvertParams {

@@ -416,3 +416,82 @@ __device__ __forceinline__ void row_softmax_block_body(const SoftmaxParams& p) {
     store(c, v);
   }
 }
+
+// A row in parts over workgroups, for softmax of a few very long rows (fewer rows than CUs): workgroup (row, part)
+// takes the accesses part_chunks * part .. + part_chunks of its row.  PASS 0 computes the part's (m, s) pair as
+// the block kernel's first pass does and stores it; PASS 1 (a second launch) combines the pairs of its row in part
+// order and writes its part of the result.  HBM sees the row twice on the way in, once on the way out.
+template <int MODE, bool VEC, int PASS>
+__device__ __forceinline__ void row_softmax_parts_body(const SoftmaxParams& p) {
+  static_assert(MODE == 0 || MODE == 4, "softmax only");
+  __shared__ float red[2][16];
+  const uint32_t row = blockIdx.x / p.parts, part = blockIdx.x - row * p.parts;
+  const float* __restrict__ x = p.x + (size_t)row * p.cols;
+  float* __restrict__ y = p.y + (size_t)row * p.cols;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  constexpr int W = VEC ? 4 : 1;
+  const uint32_t chunks = VEC ? p.cols / 4 : p.cols;
+  const uint32_t first = part * p.part_chunks, last = first + p.part_chunks < chunks ? first + p.part_chunks : chunks;
+  auto load = [&](uint32_t c) {
+    f32x4 v;
+    if constexpr (VEC) v = *reinterpret_cast<const f32x4*>(x + 4 * (size_t)c);
+    else v[0] = x[c];
+    return v;
+  };
+  const float sc = MODE == 4 ? load_scale(p.scale_ptr, p.scale_value) : 1.0f;
+  auto weight = [](float from, float to) { return from == to ? 1.0f : fast_exp2(from - to); };
+  auto merge = [&](float& ma, float& sa, float mb, float sb) {
+    const float mn = fmaxf(ma, mb);
+    sa = sa * weight(ma, mn) + sb * weight(mb, mn);
+    ma = mn;
+  };
+  float* stats = p.stats + (size_t)row * p.parts * 2;
+  if constexpr (PASS == 0) {
+    float m = -INFINITY, s = 0.0f;
+#pragma unroll 4
+    for (uint32_t c = first + threadIdx.x; c < last; c += blockDim.x) {
+      f32x4 v = load(c);
+      float cm = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < W; ++e) {
+        v[e] = v[e] * sc * I_LOG2_E32;
+        cm = fmaxf(cm, v[e]);
+      }
+      const float mn = fmaxf(m, cm);
+      s *= weight(m, mn);
+#pragma unroll
+      for (int e = 0; e < W; ++e) s += fast_exp2(v[e] - mn);
+      m = mn;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float mo = __shfl_xor(m, o, 64), so = __shfl_xor(s, o, 64);
+      merge(m, s, mo, so);
+    }
+    if (lane == 0) {
+      red[0][wave] = m;
+      red[1][wave] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      m = red[0][0];
+      s = red[1][0];
+      for (int w = 1; w < nw; ++w) merge(m, s, red[0][w], red[1][w]);
+      stats[2 * part] = m;
+      stats[2 * part + 1] = s;
+    }
+  } else {
+    float m = stats[0], s = stats[1];
+    for (uint32_t t = 1; t < p.parts; ++t) merge(m, s, stats[2 * t], stats[2 * t + 1]);
+    const float inv = 1.0f / s;
+#pragma unroll 4
+    for (uint32_t c = first + threadIdx.x; c < last; c += blockDim.x) {
+      f32x4 v = load(c);
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = fast_exp2(v[e] * sc * I_LOG2_E32 - m) * inv;
+      if constexpr (VEC) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(y + 4 * (size_t)c));
+      else y[c] = v[0];
+    }
+  }
+}
+

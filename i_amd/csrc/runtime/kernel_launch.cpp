@@ -492,8 +492,17 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   return launch(fn, (unsigned)rgrid, 1, 1, 256, &r, sizeof(r), stream);
 }
 
+// Into how many parts to cut each row of a softmax (1: do not): fewer rows than half the CUs, each of 2^17 columns
+// and more, which one workgroup per row would leave to a few CUs; parts of at least 2^15 columns, as many as give
+// every CU a workgroup.
+unsigned row_softmax_parts(size_t rows, size_t cols, int mode) {
+  if ((mode != 0 && mode != 4) || rows == 0 || rows > 128 || cols < (size_t(1) << 17)) return 1;
+  const size_t parts = std::min<size_t>(std::min<size_t>(256 / rows, cols >> 15), 64);
+  return parts < 2 ? 1u : (unsigned)parts;
+}
+
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode,
-                       LaunchNote* note, const float* scale_ptr, float scale) {
+                       LaunchNote* note, const float* scale_ptr, float scale, float* stats, unsigned parts) {
   if (rows == 0 || cols == 0) return {};
   if (!fits_u32(rows) || !fits_u32(cols)) return "row_softmax kernel: extent exceeds 32 bits";
   if (!x || !y) return "row_softmax kernel: null device pointer";
@@ -503,6 +512,22 @@ Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipSt
   SoftmaxParams p{x, y, (uint32_t)rows, (uint32_t)cols, scale_ptr, scale};
   hipFunction_t fn;
   const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+  if (parts > 1 && (mode == 0 || mode == 4)) {
+    // every row in parts over workgroups: the parts' (max, sum) pairs into `stats`, then a second launch that
+    // combines them and writes
+    if (!stats) return "row_softmax kernel: rows in parts need their temporary";
+    const size_t chunks = vec ? cols / 4 : cols;
+    p.part_chunks = (uint32_t)((chunks + parts - 1) / parts);
+    p.parts = (uint32_t)((chunks + p.part_chunks - 1) / p.part_chunks);
+    p.stats = stats;
+    if (rows * p.parts > kMaxGrid) return "row_softmax kernel: grid too large";
+    const std::string base = std::string("row_") + kOps[mode] + "_parts_";
+    if (note) *note = LaunchNote{base + "stats" + (vec ? "_v" : "") + " + " + base + "apply" + (vec ? "_v" : "") + " (rows in " + std::to_string(p.parts) + " parts)", 0, 0};
+    if (Err e = builtin_function((base + "stats" + (vec ? "_v" : "")).c_str(), &fn); !e.empty()) return e;
+    if (Err e = launch(fn, (unsigned)(rows * p.parts), 1, 1, 1024, &p, sizeof(p), stream); !e.empty()) return e;
+    if (Err e = builtin_function((base + "apply" + (vec ? "_v" : "")).c_str(), &fn); !e.empty()) return e;
+    return launch(fn, (unsigned)(rows * p.parts), 1, 1, 1024, &p, sizeof(p), stream);
+  }
   if (cols <= 128) {
     // G lanes per row, one float4 chunk each: 64 / G rows per wavefront
     size_t g = 1;

@@ -81,7 +81,11 @@ bool gemm_nt_f32_supported(size_t k);
 // 4: softmax of s * x with s = scale * (scale_ptr ? *scale_ptr : 1), scale_ptr a rank-0 f32 operand in device memory.
 // y may be x: every kernel has read a row's element before it writes it.
 Err launch_row_softmax(const float* x, float* y, size_t rows, size_t cols, hipStream_t stream, int mode = 0,
-                       LaunchNote* note = nullptr, const float* scale_ptr = nullptr, float scale = 1.0f);
+                       LaunchNote* note = nullptr, const float* scale_ptr = nullptr, float scale = 1.0f,
+                       float* stats = nullptr, unsigned parts = 1);
+// (parts > 1, softmax modes only: every row in that many parts over workgroups, two launches; `stats` is room for
+// 2 * rows * parts floats; row_softmax_parts says when it pays: fewer rows than half the CUs, 2^17 columns and more)
+unsigned row_softmax_parts(size_t rows, size_t cols, int mode);
 
 // dst[b][c][r] = src[b][r][c]; elem_bytes is 2 or 4.  An NN product that the direct kernels cannot read runs as transpose + NT kernel.
 Err launch_transpose(const void* src, void* dst, size_t bh, size_t rows, size_t cols, size_t elem_bytes,

@@ -50,7 +50,9 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert rec["pre_warmup_launches"] == 41 and rec["rel_err"] <= 2e-2
     assert rec["roofline"]["kernel"] == "attn_fwd_bf16_d128_bn64_direct_w8"
     second = rec["secondary"]
-    assert len(second) == 6
+    assert len(second) == 7
+    one_head = second[6]  # (one head on its own: its keys in parts over workgroups, beside the same call unsplit)
+    assert "(keys in " in one_head["launches"] and one_head["ms_per_call_unsplit"] > 0 and one_head["rel_err_against_unsplit"] <= 2e-3
     for entry, bar in zip(second, (1e-4, 1e-4, 2e-2, 2e-2, 1e-4, 1e-4)):
         assert entry["cpu_baseline"]["value"] > 0 and entry["rel_err"] <= bar, entry["workload"]
     f32_line = second[5]

@@ -623,6 +623,26 @@ def test_random_shapes_through_the_split_loops(torch, monkeypatch):
     assert split >= 25  # (m * n that is no multiple of 4 runs unsplit)
 
 
+def test_softmax_of_a_few_very_long_rows_runs_every_row_in_parts(torch):
+    """Fewer rows than half the CUs, 2^17 columns and more: every row in parts over workgroups (a first launch leaves
+    each part's running max and sum of exponentials, a second combines them and writes).  Aligned and unaligned
+    widths, one row and several, a row whose largest element sits in its last part, against float64; rows that are
+    many or short keep the one-workgroup-per-row kernels."""
+    sm = softmax_rowstaged()
+    for rows, cols in ((1, 1 << 20), (3, 1 << 17), (8, (1 << 18) + 3), (100, 200001), (5, 150000)):
+        g = torch.Generator(device="cuda").manual_seed(rows)
+        x = torch.randn(rows, cols, device="cuda", generator=g) * 3
+        x[0, cols - 7] = 40.0
+        y = sm.exec_torch(x)
+        assert "(rows in " in sm.report(), sm.report()
+        ref = torch.softmax(x.double(), -1)
+        assert float((y.double() - ref).abs().max()) <= RTOL_F32 * float(ref.abs().max())
+        assert float((y.double().sum(-1) - 1).abs().max()) <= 1e-4
+    for rows, cols in ((200, 1 << 17), (8, 70000)):
+        sm.exec_torch(torch.randn(rows, cols, device="cuda"))
+        assert "rows in" not in sm.report()
+
+
 def test_temporaries_are_kept_from_call_to_call_on_a_stream(torch):
     """Calls enqueued back to back on one stream carve their temporaries (here the two [rows, cols] intermediates
     of the naive softmax) from one block that the library keeps and replaces when a call needs more: operands that
