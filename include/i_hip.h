@@ -158,7 +158,9 @@ int i_hip_gemm_nt_f32(const float* a, const float* b, float* c,
  * Any cols: up to 65536 columns a row is read once and written once (it lives
  * in the registers of a group of lanes, a wavefront or a workgroup), wider
  * rows are read twice.  16-byte aligned operands with cols % 4 == 0 take the
- * float4 forms.
+ * float4 forms.  One launch with a workgroup (or less) per row, no temporaries:
+ * a few very long rows are cut into parts over workgroups only by programs run
+ * through i_exec*.
  */
 int i_hip_row_softmax(const float* x, float* y, size_t rows, size_t cols, void* stream);
 
