@@ -251,7 +251,8 @@ extern "C" __global__ void __launch_bounds__(256) splitk_reduce(SplitReduceParam
     const uint64_t b = at / quads, i = at - b * quads;
     const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)b * p.splits * p.count) + i;
     f32x4 sum = src[0];
-    for (uint32_t s = 1; s < p.splits; ++s) sum += src[(size_t)s * quads];
+#pragma unroll 8
+    for (uint32_t s = 1; s < p.splits; ++s) sum += src[(size_t)s * quads];  // (unrolled: eight loads in flight per lane)
     if (p.out_bf16) {
       bf16x4 v;
 #pragma unroll

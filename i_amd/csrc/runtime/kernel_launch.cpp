@@ -298,7 +298,7 @@ unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k) {
   // 256 x 256 tile, plus two slabs' worth before and after its loop; the chip holds 512 / 256 of them at a time;
   // the second launch costs 4 us and the pass over the partial products runs at 3 TB/s.  Examples (unsplit ->
   // split): 64 x 8192 x 8192 79 -> 30 us in 8 parts, 512 x 512 x 4096 52 -> 27 in 8, 256 x 4096 x 4096 41 -> 29
-  // in 8, 256 x 256 x 65536 812 -> 73 in 32; left whole: 1024^3 (10 us; 25 in 2 parts), 2048^3 (28; 40).
+  // in 8, 256 x 256 x 65536 576 -> 49 in 32; left whole: 1024^3 (10 us; 25 in 2 parts), 2048^3 (28; 40).
   if (k > (size_t(1) << 22)) return 1;
   const size_t slabs = (k + 63) / 64;
   const size_t t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh, t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
@@ -311,7 +311,7 @@ unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k) {
   best *= 0.85;  // a split has to gain at least 15 %
   const size_t tiles = tile == 256 ? t256 : t128;
   size_t splits = 1;
-  for (size_t s = 2; s <= 32 && k / s >= (s == 32 ? 2048u : 512u) && bh * s <= 65535; s *= 2) {
+  for (size_t s = 2; s <= 32 && k / s >= 512 && bh * s <= 65535; s *= 2) {
     const double t = time_of(tile, tiles * s, (slabs + s - 1) / s) + 4.0 + (double)(bh * s * m * n * 4) / 3e6;
     if (t < best) {
       best = t;
