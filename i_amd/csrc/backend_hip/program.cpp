@@ -221,6 +221,15 @@ DType product_dtype(const Run& run, const Recognized& r) {
   return run.dtype_of(r.a.buffer) == DType::BF16 && run.dtype_of(r.b.buffer) == DType::BF16 ? DType::BF16 : DType::F32;
 }
 
+// The arithmetic of an attention: bf16 when Q, K and V all are; with an f32 operand among them the f32 kernels run
+// and the bf16 operands are widened first (as for a product).
+DType attention_dtype(const Run& run, const Recognized& r) {
+  return run.dtype_of(r.a.buffer) == DType::BF16 && run.dtype_of(r.b.buffer) == DType::BF16 &&
+                 run.dtype_of(r.c.buffer) == DType::BF16
+             ? DType::BF16
+             : DType::F32;
+}
+
 bool hand_usable(const Run& run, const Recognized& r) {
   // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
   if (const char* v = std::getenv("ILANG_HIP_GENERATED_ONLY"))
@@ -229,8 +238,7 @@ bool hand_usable(const Run& run, const Recognized& r) {
   switch (r.kind) {
     case Recognized::None: return false;
     case Recognized::Attention: {
-      const DType t = run.dtype_of(r.a.buffer);
-      if (run.dtype_of(r.b.buffer) != t || run.dtype_of(r.c.buffer) != t) return false;
+      const DType t = attention_dtype(run, r);
       const auto q = rows_cols(r.a), v = rows_cols(r.c);
       if (q.size() < 2 || v.size() < 2) return false;
       if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back())) return true;
@@ -298,6 +306,24 @@ ihip::Err launch_product_f32(Run& run, const void* a, const void* b, void* c, si
                                   run.stream, note, static_cast<float*>(partial), splits);
 }
 
+// Q, K and V in the arithmetic type of the attention: as they are, or read as f32 (bf16 ones widened into temporaries).
+ihip::Err attention_operands(Run& run, const Recognized& r, bool bf16, const void** q, const void** k, const void** v) {
+  if (bf16) {
+    *q = run.raw_ptr(r.a.buffer);
+    *k = run.raw_ptr(r.b.buffer);
+    *v = run.raw_ptr(r.c.buffer);
+    return {};
+  }
+  void *pq = nullptr, *pk = nullptr, *pv = nullptr;
+  if (ihip::Err e = run.read_f32(r.a.buffer, &pq); !e.empty()) return e;
+  if (ihip::Err e = run.read_f32(r.b.buffer, &pk); !e.empty()) return e;
+  if (ihip::Err e = run.read_f32(r.c.buffer, &pv); !e.empty()) return e;
+  *q = pq;
+  *k = pk;
+  *v = pv;
+  return {};
+}
+
 ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
                              const float* scale_ptr, ihip::LaunchNote* note) {
   void* out = nullptr;
@@ -305,7 +331,8 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
   void* scores = nullptr;  // [bh, nq, nk] f32: S, then P in place
   if (ihip::Err e = run.alloc(&scores, bh * nq * nk * 4); !e.empty()) return e;
   float* s = static_cast<float*>(scores);
-  const void *q = run.raw_ptr(r.a.buffer), *k = run.raw_ptr(r.b.buffer), *v = run.raw_ptr(r.c.buffer);
+  const void *q = nullptr, *k = nullptr, *v = nullptr;
+  if (ihip::Err e = attention_operands(run, r, bf16, &q, &k, &v); !e.empty()) return e;
   ihip::LaunchNote first, middle, last;
   if (ihip::Err e = bf16 ? ihip::launch_gemm_nt_bf16(q, k, s, bh, nq, nk, d, run.stream, 0, 0, &first)
                          : ihip::launch_gemm_nt_f32(static_cast<const float*>(q), static_cast<const float*>(k), s, bh, nq, nk,
@@ -385,7 +412,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       for (size_t d = 0; d < nb; ++d)
         if (k[d] != q[d] || v[d] != q[d]) return "attention operands disagree on a batch extent";
       if (k[nb + 1] != dq || v[nb] != nk) return "attention operands disagree on a contracted extent";
-      const bool bf16 = run.dtype_of(r.a.buffer) == DType::BF16;
+      const bool bf16 = attention_dtype(run, r) == DType::BF16;
       const float* scale_ptr = nullptr;
       if (r.has_scale) {
         void* sp = nullptr;
@@ -414,7 +441,9 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
           options.partial_lse = static_cast<float*>(partial) + rows * dv;
         }
       }
-      return ihip::launch_attention(run.raw_ptr(r.a.buffer), run.raw_ptr(r.b.buffer), run.raw_ptr(r.c.buffer), out,
+      const void *pq = nullptr, *pk = nullptr, *pv = nullptr;
+      if (ihip::Err e = attention_operands(run, r, bf16, &pq, &pk, &pv); !e.empty()) return e;
+      return ihip::launch_attention(pq, pk, pv, out,
                                     bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream,
                                     options, note);
     }

@@ -643,6 +643,20 @@ def test_softmax_of_a_few_very_long_rows_runs_every_row_in_parts(torch):
         assert "rows in" not in sm.report()
 
 
+def test_attention_with_operands_of_both_types_runs_on_the_f32_kernels(torch):
+    """Q in bf16 against K and V in f32 (and the other way round): an f32 attention, the bf16 operands widened on the
+    device first, not a generated kernel; head sizes of the fused f32 kernel and of the three-kernel form."""
+    comp = flash(prefix="b", scaled=True)
+    for d, types in ((64, (torch.bfloat16, torch.float32, torch.float32)), (128, (torch.float32, torch.bfloat16, torch.bfloat16)),
+                     (160, (torch.bfloat16, torch.float32, torch.bfloat16))):
+        g = torch.Generator(device="cuda").manual_seed(d)
+        q, k, v = ((torch.randn(2, n, d, device="cuda", generator=g) * 0.5).to(t) for n, t in zip((200, 332, 332), types))
+        got = comp.exec_torch(q, k, torch.tensor(d ** -0.5, device="cuda"), v)
+        assert "generated" not in comp.report() and "f32" in comp.report(), comp.report()
+        ref = torch.softmax((q.double() @ k.double().transpose(1, 2)) * d ** -0.5, -1) @ v.double()
+        assert float((got.double() - ref).abs().max()) <= RTOL_F32 * float(ref.abs().max())
+
+
 def test_temporaries_are_kept_from_call_to_call_on_a_stream(torch):
     """Calls enqueued back to back on one stream carve their temporaries (here the two [rows, cols] intermediates
     of the naive softmax) from one block that the library keeps and replaces when a call needs more: operands that
