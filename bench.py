@@ -23,13 +23,21 @@ Prints ONE JSON line.  Besides the headline TFLOP/s it carries
 Operands follow the recipe of the reference's scripts (NumPy default_rng(seed),
 seeds 1, 2, 3 for the first, second, third operand; ilang-python/flash-attn.py:33-35).
 
+roofline.shader_clock_ghz is measured inside the timed region: the attention kernels count, per workgroup, the
+cycles of the shader clock (the frequency the power manager grants) and the ticks of the constant 100 MHz clock
+that pass while they are resident (i_hip_program_clock_probe); for kernels that cannot count for themselves
+(the vendor library's GEMM, mm_t) a one-wavefront kernel on a second stream reads the same two clocks while a
+second batch of launches runs (i_hip_shader_clock_probe; its own line, not the timed one, because the wavefront
+keeps one compute unit from taking a workgroup that needs all of it).  frac_at_measured_clock is the roofline
+fraction with the peak scaled to that clock (peak * clock / 2.4 GHz): the share of the matrix cores' cycles the
+kernel fills.
+
 roofline.traffic is the HBM traffic per launch measured with rocprofv3
 (FETCH_SIZE + WRITE_SIZE passes, scaled by a plain copy of known size); it is read
 from the committed summary under profiles/ and is null when that is missing.
 """
 import argparse
 import json
-import os
 import re
 import sys
 import time
@@ -88,7 +96,40 @@ def measured_traffic(summary):
     return (int(m.group(1)) + int(m.group(2))) * 2 ** 20 if m else None
 
 
-def time_steps(torch, fn, steps, warmup):
+def profile_cycles(kernel):
+    """Shader cycles per launch of `kernel` from the committed SQ-counter summary (GRBM_GUI_ACTIVE / 8), or None."""
+    try:
+        text = (ROOT / "profiles" / "sq_counters_bench_kernels.md").read_text()
+    except OSError:
+        return None
+    header = next((l for l in text.splitlines() if l.startswith("| figure |")), None)
+    row = next((l for l in text.splitlines() if l.startswith("| cycles per launch")), None)
+    if not header or not row:
+        return None
+    names = [c.strip() for c in header.strip("|").split("|")]
+    cells = [c.strip() for c in row.strip("|").split("|")]
+    return int(cells[names.index(kernel)]) if kernel in names else None
+
+
+NOMINAL_GHZ = 2.4  # the shader clock the published matrix-core peaks are quoted at
+
+
+def clock_fields(ghz, frac, kernel, kernel_ms):
+    """The roofline fields that make a power-limited reading checkable: the measured shader clock, the fraction of
+    the peak at that clock, and the kernel time that the committed profile's cycle count predicts at that clock."""
+    if not ghz:
+        return {"shader_clock_ghz": None, "frac_at_measured_clock": None}
+    out = {"shader_clock_ghz": ghz, "frac_at_measured_clock": frac * NOMINAL_GHZ / ghz,
+           "cycles_per_launch": kernel_ms * 1e-3 * ghz * 1e9}
+    cycles = profile_cycles(kernel)
+    if cycles:
+        out["cycles_per_launch_profile"] = cycles
+        out["kernel_ms_from_profile_cycles"] = cycles / (ghz * 1e9) * 1e3
+        out["kernel_ms_measured_over_predicted"] = kernel_ms / out["kernel_ms_from_profile_cycles"]
+    return out
+
+
+def time_steps(torch, fn, steps, warmup, before_timed=None):
     """Wall time per step over exactly `steps` calls, and the average launch duration from one pair of events
     on the launch stream around the timed region (the launches queue back to back on the stream).
 
@@ -103,6 +144,8 @@ def time_steps(torch, fn, steps, warmup):
     try:
         for _ in range(warmup):
             fn()
+        if before_timed:
+            before_timed()  # (enqueued work, e.g. clearing counters: ordered before the first timed launch)
         torch.cuda.synchronize()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
@@ -173,6 +216,7 @@ def main():
     import torch
 
     from i_amd import Component as i, I
+    from i_amd import _native as nat
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -208,7 +252,34 @@ def main():
     for _ in range(PRE_WARMUP_LAUNCHES - 1):
         attn.into(out, q, k, scale, v)
     torch.cuda.synchronize()
-    wall_ms, kernel_ms = time_steps(torch, lambda: attn.into(out, q, k, scale, v), args.steps, args.warmup)
+    # the kernel's own clock accounting, cleared after the warm-up: it covers exactly the timed launches
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    attn.clock_probe(ticks)
+    wall_ms, kernel_ms = time_steps(torch, lambda: attn.into(out, q, k, scale, v), args.steps, args.warmup, ticks.zero_)
+    attn.clock_probe(None)
+
+    def ghz_of(counters):
+        shader, constant = (int(x) for x in counters.tolist())
+        return shader / constant / 10.0 if constant > 0 else None
+
+    attn_ghz = ghz_of(ticks)
+    side = torch.cuda.Stream()
+
+    def clock_beside(fn, ms_per_call):
+        """The shader clock while `fn`'s launches run, read by a one-wavefront kernel on a second stream over the
+        middle of a batch of launches of its own (about 30 ms of them, never the timed ones)."""
+        n = max(20, int(30.0 / ms_per_call))
+        counters = torch.zeros(2, dtype=torch.int64, device=dev)
+        torch.cuda.synchronize()
+        for _ in range(n // 4):
+            fn()
+        nat.check(nat.core.i_hip_shader_clock_probe(counters.data_ptr(), int(n * ms_per_call * 1000 * 0.4), side.cuda_stream))
+        for _ in range(n - n // 4):
+            fn()
+        torch.cuda.synchronize()
+        return ghz_of(counters)
+
+    attn_ghz_beside = clock_beside(lambda: attn.into(out, q, k, scale, v), kernel_ms)
     attn_kernel = attn.report().split()[1]
     flop = 4.0 * B * H * N * N * D
     tflops = flop / (wall_ms * 1e-3) / 1e12
@@ -218,7 +289,10 @@ def main():
     # (every element 0.01): what the kernel does when the chip can hold its clock.  Reported beside the
     # headline, never as the headline; the gap between the two is power management, not scheduling.
     qc, kc, vc = (torch.full_like(q, 0.01) for _ in range(3))
-    _, const_ms = time_steps(torch, lambda: attn.into(out, qc, kc, scale, vc), max(args.steps // 2, 5), 2)
+    attn.clock_probe(ticks)
+    _, const_ms = time_steps(torch, lambda: attn.into(out, qc, kc, scale, vc), max(args.steps // 2, 5), 2, ticks.zero_)
+    attn.clock_probe(None)
+    const_ghz = ghz_of(ticks)
     del qc, kc, vc
     attn.into(out, q, k, scale, v)  # leave the seeded result in `out` for the parity check below
 
@@ -271,6 +345,7 @@ def main():
     mm_kernel = mm.report().split()[1]
     _, mm_ms = time_steps(torch, lambda: mm.into(c, a, b), short_steps, short_warmup)
     mm_tflops = 2.0 * M ** 3 / (mm_ms * 1e-3) / 1e12
+    mm_ghz = clock_beside(lambda: mm.into(c, a, b), mm_ms) if args.steps >= 20 else None
 
     # ------------------------------------------------------------------ long-sequence attention B1 H16 N32768 d64, x 2.0
     scale5 = torch.tensor(np.float32(1.0 / np.sqrt(D5)), dtype=torch.float32, device=dev)
@@ -278,8 +353,18 @@ def main():
     attn5 = flash_component(i, I, "i:512,j:32")  # 512 query rows per workgroup, 32-key LDS tiles: the d = 64 kernel
     attn5.into(out5, q5, k5, scale5, v5)
     c5_kernel = attn5.report().split()[1]
-    _, c5_ms = time_steps(torch, lambda: attn5.into(out5, q5, k5, scale5, v5), max(args.steps // 2, 5), 2)
+    attn5.clock_probe(ticks)
+    _, c5_ms = time_steps(torch, lambda: attn5.into(out5, q5, k5, scale5, v5), max(args.steps // 2, 5), 2, ticks.zero_)
+    attn5.clock_probe(None)
+    c5_ghz = ghz_of(ticks)
     c5_tflops = 4.0 * B5 * H5 * N5 * N5 * D5 / (c5_ms * 1e-3) / 1e12
+    # The second bound of this line: at d = 64 there are only 256 matrix-core FLOP per exponential.  Per pair of scores
+    # a lane's wave issues two v_exp_f32 (8 cycles each, a quarter of the vector rate), one v_cvt_pk_bf16_f32 and
+    # one v_dot2c_f32_bf16 (4 cycles each): 12 vector cycles per score and wave instruction of 64 lanes, on 1024
+    # SIMDs.  The matrix cores need 256 / 1024 = 0.25 cycles per score and lane, the vector pipe 12 / 64 = 0.1875.
+    c5_scores = float(B5 * H5) * N5 * N5
+    c5_valu_ms_nominal = c5_scores * 12.0 / 64.0 / 1024.0 / (NOMINAL_GHZ * 1e9) * 1e3
+    c5_mfma_ms_nominal = 4.0 * c5_scores * D5 / (PEAK_BF16_TFLOPS * 1e12) * 1e3
 
     # ------------------------------------------------------------------ the reference's own demo: attention f32 [512, 64]
     # (BASELINE configs[0]): no scale, i:16,j:16, through the f32 kernel.  Timed here, with the other GPU work and
@@ -304,13 +389,11 @@ def main():
     one_launches = attn_one.report().strip()
     _, one_ms = time_steps(torch, lambda: attn_one.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
     one_split = one_out.clone()
-    os.environ["ILANG_ATTN_KV_SPLITS"] = "1"
-    try:
-        attn_one.into(one_out, q1, k1, scale, v1)
-        one_err = float((one_split - one_out).abs().max() / one_out.abs().max())
-        _, one_whole_ms = time_steps(torch, lambda: attn_one.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
-    finally:
-        del os.environ["ILANG_ATTN_KV_SPLITS"]
+    attn_one.option("attention.kv_parts", 1)  # the same program with its key loops left whole
+    attn_one.into(one_out, q1, k1, scale, v1)
+    one_err = float((one_split - one_out).abs().max() / one_out.abs().max())
+    _, one_whole_ms = time_steps(torch, lambda: attn_one.into(one_out, q1, k1, scale, v1), short_steps, short_warmup)
+    attn_one.option("attention.kv_parts", 0)
     one_flop = 4.0 * (2 * N) * (2 * N) * D
 
     # ------------------------------------------------------------------ the attention workload in f32 (the reference's
@@ -327,11 +410,12 @@ def main():
     # on the same operands as the mm_t line: a practical ceiling for dense bf16 on random data on this box, next to
     # which the MFMA lines can be read.  Not part of the product path; the shader clock under dense MFMA work on
     # random operands stays well below the 2.4 GHz the 2.5 PFLOP/s peak is quoted at.
-    lib_ms = None
+    lib_ms = lib_ghz = None
     if args.steps >= 20:
         bt_ = b.t()
         torch.matmul(a, bt_)
         _, lib_ms = time_steps(torch, lambda: torch.matmul(a, bt_), short_steps, short_warmup)
+        lib_ghz = clock_beside(lambda: torch.matmul(a, bt_), lib_ms)
 
     if args.calibrate_copy:
         y.copy_(x)  # 256 MiB read + 256 MiB written
@@ -359,7 +443,7 @@ def main():
             oracle, sm, [wide_in], sm_bytes_of(64, wide_cols) / 1e9, "GB/s",
             f"rows 0..63 of {wide_rows} (algorithmic bytes of those rows)", wide_got)
         # C3: output tiles are independent; all of k
-        m3 = M if args.cpu_full else 1024
+        m3 = M if args.cpu_full else 2048  # (a quarter of the output: about 40 s; --cpu-full: all of it, four minutes)
         cpu3, err3 = emitted_c_baseline(
             oracle, mm, [a_host[:m3], b_host[:m3]], 2.0 * m3 * m3 * M / 1e12, "TFLOP/s",
             f"rows 0..{m3 - 1} of A against rows 0..{m3 - 1} of B, all {M} of k: 1/{(M // m3) ** 2} of the workload",
@@ -396,9 +480,12 @@ def main():
         else:
             cpu1, err1 = emitted_c_baseline(oracle, demo, demo_in, c1_flop / 1e12, "TFLOP/s", "the whole workload", got1, 5)
 
-    def roof(bound, achieved_, peak, unit, summary, kernel, ms):
-        return {"bound": bound, "achieved": achieved_, "peak": peak, "unit": unit, "frac": achieved_ / peak,
-                "traffic": measured_traffic(summary), "kernel": kernel, "kernel_ms": ms}
+    def roof(bound, achieved_, peak, unit, summary, kernel, ms, ghz=None):
+        fields = {"bound": bound, "achieved": achieved_, "peak": peak, "unit": unit, "frac": achieved_ / peak,
+                  "traffic": measured_traffic(summary), "kernel": kernel, "kernel_ms": ms}
+        if bound == "mfma":
+            fields.update(clock_fields(ghz, achieved_ / peak, kernel, ms))
+        return fields
 
     line = {
         "metric": "attn TFLOP/s & %MFMA peak (B8,H32,N4096,d128); row-softmax HBM GB/s",
@@ -409,18 +496,25 @@ def main():
         "config": {"workload": "flash_attention_fwd B8 H32 N4096 d128, bf16 in / f32 accumulate / f32 out, "
                                "1/sqrt(d) scale, non-causal (BASELINE configs[3]); compiled from 𝚒 component strings",
                    "schedule": "i:256,j:64 (256 query rows per workgroup, 64-key LDS tiles)", "entry": "i_exec_into_device"},
-        "roofline": roof("mfma", achieved, PEAK_BF16_TFLOPS, "TFLOP/s", "flash_attention_B8_H32_N4096_d128_bf16.md",
-                         attn_kernel, kernel_ms),
+        "roofline": dict(roof("mfma", achieved, PEAK_BF16_TFLOPS, "TFLOP/s", "flash_attention_B8_H32_N4096_d128_bf16.md",
+                              attn_kernel, kernel_ms, attn_ghz),
+                         shader_clock_source="counted by the kernel's own workgroups over the timed launches "
+                                             "(s_memtime / s_memrealtime, i_hip_program_clock_probe)",
+                         shader_clock_ghz_beside=attn_ghz_beside),
         "cpu_baseline": cpu, "rel_err": err4,
         "constant_operand_probe": {
             "workload": "the same launch with every element of Q, K, V equal to 0.01 (not the benchmark data)",
             "value": flop / (const_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": const_ms,
-            "frac_of_peak": flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+            "frac_of_peak": flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            **clock_fields(const_ghz, flop / (const_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, attn_kernel, const_ms)},
         "library_gemm_probe": None if lib_ms is None else {
             "workload": "torch.matmul (hipBLASLt) bf16 4096^3, bf16 out, on the operands of the mm_t line: the vendor "
                         "library's dense bf16 rate on this box, for reading the MFMA fractions against",
             "value": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel_ms": lib_ms,
-            "frac_of_peak": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+            "frac_of_peak": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "shader_clock_ghz": lib_ghz,
+            "frac_at_measured_clock": None if not lib_ghz else 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS * NOMINAL_GHZ / lib_ghz,
+            "shader_clock_source": "a one-wavefront kernel on a second stream beside a second batch of launches (i_hip_shader_clock_probe)"},
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
              "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),
@@ -432,14 +526,24 @@ def main():
              "roofline": roof("hbm", smw_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_2048x32768_f32.md", smw_kernel, smw_ms),
              "steps": short_steps, "warmup": short_warmup, "cpu_baseline": cpu2w, "rel_err": err2w},
             {"workload": "mm_t bf16 M=N=K=4096, f32 out (BASELINE configs[2])", "value": mm_tflops, "unit": "TFLOP/s",
-             "roofline": roof("mfma", mm_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_nt_4096x4096x4096_bf16.md", mm_kernel, mm_ms),
+             "roofline": roof("mfma", mm_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_nt_4096x4096x4096_bf16.md", mm_kernel, mm_ms, mm_ghz),
              "steps": short_steps, "warmup": short_warmup,
              "cpu_baseline": cpu3, "rel_err": err3},
             {"workload": "flash_attention_fwd B1 H16 N32768 d64, bf16 inputs x 2.0 (BASELINE configs[4])",
              "schedule": "i:512,j:32 (512 query rows per workgroup, 64 per wave; 32-key LDS tiles)",
              "value": c5_tflops, "unit": "TFLOP/s",
              "roofline": roof("mfma", c5_tflops, PEAK_BF16_TFLOPS, "TFLOP/s", "flash_attention_B1_H16_N32768_d64_bf16.md",
-                              c5_kernel, c5_ms),
+                              c5_kernel, c5_ms, c5_ghz),
+             "second_bound": {
+                 "what": "vector pipe: per pair of scores two v_exp_f32 (8 cycles), one v_cvt_pk_bf16_f32 and one "
+                         "v_dot2c_f32_bf16 (4 cycles each) per 64 lanes on 1024 SIMDs; the matrix cores need 0.25 cycles "
+                         "per score and lane at d = 64, the vector pipe 0.1875",
+                 "valu_ms_at_2.4GHz": c5_valu_ms_nominal, "mfma_ms_at_2.4GHz": c5_mfma_ms_nominal,
+                 "frac_of_valu_bound": c5_valu_ms_nominal / c5_ms,
+                 "frac_of_max_bound": max(c5_valu_ms_nominal, c5_mfma_ms_nominal) / c5_ms,
+                 "frac_of_max_bound_at_measured_clock": None if not c5_ghz else max(c5_valu_ms_nominal, c5_mfma_ms_nominal) / c5_ms * NOMINAL_GHZ / c5_ghz,
+                 "frac_of_sum_of_bounds_at_measured_clock": None if not c5_ghz else (c5_valu_ms_nominal + c5_mfma_ms_nominal) / c5_ms * NOMINAL_GHZ / c5_ghz,
+                 "binds": "mfma" if c5_mfma_ms_nominal >= c5_valu_ms_nominal else "valu"},
              "cpu_baseline": cpu5, "rel_err": err5},
             {"workload": "demo flash_attention f32 [512,64], no scale, i:16,j:16 (BASELINE configs[0])",
              "value": c1_flop / (c1_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "kernel": c1_kernel, "kernel_ms": c1_ms,

@@ -40,6 +40,15 @@ core.i_hip_attention.restype = ctypes.c_int
 core.i_hip_attention_ex.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, sz, sz, sz, sz, sz, ctypes.c_float, sz, sz,
                                     ctypes.c_int, vp]
 core.i_hip_attention_ex.restype = ctypes.c_int
+core.i_hip_attention_opt.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, sz, sz, sz, sz, sz, ctypes.c_float, sz, sz,
+                                     ctypes.c_char_p, vp]
+core.i_hip_attention_opt.restype = ctypes.c_int
+core.i_hip_gemm_opt.argtypes = [vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, sz, sz, sz, sz, ctypes.c_char_p, vp]
+core.i_hip_gemm_opt.restype = ctypes.c_int
+core.i_hip_program_clock_probe.argtypes = [vp, vp]
+core.i_hip_program_clock_probe.restype = ctypes.c_int
+core.i_hip_shader_clock_probe.argtypes = [vp, ctypes.c_uint, vp]
+core.i_hip_shader_clock_probe.restype = ctypes.c_int
 core.i_hip_program_option.argtypes = [vp, ctypes.c_char_p, ctypes.c_int]
 core.i_hip_program_option.restype = ctypes.c_int
 core.i_hip_program_report.argtypes = [vp]

@@ -84,6 +84,7 @@ struct Run {
   Arena* arena = nullptr;                    // when set (and locked by this call), temporaries come off it while they fit
   size_t arena_used = 0, arena_needed = 0;
   bool capturing = false;                    // the stream is being captured into a graph
+  ihip::KernelOptions knobs;                 // the program's options as they were when the call started
 
   size_t dim(DimRef<size_t> d) const { return inputs[d.buffer].shape[d.dim]; }
   size_t extent(const Extent<size_t>& e) const {
@@ -231,9 +232,8 @@ DType attention_dtype(const Run& run, const Recognized& r) {
 }
 
 bool hand_usable(const Run& run, const Recognized& r) {
-  // ILANG_HIP_GENERATED_ONLY=1 runs every kernel in its generated form (used to test that path)
-  if (const char* v = std::getenv("ILANG_HIP_GENERATED_ONLY"))
-    if (*v && *v != '0') return false;
+  // option generated.only = 1 runs every kernel in its generated form (used to test that path)
+  if (run.knobs.generated_only) return false;
   auto rows_cols = [&](const Operand& o) { return run.shape_of(o.buffer); };
   switch (r.kind) {
     case Recognized::None: return false;
@@ -241,7 +241,7 @@ bool hand_usable(const Run& run, const Recognized& r) {
       const DType t = attention_dtype(run, r);
       const auto q = rows_cols(r.a), v = rows_cols(r.c);
       if (q.size() < 2 || v.size() < 2) return false;
-      if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back())) return true;
+      if (ihip::attention_supported(t == DType::BF16 ? ihip::BF16 : ihip::F32, q.back(), v.back(), run.knobs)) return true;
       const auto k = rows_cols(r.b);
       if (k.size() < 2) return false;
       size_t bh = 1;
@@ -300,10 +300,10 @@ bool bf16_result_in_place(const Run& run, const Recognized& r) {
 ihip::Err launch_product_f32(Run& run, const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                              ihip::LaunchNote* note) {
   void* partial = nullptr;
-  unsigned splits = ihip::gemm_nt_f32_split_k(bh, m, n, k);
+  unsigned splits = ihip::gemm_nt_f32_split_k(bh, m, n, k, run.knobs);
   if (splits > 1 && ((m * n) % 4 != 0 || !run.alloc_optional(&partial, bh * splits * m * n * 4))) splits = 1;
   return ihip::launch_gemm_nt_f32(static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(c), bh, m, n, k,
-                                  run.stream, note, static_cast<float*>(partial), splits);
+                                  run.stream, note, static_cast<float*>(partial), splits, run.knobs);
 }
 
 // Q, K and V in the arithmetic type of the attention: as they are, or read as f32 (bf16 ones widened into temporaries).
@@ -324,6 +324,17 @@ ihip::Err attention_operands(Run& run, const Recognized& r, bool bf16, const voi
   return {};
 }
 
+// An operand that a kernel moving 16 bytes per lane cannot read where it lies (a view that starts off a 16-byte
+// boundary): copied, element by element, into a temporary that it can.
+ihip::Err aligned_copy(Run& run, const void** ptr, size_t bytes, size_t elem_bytes) {
+  if (reinterpret_cast<uintptr_t>(*ptr) % 16 == 0 || bytes == 0) return {};
+  void* tmp = nullptr;
+  if (ihip::Err e = run.alloc(&tmp, bytes); !e.empty()) return e;
+  if (ihip::Err e = ihip::launch_pad_rows(*ptr, tmp, 1, bytes / elem_bytes, bytes / elem_bytes, elem_bytes, run.stream); !e.empty()) return e;
+  *ptr = tmp;
+  return {};
+}
+
 ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
                              const float* scale_ptr, ihip::LaunchNote* note) {
   void* out = nullptr;
@@ -334,9 +345,13 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
   const void *q = nullptr, *k = nullptr, *v = nullptr;
   if (ihip::Err e = attention_operands(run, r, bf16, &q, &k, &v); !e.empty()) return e;
   ihip::LaunchNote first, middle, last;
-  if (ihip::Err e = bf16 ? ihip::launch_gemm_nt_bf16(q, k, s, bh, nq, nk, d, run.stream, 0, 0, &first)
+  // (operands the kernels cannot read where they lie, for their alignment: aligned copies)
+  if (ihip::Err e = aligned_copy(run, &q, bh * nq * d * (bf16 ? 2 : 4), bf16 ? 2 : 4); !e.empty()) return e;
+  if (ihip::Err e = aligned_copy(run, &k, bh * nk * d * (bf16 ? 2 : 4), bf16 ? 2 : 4); !e.empty()) return e;
+  if (ihip::Err e = aligned_copy(run, &v, bh * nk * dv * (bf16 ? 2 : 4), bf16 ? 2 : 4); !e.empty()) return e;
+  if (ihip::Err e = bf16 ? ihip::launch_gemm_nt_bf16(q, k, s, bh, nq, nk, d, run.stream, 0, 0, &first, ihip::F32, run.knobs)
                          : ihip::launch_gemm_nt_f32(static_cast<const float*>(q), static_cast<const float*>(k), s, bh, nq, nk,
-                                                    d, run.stream, &first);
+                                                    d, run.stream, &first, nullptr, 1, run.knobs);
       !e.empty())
     return e;
   if (ihip::Err e = ihip::launch_row_softmax(s, s, bh * nq, nk, run.stream, 4, &middle, scale_ptr, 1.0f); !e.empty()) return e;
@@ -344,15 +359,17 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
     void* pb = nullptr;  // the probabilities rounded to bf16, as the fused kernels round them
     if (ihip::Err e = run.alloc(&pb, bh * nq * nk * 2); !e.empty()) return e;
     if (ihip::Err e = ihip::launch_convert(s, pb, ihip::F32, ihip::BF16, bh * nq * nk, run.stream); !e.empty()) return e;
-    if (ihip::gemm_nn_bf16_supported(bh, nq, dv, nk)) {
-      if (ihip::Err e = ihip::launch_gemm_nn_bf16(pb, v, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last);
+    if (ihip::gemm_nn_bf16_supported(bh, nq, dv, nk, run.knobs)) {
+      if (ihip::Err e = ihip::launch_gemm_nn_bf16(pb, v, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last, ihip::F32,
+                                                  nullptr, 1, run.knobs);
           !e.empty())
         return e;
     } else {
       void* vt = nullptr;
       if (ihip::Err e = run.alloc(&vt, bh * dv * nk * 2); !e.empty()) return e;
       if (ihip::Err e = ihip::launch_transpose(v, vt, bh, nk, dv, 2, run.stream); !e.empty()) return e;
-      if (ihip::Err e = ihip::launch_gemm_nt_bf16(pb, vt, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last);
+      if (ihip::Err e = ihip::launch_gemm_nt_bf16(pb, vt, static_cast<float*>(out), bh, nq, dv, nk, run.stream, 0, 0, &last, ihip::F32,
+                                                  run.knobs);
           !e.empty())
         return e;
     }
@@ -367,12 +384,12 @@ ihip::Err attention_in_parts(Run& run, const Recognized& r, bool bf16, size_t bh
 }
 
 // The two operands of an NT product ([rows_a, k] and [rows_b, k], dense) as the matrix-instruction kernels can
-// read them: untouched when k is a multiple of their quantum (and, for f32, both are 16-byte aligned), otherwise
+// read them: untouched when k is a multiple of their quantum and both are 16-byte aligned, otherwise
 // copied into stream-ordered temporaries with every row padded with zeros up to the next multiple; *k becomes the
 // padded extent.
 ihip::Err padded_operands(Run& run, DType t, const void** a, size_t rows_a, const void** b, size_t rows_b, size_t* k) {
   const size_t q = product_k_quantum(t), kp = (*k + q - 1) / q * q, elem = t == DType::BF16 ? 2 : 4;
-  const bool misaligned = t == DType::F32 && (reinterpret_cast<uintptr_t>(*a) % 16 != 0 || reinterpret_cast<uintptr_t>(*b) % 16 != 0);
+  const bool misaligned = reinterpret_cast<uintptr_t>(*a) % 16 != 0 || reinterpret_cast<uintptr_t>(*b) % 16 != 0;
   if (kp == *k && !misaligned) return {};
   void *ta = nullptr, *tb = nullptr;
   if (ihip::Err e = run.alloc(&ta, std::max<size_t>(rows_a * kp * elem, 16)); !e.empty()) return e;
@@ -419,7 +436,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
         if (ihip::Err e = run.read_f32(r.scale.buffer, &sp); !e.empty()) return e;
         scale_ptr = static_cast<const float*>(sp);
       }
-      if (!ihip::attention_supported(bf16 ? ihip::BF16 : ihip::F32, dq, dv))
+      if (!ihip::attention_supported(bf16 ? ihip::BF16 : ihip::F32, dq, dv, run.knobs))
         return attention_in_parts(run, r, bf16, bh, nq, nk, dq, dv, scale_ptr, note);
       void* out = nullptr;
       ihip::DType out_dt = ihip::F32;
@@ -429,7 +446,15 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       } else if (ihip::Err e = run.write_f32(r.out, &out); !e.empty()) {
         return e;
       }
-      ihip::AttentionOptions options{r.tile_i, r.tile_j, run.p.attention_f32_scale.load()};
+      // an output view that the bf16 kernels cannot store to where it lies (they store 8 or 16 bytes per lane): the
+      // result goes to an aligned temporary and is copied out, element by element, after the launch
+      void* out_view = nullptr;
+      const size_t out_elem = out_dt == ihip::BF16 ? 2 : 4;
+      if (bf16 && reinterpret_cast<uintptr_t>(out) % (out_dt == ihip::BF16 ? 8 : 16) != 0) {
+        out_view = out;
+        if (ihip::Err e = run.alloc(&out, bh * nq * dv * out_elem); !e.empty()) return e;
+      }
+      ihip::AttentionOptions options{r.tile_i, r.tile_j, run.knobs};
       // few workgroups under a long key loop (a single head, a few long sequences): the keys of a head in parts
       // over workgroups, each part's result in a temporary (no room for it: the unsplit kernel)
       if (const unsigned splits = ihip::attention_kv_splits(bf16 ? ihip::BF16 : ihip::F32, bh, nq, nk, dq, dv, options); splits > 1) {
@@ -443,9 +468,16 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       }
       const void *pq = nullptr, *pk = nullptr, *pv = nullptr;
       if (ihip::Err e = attention_operands(run, r, bf16, &pq, &pk, &pv); !e.empty()) return e;
-      return ihip::launch_attention(pq, pk, pv, out,
-                                    bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr, 1.0f, run.stream,
-                                    options, note);
+      if (bf16) {  // (f32 operands off a 16-byte boundary take the register-staged f32 kernel, which reads element by element)
+        if (ihip::Err e = aligned_copy(run, &pq, bh * nq * dq * 2, 2); !e.empty()) return e;
+        if (ihip::Err e = aligned_copy(run, &pk, bh * nk * dq * 2, 2); !e.empty()) return e;
+        if (ihip::Err e = aligned_copy(run, &pv, bh * nk * dv * 2, 2); !e.empty()) return e;
+      }
+      if (ihip::Err e = ihip::launch_attention(pq, pk, pv, out, bf16 ? ihip::BF16 : ihip::F32, out_dt, bh, nq, nk, dq, dv, scale_ptr,
+                                               1.0f, run.stream, options, note);
+          !e.empty() || !out_view)
+        return e;
+      return ihip::launch_pad_rows(out, out_view, 1, bh * nq * dv, bh * nq * dv, out_elem, run.stream);
     }
     case Recognized::GemmNT: {
       const auto a = run.shape_of(r.a.buffer), b = run.shape_of(r.b.buffer);
@@ -473,14 +505,14 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       // few output tiles under a long k loop: the loop is split over workgroups, partial products in a temporary
       // (unless the schedule names one of the kernels' own tiles: then that kernel runs as asked)
       const bool tile_asked = (r.tile_i == 128 && r.tile_j == 128) || (r.tile_i == 256 && r.tile_j == 256);
-      if (const unsigned splits = tile_asked ? 1u : ihip::gemm_nt_bf16_split_k(bh, a[nb], b[nb], k);
+      if (const unsigned splits = tile_asked && run.knobs.gemm_k_parts < 2 ? 1u : ihip::gemm_nt_bf16_split_k(bh, a[nb], b[nb], k, run.knobs);
           splits > 1 && (a[nb] * b[nb]) % 4 == 0) {
         void* partial = nullptr;
         if (run.alloc_optional(&partial, bh * splits * a[nb] * b[nb] * 4))  // (no room for it: the unsplit kernel)
           return ihip::launch_gemm_nt_bf16_split_k(pa, pb, out, static_cast<float*>(partial), splits, bh, a[nb], b[nb], k, run.stream,
                                                    note, out_dt);
       }
-      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, a[nb], b[nb], k, run.stream, r.tile_i, r.tile_j, note, out_dt);
+      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, a[nb], b[nb], k, run.stream, r.tile_i, r.tile_j, note, out_dt, run.knobs);
     }
     case Recognized::GemmNN: {
       // b [B.., K, J]: the direct bf16 kernels read it in place; otherwise it is transposed into a stream-ordered
@@ -505,13 +537,14 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       }
       const void *pa = nullptr, *pb_rows = nullptr;
       if (ihip::Err e = product_operands(run, r, f32 ? DType::F32 : DType::BF16, &pa, &pb_rows); !e.empty()) return e;
-      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k)) {  // the direct kernels read a row-major right operand themselves
+      if (!f32 && ihip::gemm_nn_bf16_supported(bh, m, n, k, run.knobs) && reinterpret_cast<uintptr_t>(pa) % 16 == 0 &&
+          reinterpret_cast<uintptr_t>(pb_rows) % 16 == 0) {  // the direct kernels read a row-major right operand themselves
         const bool tile_asked = (r.tile_i == 128 && r.tile_j == 128) || (r.tile_i == 256 && r.tile_j == 256);
-        unsigned splits = tile_asked ? 1u : ihip::gemm_nt_bf16_split_k(bh, m, n, k);
+        unsigned splits = tile_asked && run.knobs.gemm_k_parts < 2 ? 1u : ihip::gemm_nt_bf16_split_k(bh, m, n, k, run.knobs);
         void* partial = nullptr;
         if (splits > 1 && ((m * n) % 4 != 0 || !run.alloc_optional(&partial, bh * splits * m * n * 4))) splits = 1;
         return ihip::launch_gemm_nn_bf16(pa, pb_rows, out, bh, m, n, k, run.stream, r.tile_i, r.tile_j, note, out_dt,
-                                         static_cast<float*>(partial), splits);
+                                         static_cast<float*>(partial), splits, run.knobs);
       }
       const size_t elem = f32 ? 4 : 2;
       void* bt = nullptr;
@@ -521,7 +554,7 @@ ihip::Err launch_hand_noted(Run& run, const Recognized& r, ihip::LaunchNote* not
       size_t kp = k;
       if (ihip::Err e = padded_operands(run, f32 ? DType::F32 : DType::BF16, &pa, bh * m, &pb, bh * n, &kp); !e.empty()) return e;
       if (f32) return launch_product_f32(run, pa, pb, out, bh, m, n, kp, note);
-      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, m, n, kp, run.stream, r.tile_i, r.tile_j, note, out_dt);
+      return ihip::launch_gemm_nt_bf16(pa, pb, out, bh, m, n, kp, run.stream, r.tile_i, r.tile_j, note, out_dt, run.knobs);
     }
     case Recognized::RowSoftmax:
     case Recognized::RowMaxShift:
@@ -641,13 +674,13 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
     if (total == 0) continue;
     // The wavefront-per-iteration form (reduction loops spread over 64 lanes), when the nest has one: taken when
     // the reduction is long enough to occupy the lanes and either consecutive lanes read consecutive elements
-    // or there are too few iterations to fill the chip with one work-item each.  ILANG_HIP_WAVE=0|1 overrides.
+    // or there are too few iterations to fill the chip with one work-item each.  Option generated.wave = 0 | 1 overrides.
     if (!ph.wave_loops.empty()) {
       const auto& e = ph.wave_extent;
       const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
       const size_t reduced = run.extent(Extent<size_t>{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind});
       bool wave = reduced >= 128 && (ph.wave_contiguous || total < 65536);
-      if (const char* force = std::getenv("ILANG_HIP_WAVE")) wave = force[0] == '1';
+      if (run.knobs.generated_wave >= 0) wave = run.knobs.generated_wave == 1;
       if (wave) {
         const size_t waves = std::min<size_t>(total, size_t(1) << 16);
         const unsigned per_group = GenericPhase::kWaveThreads / 64;
@@ -860,6 +893,10 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
   }
   if (outputs.size() != plan.count) return "wrong output count";
   Run run{p, plan, inputs, outputs, stream, {}, std::vector<void*>(plan.intermediates.size(), nullptr), {}, {}, workspace};
+  {
+    std::lock_guard<std::mutex> lock(p.mu);
+    run.knobs = p.options;
+  }
   for (size_t o = 0; o < outputs.size(); ++o) {
     const auto want = run.shape_of({BufferRef::Output, o});
     if (!outputs[o].shape.empty() && outputs[o].shape != want) return "output " + std::to_string(o) + " has the wrong shape";
@@ -938,11 +975,15 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
 }
 
 std::string set_option(Program& p, const std::string& name, int value) {
-  if (name == "attention.f32_scale") {
-    p.attention_f32_scale.store(value != 0);
-    return {};
-  }
-  return "unknown program option '" + name + "' (known: attention.f32_scale)";
+  std::lock_guard<std::mutex> lock(p.mu);
+  return ihip::set_kernel_option(p.options, name, value);
+}
+
+std::string set_clock_probe(Program& p, void* ticks) {
+  if (reinterpret_cast<uintptr_t>(ticks) % 8 != 0) return "clock probe: the counters must be 8-byte aligned";
+  std::lock_guard<std::mutex> lock(p.mu);
+  p.options.clock_ticks = static_cast<unsigned long long*>(ticks);
+  return {};
 }
 
 std::string last_report(Program& p) {

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "../compiler/ir.h"
+#include "../runtime/kernel_launch.h"
 #include "emit_hip.h"
 #include "recognize.h"
 
@@ -39,8 +40,9 @@ struct Program {
   bool image_built = false;
   std::mutex mu;
   std::map<int, hipModule_t> modules;  // per device
-  // options (set_option): apply the attention score scale in f32 to every score instead of folding it into Q
-  std::atomic<bool> attention_f32_scale{false};
+  // what set_option / set_clock_probe have stored (kernel choices that the caller takes from the launchers, and where
+  // the attention kernels count their clocks); guarded by mu, copied by every execute() when it starts
+  ihip::KernelOptions options;
   // what the last execute() dispatched: one line per kernel, "f<k>: <kernel name> (tile ...)"; guarded by mu
   std::string last_report;
 
@@ -78,8 +80,11 @@ struct Workspace {
 std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
                     hipStream_t stream, Workspace* workspace = nullptr);
 
-// Program options by name; returns "" or the failure text.  Known: "attention.f32_scale" (0 / 1).
+// Program options by name (ihip::set_kernel_option lists them); returns "" or the failure text.
 std::string set_option(Program& p, const std::string& name, int value);
+// Device memory for two 64-bit counters (or nullptr: off) to which the program's bf16 direct-to-LDS attention kernels
+// add the time their workgroups were resident, on the shader clock and on the constant 100 MHz clock.
+std::string set_clock_probe(Program& p, void* ticks);
 // The kernels the last execute() of this program dispatched, one per line.
 std::string last_report(Program& p);
 

@@ -468,6 +468,12 @@ int i_hip_program_option(i_program* program, const char* name, int value) {
   return err.empty() ? 0 : fail(err);
 }
 
+int i_hip_program_clock_probe(i_program* program, void* ticks) {
+  if (!program) return fail("null program");
+  const std::string err = ihipc::set_clock_probe(*program->inner, ticks);
+  return err.empty() ? 0 : fail(err);
+}
+
 char* i_hip_program_report(const i_program* program) {
   if (!program) {
     icore::set_error("null program");

@@ -45,6 +45,7 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
   uint32_t head, qt;
   xcd_map(blockIdx.x, p.nqt, p.bh, head, qt);
   if (head >= p.bh) return;
+  clock_note(p.clock, false);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -589,4 +590,5 @@ __device__ __forceinline__ void attn_fwd_bf16_q64_body(const AttnParams& p) {
       }
     }
   }
+  clock_note(p.clock, true);
 }

@@ -124,6 +124,18 @@ __device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t 
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// The two device clocks: the shader clock (s_memtime: it follows the frequency the power manager grants) and the
+// constant 100 MHz clock (s_memrealtime).  A workgroup that is asked to (clock != nullptr) subtracts both readings
+// from clock[0] and clock[1] when it starts and adds them when it ends (unsigned arithmetic: the sums come out as
+// the time the workgroups were resident on either clock); nothing is held in registers in between.
+__device__ __forceinline__ void clock_note(unsigned long long* clock, bool leaving) {
+  if (clock && threadIdx.x == 0) {
+    const unsigned long long shader = __builtin_amdgcn_s_memtime(), constant = __builtin_amdgcn_s_memrealtime();
+    atomicAdd(clock, leaving ? shader : 0ull - shader);
+    atomicAdd(clock + 1, leaving ? constant : 0ull - constant);
+  }
+}
+
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }

@@ -313,6 +313,22 @@ __device__ __forceinline__ void pad_rows_body(const PadParams& p) {
 extern "C" __global__ void __launch_bounds__(256) pad_rows_b16(PadParams p) { pad_rows_body<uint16_t>(p); }
 extern "C" __global__ void __launch_bounds__(256) pad_rows_b32(PadParams p) { pad_rows_body<uint32_t>(p); }
 
+// see ClockProbeParams
+extern "C" __global__ void __launch_bounds__(64) shader_clock_probe(ClockProbeParams p) {
+  const uint64_t shader0 = __builtin_amdgcn_s_memtime(), constant0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t constant1 = constant0;
+  // (the loop ends on the constant clock, and after a bounded number of sleeps whatever that clock reads)
+  for (uint32_t n = 0; n < (1u << 22) && constant1 - constant0 < p.ticks; ++n) {
+    __builtin_amdgcn_s_sleep(64);
+    constant1 = __builtin_amdgcn_s_memrealtime();
+  }
+  const uint64_t shader1 = __builtin_amdgcn_s_memtime();
+  if (threadIdx.x == 0) {
+    atomicAdd(p.out, (unsigned long long)(shader1 - shader0));
+    atomicAdd(p.out + 1, (unsigned long long)(constant1 - constant0));
+  }
+}
+
 extern "C" __global__ void __launch_bounds__(256) transpose_b16(TransposeParams p) { transpose_body<uint16_t>(p); }
 extern "C" __global__ void __launch_bounds__(256) transpose_b32(TransposeParams p) { transpose_body<uint32_t>(p); }
 

@@ -23,6 +23,19 @@ struct AttnParams {
   uint32_t kv_splits;
   uint32_t kv_chunk;  // a multiple of 64
   float* lse;
+  // Optional (the bf16 direct-to-LDS kernels): two 64-bit counters to which every workgroup adds what its first wave
+  // saw pass between entry and exit on the shader clock (s_memtime, which follows the clock the power manager
+  // grants) and on the constant 100 MHz clock (s_memrealtime).  clock[0] / clock[1] * 0.1 is the average shader
+  // clock in GHz over the launch, weighted by the time the workgroups were resident.
+  unsigned long long* clock;
+};
+
+// One wavefront that reads both clocks, sleeps until `ticks` of the 100 MHz clock have passed, reads them again and
+// adds the differences to out[0] (shader clock) and out[1] (100 MHz clock): the shader clock under whatever else
+// the GPU runs meanwhile, for kernels that cannot count for themselves.
+struct ClockProbeParams {
+  unsigned long long* out;
+  uint32_t ticks;  // of 10 ns; the host bounds it to two seconds
 };
 
 // out[b][r][:] = sum_s w_s partial[b * splits + s][r][:],  w_s = 2^lse[b * splits + s][r] / sum_t 2^lse[b * splits + t][r]

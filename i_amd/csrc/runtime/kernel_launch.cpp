@@ -2,6 +2,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <initializer_list>
 #include <cstdint>
 #include <string>
 
@@ -12,13 +13,87 @@ namespace {
 constexpr size_t kMaxGrid = 0x7fffffffu;
 
 bool fits_u32(size_t v) { return v <= 0xffffffffull; }
+bool aligned16(const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; }
 }  // namespace
 
-bool attention_supported(DType in_dtype, size_t d, size_t dv) {
+Err set_kernel_option(KernelOptions& o, const std::string& name, int value) {
+  auto one_of = [&](std::initializer_list<int> allowed) {
+    for (int a : allowed)
+      if (a == value) return true;
+    return false;
+  };
+  auto bad = [&](const char* allowed) { return "program option '" + name + "' must be " + allowed + ", not " + std::to_string(value); };
+  if (name == "attention.f32_scale") {
+    o.attention_f32_scale = value != 0;
+  } else if (name == "attention.kv_parts") {
+    if (value < 0) return bad("0 (the launcher decides), 1 (never) or a number of parts");
+    o.attention_kv_parts = value;
+  } else if (name == "attention.waves") {
+    if (!one_of({0, 2, 4, 8, 64})) return bad("0, 2, 4 or 8 (or 64: the 64-queries-per-wave kernel for d = 64)");
+    o.attention_waves = value;
+  } else if (name == "attention.direct") {
+    o.attention_direct = value != 0;
+  } else if (name == "gemm.k_parts") {
+    if (value < 0) return bad("0 (the launcher decides), 1 (never) or a number of parts");
+    o.gemm_k_parts = value;
+  } else if (name == "gemm.waves") {
+    if (!one_of({0, 4, 8})) return bad("0, 4 or 8");
+    o.gemm_waves = value;
+  } else if (name == "gemm.tile") {
+    if (!one_of({0, 128, 256})) return bad("0, 128 or 256");
+    o.gemm_tile = value;
+  } else if (name == "gemm.direct") {
+    o.gemm_direct = value != 0;
+  } else if (name == "generated.only") {
+    o.generated_only = value != 0;
+  } else if (name == "generated.wave") {
+    if (!one_of({-1, 0, 1})) return bad("-1 (the launcher decides), 0 or 1");
+    o.generated_wave = value;
+  } else {
+    return "unknown program option '" + name +
+           "' (known: attention.f32_scale, attention.kv_parts, attention.waves, attention.direct, gemm.k_parts, gemm.waves, "
+           "gemm.tile, gemm.direct, generated.only, generated.wave)";
+  }
+  return {};
+}
+
+Err parse_kernel_options(const char* text, KernelOptions* options) {
+  if (!text) return {};
+  const std::string all(text);
+  size_t at = 0;
+  auto separator = [](char c) { return c == ' ' || c == ',' || c == ';' || c == '\t' || c == '\n'; };
+  while (at < all.size()) {
+    while (at < all.size() && separator(all[at])) ++at;
+    size_t end = at;
+    while (end < all.size() && !separator(all[end])) ++end;
+    if (end == at) break;
+    const std::string pair = all.substr(at, end - at);
+    at = end;
+    const size_t eq = pair.find('=');
+    if (eq == std::string::npos || eq == 0 || eq + 1 == pair.size()) return "option '" + pair + "' is not of the form name=value";
+    char* tail = nullptr;
+    const long value = std::strtol(pair.c_str() + eq + 1, &tail, 10);
+    if (*tail != '\0') return "option '" + pair + "' has no integer value";
+    if (Err e = set_kernel_option(*options, pair.substr(0, eq), (int)value); !e.empty()) return e;
+  }
+  return {};
+}
+
+Err launch_shader_clock_probe(unsigned long long* ticks, unsigned microseconds, hipStream_t stream) {
+  if (!ticks) return "clock probe: null device pointer";
+  if (reinterpret_cast<uintptr_t>(ticks) % 8 != 0) return "clock probe: the counters must be 8-byte aligned";
+  if (microseconds > 2000000u) return "clock probe: at most two seconds";
+  ClockProbeParams p{ticks, microseconds * 100u};
+  hipFunction_t fn;
+  if (Err e = builtin_function("shader_clock_probe", &fn); !e.empty()) return e;
+  return launch(fn, 1, 1, 1, 64, &p, sizeof(p), stream);
+}
+
+bool attention_supported(DType in_dtype, size_t d, size_t dv, const KernelOptions& knobs) {
   if (d == 0 || dv == 0) return false;
   // head sizes above 128 up to 256: bf16, on the direct kernels only
   if (d > 128 || dv > 128)
-    return in_dtype == BF16 && d <= 256 && dv <= 256 && d % 8 == 0 && dv % 8 == 0 && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+    return in_dtype == BF16 && d <= 256 && dv <= 256 && d % 8 == 0 && dv % 8 == 0 && knobs.attention_direct;
   if (in_dtype == BF16) return d % 8 == 0 && dv % 8 == 0;
   return true;
 }
@@ -26,7 +101,8 @@ bool attention_supported(DType in_dtype, size_t d, size_t dv) {
 Err launch_attention(const void* q, const void* k, const void* v, void* o, DType in_dtype, DType out_dtype, size_t bh,
                      size_t nq, size_t nk, size_t d, size_t dv, const float* scale_ptr, float scale, hipStream_t stream,
                      const AttentionOptions& options, LaunchNote* note) {
-  if (!attention_supported(in_dtype, d, dv))
+  const KernelOptions& knobs = options.knobs;
+  if (!attention_supported(in_dtype, d, dv, knobs))
     return "attention kernel: unsupported operands (need 0 < d, dv <= 128, or bf16 with d, dv <= 256; bf16 needs d, dv % 8 == 0)";
   if ((d > 128 || dv > 128) && nk * (d > dv ? d : dv) * 2 >= (size_t(1) << 32))
     return "attention kernel: too many keys for a head size above 128";
@@ -36,6 +112,9 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   if (nk == 0) return "attention kernel: no keys";
   if (!fits_u32(bh) || !fits_u32(nq) || !fits_u32(nk)) return "attention kernel: extent exceeds 32 bits";
   if (!q || !k || !v || !o) return "attention kernel: null device pointer";
+  // every bf16 kernel moves 16 bytes per lane (the direct ones straight into LDS) and stores 8 (bf16) or 16 (f32)
+  if (in_dtype == BF16 && (!aligned16(q) || !aligned16(k) || !aligned16(v) || reinterpret_cast<uintptr_t>(o) % (out_dtype == BF16 ? 8 : 16) != 0))
+    return "attention kernel: bf16 operands must be 16-byte aligned (the output 8-byte for bf16, 16-byte for f32)";
 
   const size_t dmax = d > dv ? d : dv;
   const size_t query_tile = options.query_tile, key_tile = options.key_tile;
@@ -50,18 +129,19 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   //     rows padded to 64 or 128 columns (the larger of d and dv decides).
   //   d or dv above 128 up to 256 (multiples of 8): the kernel for 256-column rows (padded below 256), 4 waves, one
   //     per SIMD, 32-key tiles; nothing else exists above 128, so callers ask attention_supported() first.
-  //   otherwise (ILANG_ATTN_NO_DIRECT=1, key offsets beyond 32 bits): register-staged kernel with guarded columns
-  //     (always multiplies the scores in f32)
-  // ILANG_ATTN_WAVES=2|4|8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave kernel,
-  // d == 64 only) and ILANG_ATTN_NO_DIRECT=1 forces the register-staged kernel; both exist so that tests can
-  // reach every kernel with small inputs.
+  //   otherwise (knobs.attention_direct == 0, key offsets beyond 32 bits): register-staged kernel with guarded
+  //     columns (always multiplies the scores in f32)
+  // knobs.attention_waves = 2 | 4 | 8 forces the workgroup size of the direct kernel (64: the 64-queries-per-wave
+  // kernel, d == 64 only) and knobs.attention_direct = 0 the register-staged kernel; both exist so that tests and
+  // searches can reach every kernel with small inputs.
   unsigned bm = 128, bn = 64;
   bool q64 = false;
   const bool exact = in_dtype == BF16 && d == dv && (d == 64 || d == 128);
   const bool wide = in_dtype == BF16 && dmax > 128;  // (supported: d, dv <= 256, multiples of 8)
   const bool padded = in_dtype == BF16 && !exact && d % 8 == 0 && dv % 8 == 0 && !(d == 256 && dv == 256);
   // per-head K/V byte offsets are 32-bit in the direct-to-LDS kernel
-  const bool direct = (exact || padded || wide) && nk * dmax * 2 < (size_t(1) << 32) && std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+  const bool direct = (exact || padded || wide) && nk * dmax * 2 < (size_t(1) << 32) && knobs.attention_direct;
+  const bool f32_scale = knobs.attention_f32_scale != 0;
   if (direct && wide) {
     bm = 128;  // 4 waves, one per SIMD
     bn = 32;
@@ -70,16 +150,15 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
     if (query_tile == 256 || (query_tile != 128 && bh * ((nq + 255) / 256) >= 2 * 256 && nk >= 2560 &&
                               10 * ((nq + 255) / 256 * 256) <= 11 * ((nq + 127) / 128 * 128)))
       bm = 256;
-    if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
-      const int waves = std::atoi(w);
-      if (waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 4 or 8 for a padded head size";
+    if (const int waves = knobs.attention_waves) {
+      if (waves != 4 && waves != 8) return "attention kernel: attention.waves must be 4 or 8 for a padded head size";
       bm = 32u * (unsigned)waves;
     }
   } else if (direct) {
     const bool tile_known = query_tile == 64 || query_tile == 128 || query_tile == 256;
-    if (key_tile == 32 && !options.f32_scale && tile_known && !(d == 64 && query_tile == 256)) bn = 32;
-    if (tile_known && !(options.f32_scale && query_tile == 64)) bm = (unsigned)query_tile;  // the schedule's i split
-    else if (d == 64 && !options.f32_scale &&
+    if (key_tile == 32 && !f32_scale && tile_known && !(d == 64 && query_tile == 256)) bn = 32;
+    if (tile_known && !(f32_scale && query_tile == 64)) bm = (unsigned)query_tile;  // the schedule's i split
+    else if (d == 64 && !f32_scale &&
              ((query_tile == 512 && (key_tile == 32 || key_tile == 0)) ||
               (query_tile == 0 && bh * ((nq + 511) / 512) >= 2 * 256 &&
                10 * ((nq + 511) / 512 * 512) <= 11 * ((nq + 127) / 128 * 128))))
@@ -89,13 +168,12 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
       bm = 256;  // ... on long key loops (two resident 4-wave workgroups hide each other's prologue and epilogue,
                  // which wins up to about 2048 keys), and unless rounding nq up to 256 instead of 128 adds more
                  // than 10 % of idle query rows
-    if (const char* w = std::getenv("ILANG_ATTN_WAVES")) {
-      const int waves = std::atoi(w);
-      q64 = waves == 64 && d == 64 && !options.f32_scale;
+    if (const int waves = knobs.attention_waves) {
+      q64 = waves == 64 && d == 64 && !f32_scale;
       if (!q64) {
-        if (waves != 2 && waves != 4 && waves != 8) return "attention kernel: ILANG_ATTN_WAVES must be 2, 4 or 8 (or 64 for d = 64)";
+        if (waves != 2 && waves != 4 && waves != 8) return "attention kernel: attention.waves must be 2, 4 or 8 (or 64 for d = 64)";
         bm = 32u * (unsigned)waves;
-        if (options.f32_scale && bm == 64) bm = 128;
+        if (f32_scale && bm == 64) bm = 128;
         if (d == 64 && bm == 256) bn = 64;
       }
     }
@@ -103,11 +181,10 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   }
   // f32: the direct-to-LDS kernel for d, dv multiples of 4 up to 128, the larger above 32 (16-byte aligned operands,
   // 32-bit byte offsets inside a head; up to 32 the register-staged kernel with 32-column tiles is the faster one), the
-  // register-staged kernel with guarded columns otherwise (and under ILANG_ATTN_NO_DIRECT=1)
-  auto aligned16 = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  // register-staged kernel with guarded columns otherwise (and with knobs.attention_direct == 0)
   const bool f32_direct = in_dtype == F32 && d % 4 == 0 && dv % 4 == 0 && dmax > 32 && dmax <= 128 &&
                           nk * dmax * 4 < (size_t(1) << 32) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) &&
-                          std::getenv("ILANG_ATTN_NO_DIRECT") == nullptr;
+                          knobs.attention_direct;
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o;
   p.bh = (uint32_t)bh; p.nq = (uint32_t)nq; p.nk = (uint32_t)nk; p.d = (uint32_t)d; p.dv = (uint32_t)dv;
@@ -115,6 +192,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
   p.out_bf16 = out_dtype == BF16 ? 1u : 0u;
   p.scale_ptr = scale_ptr;
   p.scale_value = scale;
+  p.clock = knobs.clock_ticks;
   // the keys of a head in several parts: the direct kernels take (head, part) pairs for heads and write to the
   // caller's temporaries; attn_kv_merge follows.  (A request that the kernel chosen above cannot honour, the
   // register-staged ones and the 64-queries-per-wave kernel, is ignored: the result is the same.)
@@ -143,7 +221,7 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
       name = "attn_fwd_bf16_d" + std::to_string(wide ? 256 : padded ? (dmax <= 64 ? 64 : 128) : d) + "_bn" + std::to_string(bn) + "_direct";
       if (bm == 64) name += "_w2";
       if (bm == 256) name += "_w8";
-      if (options.f32_scale) name += "_f32scale";
+      if (f32_scale) name += "_f32scale";
       if (padded) name += "_pad";
     } else if (exact) name = d == 64 ? "attn_fwd_bf16_d64_bn64" : "attn_fwd_bf16_d128_bn64";
     else name = dmax <= 64 ? "attn_fwd_bf16_d64_bn64_any" : "attn_fwd_bf16_d128_bn64_any";
@@ -181,11 +259,12 @@ Err launch_attention(const void* q, const void* k, const void* v, void* o, DType
 // demo, one head of 512 x 64, 45 -> 16 us in 8 parts; 2 heads of 128 queries x 8192 keys of 128, 1136 -> 64 in 32.  Only where the direct kernels run (launch_attention's own
 // conditions).
 unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, size_t d, size_t dv, const AttentionOptions& options) {
-  if (bh == 0 || nq == 0 || d == 0 || dv == 0 || std::getenv("ILANG_ATTN_NO_DIRECT") != nullptr) return 1;
+  const KernelOptions& knobs = options.knobs;
+  if (bh == 0 || nq == 0 || d == 0 || dv == 0 || !knobs.attention_direct || knobs.attention_kv_parts == 1) return 1;
   const size_t dmax = d > dv ? d : dv;
   if (in_dtype == BF16) {
     if (d % 8 != 0 || dv % 8 != 0 || d > 256 || dv > 256 || !(nk * dmax * 2 < (size_t(1) << 32))) return 1;
-    if (const char* w = std::getenv("ILANG_ATTN_WAVES"); w && std::atoi(w) == 64) return 1;
+    if (knobs.attention_waves == 64) return 1;
     if (options.query_tile == 512) return 1;  // (may select the 64-queries-per-wave kernel)
   } else if (d % 4 != 0 || dv % 4 != 0 || dmax <= 32 || dmax > 128 || !(nk * dmax * 4 < (size_t(1) << 32))) {
     return 1;  // (f32: the direct kernel's head sizes; operands it cannot take for their alignment run unsplit)
@@ -193,8 +272,8 @@ unsigned attention_kv_splits(DType in_dtype, size_t bh, size_t nq, size_t nk, si
   // an f32 workgroup takes about 2.8 us per 32 keys (a bf16 one 0.7 us per 64): much shorter loops are worth parts
   const size_t least_loop = in_dtype == BF16 ? 2048 : 256, least_part = in_dtype == BF16 ? 512 : 64;
   size_t want;
-  if (const char* f = std::getenv("ILANG_ATTN_KV_SPLITS")) {
-    want = (size_t)std::atoi(f);  // forced (0 or 1: never split), still bounded by whole 64-key tiles below
+  if (knobs.attention_kv_parts > 1) {
+    want = (size_t)knobs.attention_kv_parts;  // forced, still bounded by whole 64-key tiles below
   } else {
     const size_t bm = in_dtype == BF16 && (options.query_tile == 64 || options.query_tile == 256) ? options.query_tile : 128;
     const size_t groups = bh * ((nq + bm - 1) / bm);
@@ -226,11 +305,13 @@ static unsigned pick_direct_tile(size_t t256, size_t t128) {
 }
 
 Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
-                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype) {
+                        hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype,
+                        const KernelOptions& knobs) {
   if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!fits_u32(m) || !fits_u32(n) || !fits_u32(k) || !fits_u32(bh)) return "gemm_nt kernel: extent exceeds 32 bits";
   if (!a || !b || !c) return "gemm_nt kernel: null device pointer";
+  if (!aligned16(a) || !aligned16(b)) return "gemm_nt kernel: operands must be 16-byte aligned";
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
@@ -242,15 +323,16 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   //                    128-tile kernel: 4.3 against 5.9 us at 128 x 128 x 64, 9.4 against 17.0 at 128 x 128 x 1024)
   // (k that is no multiple of 64: their _ktail forms, the last slab partial)
   // and the register-staged 128 x 128 kernel beyond their offset ranges (k > 2^22, more than 65535 batches).
-  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; ILANG_GEMM_DIRECT=256 | 128 | 0
-  // forces a kernel so that tests can reach each of them at small sizes (1 is read as 256).
+  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; knobs.gemm_tile = 256 | 128 and
+  // knobs.gemm_direct = 0 force a kernel so that tests and searches can reach each of them at small sizes.
   {
     const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
     unsigned tile = 128;  // (0: register-staged kernel)
     if (k >= 512 && t256 >= 64) tile = pick_direct_tile(t256, t128);
     if (tile_m == 256 && tile_n == 256) tile = 256;
     if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
-    if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
+    if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
+    if (!knobs.gemm_direct) tile = 0;
     const bool ktail = k % 64 != 0;
     if (tile && k <= (size_t(1) << 22) && bh <= 65535) {
       p.tiles_m = (uint32_t)((m + tile - 1) / tile);
@@ -258,10 +340,9 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
       const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
-      // the 256 x 256 tile runs with four waves of 128 x 128 (ILANG_GEMM_WAVES=8: the form with eight of 128 x 64,
+      // the 256 x 256 tile runs with four waves of 128 x 128 (knobs.gemm_waves = 8: the form with eight of 128 x 64,
       // kept for comparison: equal on one round of tiles, 5-10 % behind on several)
-      const char* waves = std::getenv("ILANG_GEMM_WAVES");
-      const bool w4 = tile == 256 && !(waves && std::atoi(waves) == 8);
+      const bool w4 = tile == 256 && knobs.gemm_waves != 8;
       const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct") +
                                (ktail ? "_ktail" : "") + (w4 ? "_w4" : "");
       if (note) *note = LaunchNote{name, tile, tile};
@@ -283,11 +364,11 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
 // Tile of a split product: the large tile needs both extents to fill most of it
 static unsigned split_k_tile(size_t m, size_t n) { return m >= 192 && n >= 192 ? 256 : 128; }
 
-unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k) {
-  if (bh == 0 || m == 0 || n == 0 || k % 8 != 0 || std::getenv("ILANG_GEMM_NO_SPLIT")) return 1;
+unsigned gemm_nt_bf16_split_k(size_t bh, size_t m, size_t n, size_t k, const KernelOptions& knobs) {
+  if (bh == 0 || m == 0 || n == 0 || k % 8 != 0 || knobs.gemm_k_parts == 1) return 1;
   const unsigned tile = split_k_tile(m, n);
-  if (const char* forced = std::getenv("ILANG_GEMM_SPLITS")) {  // (tests and measurements: that many parts, whole slabs each)
-    const size_t want = std::min<size_t>((size_t)std::max(0, std::atoi(forced)), k / 64);
+  if (knobs.gemm_k_parts > 1) {  // (tests, searches and measurements: that many parts, whole slabs each)
+    const size_t want = std::min<size_t>((size_t)knobs.gemm_k_parts, k / 64);
     if (want < 2 || bh * want > 65535) return 1;
     const size_t chunk = (k / want + 63) / 64 * 64;
     return (unsigned)((k + chunk - 1) / chunk);
@@ -328,6 +409,7 @@ Err launch_gemm_nt_bf16_split_k(const void* a, const void* b, void* c, float* pa
   if (!gemm_nt_bf16_supported(k)) return "gemm_nt kernel: k must be a positive multiple of 8";
   if (splits < 2 || bh * splits > 65535 || !fits_u32(m) || !fits_u32(n) || k > (size_t(1) << 22)) return "gemm_nt kernel: bad split";
   if (!a || !b || !c || !partial) return "gemm_nt kernel: null device pointer";
+  if (!aligned16(a) || !aligned16(b)) return "gemm_nt kernel: operands must be 16-byte aligned";
   if ((m * n) % 4 != 0) return "gemm_nt kernel: a split product needs m * n to be a multiple of 4";
   GemmParams p{};
   p.a = a; p.b = b; p.c = partial;
@@ -355,26 +437,30 @@ Err launch_gemm_nt_bf16_split_k(const void* a, const void* b, void* c, float* pa
   return launch(fn, (unsigned)rgrid, 1, 1, 256, &r, sizeof(r), stream);
 }
 
-static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n) {
+static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t tile_m, size_t tile_n, const KernelOptions& knobs) {
   if (k == 0 || k % 8 != 0 || n % 8 != 0 || k > (size_t(1) << 22) || n > (size_t(1) << 24) || bh > 65535) return 0;
   if (!fits_u32(m) || !fits_u32(n)) return 0;
   const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
   unsigned tile = t256 >= 128 ? pick_direct_tile(t256, t128) : 128;
   if (tile_m == 256 && tile_n == 256) tile = 256;
   if (tile_m == 128 && tile_n == 128) tile = 128;
-  if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = f[0] == '0' ? 0 : std::atoi(f) == 128 ? 128 : 256;
+  if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
+  if (!knobs.gemm_direct) tile = 0;  // (no register-staged form of this product: callers transpose and use the NT kernels)
   return tile;
 }
 
-bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k) { return gemm_nn_tile(bh, m, n, k, 0, 0) != 0; }
+bool gemm_nn_bf16_supported(size_t bh, size_t m, size_t n, size_t k, const KernelOptions& knobs) {
+  return gemm_nn_tile(bh, m, n, k, 0, 0, knobs) != 0;
+}
 
 Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                         hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype, float* partial,
-                        unsigned splits) {
-  unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n);
+                        unsigned splits, const KernelOptions& knobs) {
+  unsigned tile = gemm_nn_tile(bh, m, n, k, tile_m, tile_n, knobs);
   if (tile == 0) return "gemm_nn kernel: needs k % 8 == 0 and n % 8 == 0 (and extents within its offset range)";
   if (bh == 0 || m == 0 || n == 0) return {};
   if (!a || !b || !c) return "gemm_nn kernel: null device pointer";
+  if (!aligned16(a) || !aligned16(b)) return "gemm_nn kernel: operands must be 16-byte aligned";
   GemmParams p{};
   p.a = a; p.b = b; p.c = c;
   p.bh = (uint32_t)bh; p.m = (uint32_t)m; p.n = (uint32_t)n; p.k = (uint32_t)k;
@@ -399,8 +485,7 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
   if (grid > kMaxGrid) return "gemm_nn kernel: grid too large";
   hipFunction_t fn;
-  const char* waves = std::getenv("ILANG_GEMM_WAVES");  // (as for the NT kernels: four waves unless 8 is asked for)
-  const bool w4 = tile == 256 && !(waves && std::atoi(waves) == 8);
+  const bool w4 = tile == 256 && knobs.gemm_waves != 8;  // (as for the NT kernels: four waves unless 8 are asked for)
   const std::string name = std::string(tile == 256 ? "gemm_nn_bf16_256x256x64_direct" : "gemm_nn_bf16_128x128x64_direct") +
                            (k % 64 != 0 ? "_ktail" : "") + (w4 ? "_w4" : "");
   if (note) *note = LaunchNote{splits > 1 ? name + " (k in " + std::to_string(splits) + " parts)" : name, tile, tile};
@@ -417,14 +502,14 @@ Err launch_gemm_nn_bf16(const void* a, const void* b, void* c, size_t bh, size_t
 
 bool gemm_nt_f32_supported(size_t k) { return k > 0 && k % 4 == 0 && k <= (size_t(1) << 21); }
 
-unsigned gemm_nt_f32_split_k(size_t bh, size_t m, size_t n, size_t k) {
-  if (bh == 0 || m == 0 || n == 0 || !gemm_nt_f32_supported(k) || std::getenv("ILANG_GEMM_NO_SPLIT")) return 1;
+unsigned gemm_nt_f32_split_k(size_t bh, size_t m, size_t n, size_t k, const KernelOptions& knobs) {
+  if (bh == 0 || m == 0 || n == 0 || !gemm_nt_f32_supported(k) || knobs.gemm_k_parts == 1) return 1;
   auto parts_of = [&](size_t want) -> unsigned {
     if (want < 2 || bh * want > 65535) return 1;
     const size_t chunk = (k / want + 63) / 64 * 64;  // what one split contracts: whole slabs
     return (unsigned)((k + chunk - 1) / chunk);
   };
-  if (const char* forced = std::getenv("ILANG_GEMM_SPLITS")) return parts_of(std::min<size_t>((size_t)std::max(0, std::atoi(forced)), k / 64));
+  if (knobs.gemm_k_parts > 1) return parts_of(std::min<size_t>((size_t)knobs.gemm_k_parts, k / 64));
   // The model of gemm_nt_bf16_split_k with this kernel's figures: 1.7 us per 32-wide slab for a workgroup on a
   // 128 x 128 tile, 256 of them at a time (the 256 x 256 tile only takes grids that fill the chip), parts of at
   // least 64 of k.  Unsplit -> split, us: 128 x 128 x 8192 444 -> 36 (32 parts), 512 x 512 x 4096 227 -> 31 (16),
@@ -447,7 +532,7 @@ unsigned gemm_nt_f32_split_k(size_t bh, size_t m, size_t n, size_t k) {
 }
 
 Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size_t m, size_t n, size_t k,
-                       hipStream_t stream, LaunchNote* note, float* partial, unsigned splits) {
+                       hipStream_t stream, LaunchNote* note, float* partial, unsigned splits, const KernelOptions& knobs) {
   if (!gemm_nt_f32_supported(k)) return "gemm_nt f32 kernel: k must be a positive multiple of 4 (at most 2^21)";
   if (reinterpret_cast<uintptr_t>(a) % 16 != 0 || reinterpret_cast<uintptr_t>(b) % 16 != 0)
     return "gemm_nt f32 kernel: operands must be 16-byte aligned";
@@ -460,7 +545,7 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   // 256 x 256 tiles when they fill at least half of the CUs, 128 x 128 tiles otherwise
   const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
   unsigned tile = t256 >= 128 ? 256 : 128;
-  if (const char* f = std::getenv("ILANG_GEMM_DIRECT")) tile = std::atoi(f) == 128 ? 128 : 256;
+  if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
   // the k loop in parts over workgroups (gemm_nt_f32_split_k says when): partial products in the caller's temporary
   if (splits > 1) {
     if (!partial) return "gemm_nt f32 kernel: a split needs its temporary";

@@ -314,6 +314,15 @@ class Component:
         nat.check(core.i_hip_program_option(self._compile(), name.encode(), int(value)))
         return self
 
+    def clock_probe(self, ticks):
+        """Shader-clock accounting for the program's attention kernels (``i_hip_program_clock_probe``): ``ticks`` is
+        a ROCm tensor of two int64 that the caller clears (or None: off); workgroups add shader-clock cycles to
+        ``ticks[0]`` and ticks of the constant 100 MHz clock to ``ticks[1]``."""
+        if ticks is not None and (ticks.numel() < 2 or ticks.element_size() != 8 or not ticks.is_cuda):
+            raise ValueError("clock_probe takes a ROCm tensor of two 64-bit integers")
+        nat.check(core.i_hip_program_clock_probe(self._compile(), None if ticks is None else ticks.data_ptr()))
+        return self
+
     def report(self):
         """The kernels the last run dispatched, one line per kernel of the plan (``i_hip_program_report``)."""
         text = nat.check_ptr(core.i_hip_program_report(self._compile()))

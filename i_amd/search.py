@@ -22,10 +22,17 @@ outputs before the comparison.
 
     ranked = search(mm_t, grid(i=[128, 256], j=[128, 256]), inputs=(a, b), rtol=2e-2)
     best = ranked[0]          # Result(schedule='i:256,j:256', ms=..., error=..., plan='hand-written ...')
+
+What a schedule has no spelling for, but what matters on this chip (into how many parts the k loop of a product or
+the keys of a head are cut over workgroups, how many waves a workgroup has), is a second axis of the search: program
+options (``Component.option``, ``i_hip_program_option``), every candidate schedule under every combination of them.
+
+    ranked = search(mm_t, ["i:16,j:16"], inputs=(a, b), rtol=2e-2, options=option_grid({"gemm.k_parts": [1, 2, 4, 8, 16]}))
+    best.options              # {'gemm.k_parts': 8}
 """
 import itertools
-from dataclasses import dataclass
-from typing import Callable, Iterable, List, Optional, Sequence
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Iterable, List, Optional, Sequence
 
 
 @dataclass
@@ -36,6 +43,7 @@ class Result:
     plan: str                # first line of the backend plan for kernel f0 (which kernel form runs)
     failure: Optional[str] = None  # compile / run error text, or "mismatch"
     kernels: str = ""        # what the run dispatched (Component.report()): kernel names and their tiles
+    options: Dict[str, int] = field(default_factory=dict)  # the program options the candidate ran under
 
 
 def grid(**factors: Sequence) -> List[str]:
@@ -46,6 +54,13 @@ def grid(**factors: Sequence) -> List[str]:
     for combo in itertools.product(*(factors[n] for n in names)):
         out.append(",".join(f"{n}:{f}" for n, f in zip(names, combo)))
     return out
+
+
+def option_grid(values: Dict[str, Sequence[int]]) -> List[Dict[str, int]]:
+    """All combinations of program option values: option_grid({"gemm.k_parts": [1, 4], "gemm.waves": [4, 8]}) ->
+    [{'gemm.k_parts': 1, 'gemm.waves': 4}, {'gemm.k_parts': 1, 'gemm.waves': 8}, ...]."""
+    names = list(values)
+    return [dict(zip(names, combo)) for combo in itertools.product(*(values[n] for n in names))]
 
 
 def _plan_line(component) -> str:
@@ -76,10 +91,11 @@ def _time_ms(torch, fn, repeats: int, warmup: int) -> float:
 
 def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Sequence, rtol: float,
            referee: Optional[Callable[..., Sequence]] = None, repeats: int = 10, warmup: int = 2,
-           out_dtype=None, view: Optional[Callable] = None) -> List[Result]:
-    """Run build(schedule) for every schedule on `inputs` (ROCm torch tensors).
+           out_dtype=None, view: Optional[Callable] = None, options: Optional[Iterable[Dict[str, int]]] = None) -> List[Result]:
+    """Run build(schedule) for every schedule on `inputs` (ROCm torch tensors), under every set of program options
+    in `options` when given (each a dict of option name -> value, see option_grid).
 
-    Returns one Result per schedule, fastest first; candidates that fail to compile, fail to run or
+    Returns one Result per candidate, fastest first; candidates that fail to compile, fail to run or
     disagree with the referee by more than `rtol` come last with `failure` set.
     """
     import torch
@@ -92,22 +108,24 @@ def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Seq
         expected = [e.float() for e in expected]
 
     results = []
-    for schedule in schedules:
+    for schedule, opts in itertools.product(list(schedules), [dict(o) for o in options] if options is not None else [{}]):
         try:
             comp = build(schedule)
+            for name, value in opts.items():
+                comp.option(name, value)
             got = comp.exec_torch(*inputs, out_dtype=out_dtype)
             got = [got] if torch.is_tensor(got) else list(got)
             full = got
             got = [(view(g) if view else g).float() for g in got]
             kernels = comp.report().strip()
         except RuntimeError as e:
-            results.append(Result(schedule, None, None, "", failure=str(e)))
+            results.append(Result(schedule, None, None, "", failure=str(e), options=opts))
             continue
         plan = _plan_line(comp)
         if expected is None:
             expected = got  # first candidate that runs is the referee
         if len(got) != len(expected) or any(g.shape != e.shape for g, e in zip(got, expected)):
-            results.append(Result(schedule, None, None, plan, failure="mismatch (output count or shape)"))
+            results.append(Result(schedule, None, None, plan, failure="mismatch (output count or shape)", options=opts))
             continue
         err = 0.0
         for g, e in zip(got, expected):
@@ -115,11 +133,11 @@ def search(build: Callable[[str], object], schedules: Iterable[str], inputs: Seq
                 scale = float(e.abs().max()) or 1.0
                 err = max(err, float((g - e).abs().max()) / scale)
         if not err <= rtol:  # also catches NaN
-            results.append(Result(schedule, None, err, plan, failure="mismatch", kernels=kernels))
+            results.append(Result(schedule, None, err, plan, failure="mismatch", kernels=kernels, options=opts))
             continue
         outs = [torch.empty_like(g, dtype=out_dtype or torch.float32) for g in full]
         target = outs[0] if len(outs) == 1 else outs
         ms = _time_ms(torch, lambda: comp.into(target, *inputs), repeats, warmup)
-        results.append(Result(schedule, ms, err, plan, kernels=kernels))
+        results.append(Result(schedule, ms, err, plan, kernels=kernels, options=opts))
     results.sort(key=lambda r: (r.failure is not None, r.ms if r.ms is not None else float("inf")))
     return results

@@ -106,11 +106,54 @@ int i_hip_attention_ex(const void* q, const void* k, const void* v, void* o,
                        float scale, size_t query_tile, size_t key_tile, int f32_scale, void* stream);
 
 /*
- * Options of a compiled program, by name (i_compile has no options argument, core/i.h:44).  Known:
+ * i_hip_attention_ex with the launcher's remaining choices by name: `options` is "name=value name=value" with the
+ * attention.* names of i_hip_program_option ("attention.waves=8 attention.direct=1"; NULL or "": none), for tests
+ * and searches that want a particular kernel on small operands.
+ */
+int i_hip_attention_opt(const void* q, const void* k, const void* v, void* o,
+                        int in_dtype, int out_dtype,
+                        size_t bh, size_t nq, size_t nk, size_t d, size_t dv,
+                        float scale, size_t query_tile, size_t key_tile, const char* options, void* stream);
+
+/*
+ * Options of a compiled program, by name (i_compile has no options argument, core/i.h:44).  The schedule's splits
+ * pick the workgroup tile (README.md:139-163); these are the choices a schedule has no spelling for.  They belong
+ * to the program, not to the process: two programs (or threads) with different wishes do not meet.  Known:
  *   "attention.f32_scale"  0 (default) / 1: what f32_scale is to i_hip_attention_ex, for the program's attention kernels
- * Returns 0, or -1 with the text in i_error() for an unknown name.  Takes effect from the next i_exec*.
+ *   "attention.kv_parts"   keys of a head in parts over workgroups: 0 (default) the launcher decides by grid size,
+ *                          1 never, n that many (whole 64-key tiles each, so fewer may result)
+ *   "attention.waves"      waves per workgroup of the direct bf16 kernels: 0 (default) by schedule tile and size,
+ *                          2 / 4 / 8, 64 = the 64-queries-per-wave kernel (d = 64)
+ *   "attention.direct"     1 (default) / 0: the register-staged kernels instead of the direct-to-LDS ones
+ *   "gemm.k_parts"         k loop of a product in parts over workgroups: 0 (default) by a model of the time, 1 never, n
+ *   "gemm.tile"            workgroup tile of the direct product kernels: 0 (default) by schedule tile and size, 128, 256
+ *   "gemm.waves"           waves of the 256 x 256 tile: 0 (default: four), 4, 8
+ *   "gemm.direct"          1 (default) / 0: the register-staged bf16 product kernel
+ *   "generated.only"       0 (default) / 1: every kernel in its generated form (no hand-written kernel)
+ *   "generated.wave"       wavefront-per-iteration form of generated reduction nests: -1 (default) by extents, 0 never, 1 always
+ * Returns 0, or -1 with the text in i_error() for an unknown name or a value the option does not take.  Takes
+ * effect from the next i_exec*.
  */
 int i_hip_program_option(i_program* program, const char* name, int value);
+
+/*
+ * Shader-clock accounting for a program's attention kernels (no counterpart in the reference).  `ticks` is device
+ * memory for two 64-bit counters, 8-byte aligned, that the caller clears; from the next i_exec* on every workgroup
+ * of the program's bf16 direct-to-LDS attention kernels adds to ticks[0] the shader-clock cycles (s_memtime: the
+ * clock the power manager grants at the moment) and to ticks[1] the ticks of the constant 100 MHz clock that passed
+ * between its first and its last instruction.  ticks[0] / ticks[1] / 10 is the shader clock in GHz under the
+ * kernel, averaged over the time its workgroups were resident: what a measured fraction of the matrix-core peak,
+ * quoted at 2.4 GHz, has to be read against.  NULL switches it off.  Costs four atomic adds per workgroup.
+ */
+int i_hip_program_clock_probe(i_program* program, void* ticks);
+
+/*
+ * The same two clocks read by a one-wavefront kernel of its own, for work that cannot count for itself (a vendor
+ * library's kernel): reads both clocks, sleeps for `microseconds` (at most 2 000 000), reads them again and adds the
+ * differences to ticks[0] (shader clock) and ticks[1] (100 MHz clock).  Enqueue it on a second stream beside the
+ * work in question.  It occupies one wave slot of one compute unit while it sleeps.
+ */
+int i_hip_shader_clock_probe(void* ticks, unsigned microseconds, void* stream);
 
 /*
  * What the last i_exec* of this program dispatched, one line per kernel of the plan that i_code prints:
@@ -151,6 +194,14 @@ int i_hip_gemm_nn_bf16(const void* a, const void* b, float* c,
  */
 int i_hip_gemm_nt_f32(const float* a, const float* b, float* c,
                       size_t bh, size_t m, size_t n, size_t k, void* stream);
+
+/*
+ * Any of the three products above with the launcher's choices by name: in_dtype I_DTYPE_BF16 (b_row_major 0: a b^T,
+ * 1: a b; c f32 or bf16) or I_DTYPE_F32 (a b^T, f32 c); `options` is "name=value name=value" with the gemm.* names of
+ * i_hip_program_option ("gemm.tile=128 gemm.waves=8"; NULL or "": none).  No temporaries, so gemm.k_parts does not apply.
+ */
+int i_hip_gemm_opt(const void* a, const void* b, void* c, int in_dtype, int out_dtype, int b_row_major,
+                   size_t bh, size_t m, size_t n, size_t k, const char* options, void* stream);
 
 /*
  * Row softmax over the last axis of an f32 [rows, cols] matrix: the fused

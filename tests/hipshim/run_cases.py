@@ -1,7 +1,8 @@
 """Runs components through the product's executor with every kernel in its generated form, on the CPU
 emulation of the HIP runtime (shim.cpp), and compares with the C the oracle backend emits for the same
 component.  Started as a subprocess by tests/test_generated_kernels_cpu.py with
-ILANG_CORE_LIB, ILANG_HIPCC, ILANG_HIP_GENERATED_ONLY, ILANG_NO_TORCH and ILANG_NO_DISK_CACHE set.
+ILANG_CORE_LIB, ILANG_HIPCC, ILANG_NO_TORCH and ILANG_NO_DISK_CACHE set; ILANG_SHIM_WAVE=1 asks for the
+wavefront-per-iteration form of reduction nests (the program option generated.wave).
 Prints the case name before running it, so a crash (a guard page hit = out-of-bounds access) names its case."""
 import sys
 from pathlib import Path
@@ -149,6 +150,9 @@ def main():
         build, shapes = CASES[name]
         print("CASE", name, flush=True)
         comp = build()
+        comp.option("generated.only", 1)
+        if os.environ.get("ILANG_SHIM_WAVE") is not None:
+            comp.option("generated.wave", int(os.environ["ILANG_SHIM_WAVE"]))
         inputs = [rnd(s, k + 1) for k, s in enumerate(shapes)]
         got = run_without_allocating(comp, inputs) if noalloc else comp.exec_numpy(*inputs)
         ref = oracle.compile_component(comp.handle).run(*inputs)

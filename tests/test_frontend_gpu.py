@@ -194,15 +194,16 @@ def test_config1_golden_reference_outputs(torch, golden):
 def test_generated_and_hand_written_forms_agree(torch):
     q, k, v = (np.random.default_rng(s).uniform(-1, 1, (200, 48)).astype(np.float32) for s in (1, 2, 3))
     hand = flash().exec_numpy(q, k, v)
-    os.environ["ILANG_HIP_GENERATED_ONLY"] = "1"
-    try:
-        gen = flash().exec_numpy(q, k, v)
-        x = rnd((70, 300), 1)
-        sm_gen = softmax_rowstaged().exec_numpy(x)
-        a, b = rnd((50, 24), 1), rnd((30, 24), 2)
-        mm_gen = (i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")).exec_numpy(a, b)
-    finally:
-        del os.environ["ILANG_HIP_GENERATED_ONLY"]
+
+    def generated(comp):
+        comp.option("generated.only", 1)
+        return comp
+
+    gen = generated(flash()).exec_numpy(q, k, v)
+    x = rnd((70, 300), 1)
+    sm_gen = generated(softmax_rowstaged()).exec_numpy(x)
+    a, b = rnd((50, 24), 1), rnd((30, 24), 2)
+    mm_gen = generated(i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")).exec_numpy(a, b)
     ref = oracle.attention_tiled(q, k, v)
     close(hand, ref, RTOL_F32)
     close(gen, ref, RTOL_F32)
@@ -238,6 +239,54 @@ def test_config3_mm_t_bf16_device(torch):
     close(c[rows].cpu().numpy(), oracle.mm_t(a[rows], b), RTOL_BF16)
     cols = np.r_[0:4, n - 4:n]
     close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
+
+
+def test_bf16_operands_that_start_off_a_16_byte_boundary(torch):
+    """Every bf16 kernel moves 16 bytes per lane (the direct ones straight from global memory into LDS).  Operands
+    that are views starting one element (2 bytes) into their allocation are copied into aligned temporaries by the
+    executor, a misaligned attention output is written through one; the launchers themselves refuse such operands.
+    Attention (d = 128 and a padded head size, f32 and bf16 results into views that are misaligned too), mm_t
+    and the product with a row-major right operand, against the oracle."""
+    from i_amd import _native as nat
+
+    def shifted(a, dtype):
+        buf = torch.zeros(a.size + 1, dtype=dtype, device="cuda")
+        view = buf[1:].view(a.shape)
+        view.copy_(torch.from_numpy(a))
+        assert view.data_ptr() % 16 != 0
+        return view
+
+    attn = flash(prefix="b", scaled=True)
+    for d, out_dtype in ((128, torch.float32), (72, torch.bfloat16), (64, torch.float32)):
+        bh, nq, nk = 2, 200, 333
+        q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), sd)) for sd, n in ((1, nq), (2, nk), (3, nk)))
+        scale = np.float32(1.0 / np.sqrt(d))
+        ref = oracle.attention_tiled(q, k, v, scale)
+        qd, kd, vd = (shifted(x, torch.bfloat16) for x in (q, k, v))
+        whole = torch.full((bh * nq * d + 2,), -7.0, dtype=out_dtype, device="cuda")
+        out = whole[1:-1].view(bh, nq, d)
+        attn.into(out, qd, kd, torch.tensor(scale, device="cuda"), vd)
+        assert "attn_fwd_bf16" in attn.report(), attn.report()
+        assert whole[0].item() == -7.0 and whole[-1].item() == -7.0
+        close(out.float().cpu().numpy(), ref, RTOL_BF16)
+    a, b = (oracle.to_bf16_f32(np.random.default_rng(sd).uniform(-1, 1, shape).astype(np.float32)) for sd, shape in ((1, (300, 136)), (2, (260, 136))))
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    got = mm_t.exec_torch(shifted(a, torch.bfloat16), shifted(b, torch.bfloat16))
+    assert "gemm_nt_bf16" in mm_t.report(), mm_t.report()
+    close(got.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
+    mm = i("ik*kj~ijk|i:16,k:16|ii'jkk'") >> i("+ijk~ij|i:16,k:16|ii'j!kk'0")
+    bt = np.ascontiguousarray(b[:256].T)  # [136, 256]
+    got = mm.exec_torch(shifted(a, torch.bfloat16), shifted(bt, torch.bfloat16))
+    assert "gemm_n" in mm.report() and "generated" not in mm.report(), mm.report()
+    close(got.cpu().numpy(), oracle.mm_t(a, b[:256]), RTOL_BF16)
+    # the launchers say so instead of reading from such an address
+    qd = shifted(oracle.to_bf16_f32(rnd((1, 64, 64), 1)), torch.bfloat16)
+    o = torch.empty(1, 64, 64, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert nat.core.i_hip_attention(qd.data_ptr(), qd.data_ptr(), qd.data_ptr(), o.data_ptr(), nat.BF16, nat.F32, 1, 64, 64, 64, 64, 0.1, stream) == -1
+    assert "16-byte aligned" in nat.last_error()
+    assert nat.core.i_hip_gemm_nt_bf16(qd.data_ptr(), qd.data_ptr(), o.data_ptr(), 1, 64, 64, 64, stream) == -1
+    assert "16-byte aligned" in nat.last_error()
 
 
 @pytest.mark.parametrize("k", [42, 40, 64])  # 42: operands padded to k = 44 first; 40: a partial last slab; 64: whole slabs
@@ -284,7 +333,7 @@ def test_products_with_any_contracted_extent_run_on_the_matrix_kernels(torch):
 def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(torch, monkeypatch):
     """One small extent against a long contraction leaves most CUs without an output tile: the executor then splits
     the k loop over workgroups (partial products in a temporary, added up by a second kernel).  Against float64,
-    with whole and partial last slabs, several batches, f32 and bf16 results; ILANG_GEMM_NO_SPLIT=1 gives the
+    with whole and partial last slabs, several batches, f32 and bf16 results; the program option gemm.k_parts = 1 gives the
     unsplit kernel and the same numbers to within the order of the sums."""
     mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
     bmm = i("bik*bjk~bijk | i:16,j:16 | bjii'j'k") >> i("+bijk~bij | i:16,j:16 | bjii'j'k0")
@@ -294,13 +343,13 @@ def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(tor
         a = (torch.rand(*shape_a, device="cuda", generator=g) * 2 - 1).bfloat16()
         b = (torch.rand(*shape_b, device="cuda", generator=g) * 2 - 1).bfloat16()
         ref = a.double() @ b.double().transpose(-1, -2)
-        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        comp.option("gemm.k_parts", 0)
         got = comp.exec_torch(a, b)
         assert "parts)" in comp.report(), comp.report()
         assert float((got.double() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
         got16 = comp.exec_torch(a, b, out_dtype=torch.bfloat16)
         assert float((got16.double() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
-        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        comp.option("gemm.k_parts", 1)
         plain = comp.exec_torch(a, b)
         assert "parts)" not in comp.report()
         assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
@@ -311,13 +360,13 @@ def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(tor
         a = (torch.rand(m, k, device="cuda", generator=g) * 2 - 1).bfloat16()
         b = (torch.rand(k, n, device="cuda", generator=g) * 2 - 1).bfloat16()
         ref = a.double() @ b.double()
-        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        mm.option("gemm.k_parts", 0)
         got = mm.exec_torch(a, b)
         assert "gemm_nn_bf16" in mm.report() and "parts)" in mm.report(), mm.report()
         assert float((got.double() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
         got16 = mm.exec_torch(a, b, out_dtype=torch.bfloat16)
         assert float((got16.double() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
-        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        mm.option("gemm.k_parts", 1)
         plain = mm.exec_torch(a, b)
         assert "parts)" not in mm.report()
         assert float((plain - got).abs().max()) <= 1e-4 * float(ref.abs().max())
@@ -327,16 +376,16 @@ def test_products_with_few_tiles_and_a_long_k_loop_are_split_over_workgroups(tor
         a = torch.rand(*shape_a, device="cuda", generator=g) * 2 - 1
         b = torch.rand(*shape_b, device="cuda", generator=g) * 2 - 1
         ref = a.double() @ b.double().transpose(-1, -2)
-        monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+        comp.option("gemm.k_parts", 0)
         got = comp.exec_torch(a, b)
         assert "_f32_" in comp.report() and "parts)" in comp.report(), comp.report()
         assert float((got.double() - ref).abs().max()) <= RTOL_F32 * float(ref.abs().max())
-        monkeypatch.setenv("ILANG_GEMM_NO_SPLIT", "1")
+        comp.option("gemm.k_parts", 1)
         plain = comp.exec_torch(a, b)
         assert "parts)" not in comp.report()
         assert float((plain - got).abs().max()) <= 1e-5 * float(ref.abs().max())
     # a product that fills the chip is left alone
-    monkeypatch.delenv("ILANG_GEMM_NO_SPLIT", raising=False)
+    mm_t.option("gemm.k_parts", 0)
     a = torch.randn(2048, 4096, device="cuda").bfloat16()
     mm_t.exec_torch(a, a)
     assert "parts)" not in mm_t.report()
@@ -496,7 +545,7 @@ def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
 def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroups(torch, monkeypatch):
     """A single head (or a few sequences) leaves most CUs without a query tile: the executor then runs parts of the
     key loop side by side (each part's normalised rows and the logarithm of its row sums in a temporary) and a
-    second kernel merges them.  ILANG_ATTN_KV_SPLITS forces a number of parts, so that small operands reach the
+    second kernel merges them.  The program option attention.kv_parts forces a number of parts, so that small operands reach the
     path: every direct bf16 kernel family (d = 128 without a reference, d = 64 with prescaled scores, padded head
     sizes, d = 256), ragged query and key counts, f32 and bf16 results, against the oracle and against the
     unsplit kernel; then the launcher's own choice for one long head."""
@@ -508,11 +557,11 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
         sd = torch.tensor(scale, device="cuda")
         rows = np.r_[0:8, NQ - 8:NQ]
         ref = oracle.attention_tiled(q[:, rows], k, v, scale)
-        monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "1")
+        comp.option("attention.kv_parts", 1)
         plain = comp.exec_torch(qd, kd, sd, vd)
         assert "keys in" not in comp.report()
-        for parts in ("2", "3", "16"):
-            monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", parts)
+        for parts in (2, 3, 16):
+            comp.option("attention.kv_parts", parts)
             got = comp.exec_torch(qd, kd, sd, vd)
             assert "(keys in " in comp.report(), comp.report()
             close(got.cpu().numpy()[:, rows], ref, RTOL_BF16)
@@ -523,7 +572,8 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
     # sends that part of the d = 128 kernel (exponentials without a reference) through its second pass with the
     # running max, and the merge then weighs parts whose sums differ by 2^115 or 2^-430
     plain_flash = flash(prefix="b")
-    monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "3")
+    plain_flash.option("attention.kv_parts", 3)
+    comp.option("attention.kv_parts", 3)
     for d in (128, 64):
         for offset in (80.0, -300.0):
             nq, nk = 300, 1500
@@ -547,7 +597,7 @@ def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroup
         got = comp.exec_torch(*(torch.from_numpy(a).cuda() for a in (q, k)), torch.tensor(scale, device="cuda"), torch.from_numpy(v).cuda())
         assert "_f32_" in comp.report() and "(keys in 3 parts)" in comp.report(), comp.report()
         close(got.cpu().numpy(), ref, RTOL_F32)
-    monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
+    comp.option("attention.kv_parts", 0)
     # the reference's demo (one f32 head of 512 x 64, 4 workgroups as it is): 8 parts of 64 keys
     q, k, v = (np.random.default_rng(s).uniform(-1, 1, (512, 64)).astype(np.float32) for s in (1, 2, 3))
     demo = flash()
@@ -594,12 +644,11 @@ def test_random_shapes_through_the_split_loops(torch, monkeypatch):
         g = torch.Generator(device="cuda").manual_seed(case)
         q, k, v = ((torch.randn(bh, n, w, device="cuda", generator=g) * 0.7).to(dt) for n, w in ((nq, d), (nk, d), (nk, dv)))
         ref = torch.softmax((q.double() @ k.double().transpose(1, 2)) * d ** -0.5, -1) @ v.double()
-        monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", str(rng.choice([2, 3, 5, 8, 13, 32])))
+        fa.option("attention.kv_parts", rng.choice([2, 3, 5, 8, 13, 32]))
         print("case attention", case, bf16, bh, nq, nk, d, dv, flush=True)
         got = fa.exec_torch(q, k, torch.tensor(d ** -0.5, device="cuda"), v)
         split += "(keys in" in fa.report()
         assert float((got.double() - ref).abs().max()) <= (RTOL_BF16 if bf16 else RTOL_F32) * float(ref.abs().max()), fa.report()
-    monkeypatch.delenv("ILANG_ATTN_KV_SPLITS")
     assert split >= 30  # (head sizes no direct kernel has run unsplit)
     split = 0
     for case in range(40):
@@ -613,9 +662,9 @@ def test_random_shapes_through_the_split_loops(torch, monkeypatch):
         a = (torch.rand(bh, m, k, device="cuda", generator=g) * 2 - 1).to(dt)
         b = (torch.rand(*((bh, n, k) if kind.startswith("nt") else (bh, k, n)), device="cuda", generator=g) * 2 - 1).to(dt)
         ref = a.double() @ (b.double().transpose(1, 2) if kind.startswith("nt") else b.double())
-        monkeypatch.setenv("ILANG_GEMM_SPLITS", str(rng.choice([2, 3, 4, 7, 16, 32])))
         print("case product", case, kind, bh, m, n, k, flush=True)
         comp = mm_t if kind.startswith("nt") else mm
+        comp.option("gemm.k_parts", rng.choice([2, 3, 4, 7, 16, 32]))
         got = comp.exec_torch(a, b)
         split += "(k in" in comp.report()
         bar = 1e-2 if kind.endswith("16") else RTOL_F32
@@ -876,13 +925,14 @@ def test_multi_nest_generated_kernels_run_as_one_workgroup(torch, monkeypatch):
     assert "one workgroup of 1024 work-items, 2 loop nests separated by barriers" in colnorm.report()
     xd = torch.from_numpy(x).cuda()
     assert torch.equal(colnorm.exec_torch(xd), colnorm.exec_torch(xd))  # repeatable
-    monkeypatch.setenv("ILANG_HIP_GENERATED_ONLY", "1")
     sm = softmax_naive()
+    sm.option("generated.only", 1)
     y = rnd((130, 257), 2)
     close(sm.exec_numpy(y), oracle.row_softmax(y), RTOL_F32)
     assert sm.report().count("one workgroup of 1024 work-items") == 2  # row_max_shift and row_normalize
     q, k, v = rnd((40, 24), 1), rnd((50, 24), 2), rnd((50, 24), 3)
     nv = naive()
+    nv.option("generated.only", 1)
     close(nv.exec_numpy(q, k, v), oracle.compile_component(nv.handle).run(q, k, v), RTOL_F32)
 
 
@@ -890,16 +940,15 @@ def test_multi_nest_generated_kernels_run_as_one_workgroup(torch, monkeypatch):
 def test_reduction_nests_in_the_wavefront_form(torch, monkeypatch, wave):
     """Generated reduction nests have a second form in which a wavefront stands where a work-item stood (the
     reduction loop spread over 64 lanes, lane shares combined by a butterfly).  Forced on, forced off and left to
-    the launcher (ILANG_HIP_WAVE unset), against NumPy in float64 and, at sizes it finishes quickly, the emitted C."""
-    if wave is None:
-        monkeypatch.delenv("ILANG_HIP_WAVE", raising=False)
-    else:
-        monkeypatch.setenv("ILANG_HIP_WAVE", wave)
+    the launcher (the program option generated.wave), against NumPy in float64 and, at sizes it finishes quickly, the
+    emitted C."""
     x = rnd((300, 2500), 1)
     x64 = x.astype(np.float64)
     for src, ref in ((">ij~i", x64.max(1)), ("<ij~i", x64.min(1)), ("+ij~i", x64.sum(1)), ("+ij~j", x64.sum(0)),
                      (">ij~j", x64.max(0)), ("+ij~i|j:16|ijj'", x64.sum(1)), ("+ij~.", x64.sum())):
         comp = i(src)
+        if wave is not None:
+            comp.option("generated.wave", int(wave))
         got = comp.exec_numpy(x)
         # sums of 2500 unit normals: the bar is relative to the sum of magnitudes, which bounds the rounding error
         assert np.abs(got - ref).max() <= RTOL_F32 * np.abs(x64).sum(1).max(), src
@@ -938,12 +987,13 @@ def test_per_nest_launches_are_refused_on_a_real_device():
     code = ("import torch\n"
             "from i_amd import Component as i, I\n"
             "c = (I & i('>ij~i|i:16,j:16|jii\\'j\\'')) >> i('ij-i~ij|i:16,j:16|1jii\\'j\\'')\n"
+            "c.option('generated.only', 1)\n"
             "try:\n"
             "    c.exec_torch(torch.ones(8, 8, device='cuda'))\n"
             "    print('RAN')\n"
             "except RuntimeError as e:\n"
             "    print('REFUSED' if 'restricted to the CPU emulation' in str(e) else 'OTHER: ' + str(e))\n")
-    env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_HIP_GENERATED_ONLY="1")
+    env = dict(os.environ, ILANG_HIP_PHASES="1")
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300,
                        cwd=Path(__file__).resolve().parent.parent)
     assert r.stdout.strip().splitlines()[-1] == "REFUSED", r.stdout + r.stderr[-1500:]

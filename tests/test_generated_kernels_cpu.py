@@ -29,7 +29,7 @@ def run_cases(shim_lib, extra_env, names=()):
     env.pop("ILANG_HIP_PHASES", None)
     # ILANG_HIP_UNCHECKED: plain accesses instead of the bounds-checked ones the product emits, so that an access
     # outside a buffer still hits a guard page here and names a lowering that is not sound
-    env.update({"ILANG_CORE_LIB": str(shim_lib), "ILANG_HIPCC": str(SHIM / "hostcc.py"), "ILANG_HIP_GENERATED_ONLY": "1",
+    env.update({"ILANG_CORE_LIB": str(shim_lib), "ILANG_HIPCC": str(SHIM / "hostcc.py"),
                 "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1", "ILANG_HIP_UNCHECKED": "1"})
     env.update(extra_env)
     r = subprocess.run([sys.executable, str(SHIM / "run_cases.py"), *names], env=env, capture_output=True, text=True, timeout=900)
@@ -54,11 +54,11 @@ def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
 
 
 def test_wavefront_form_of_reduction_nests_matches_too(shim_lib):
-    """ILANG_HIP_WAVE=1 takes the form of a nest in which a wavefront stands where a work-item stood (reduction
+    """The program option generated.wave = 1 (ILANG_SHIM_WAVE=1 to the case runner) takes the form of a nest in which a wavefront stands where a work-item stood (reduction
     loops spread over its 64 lanes, lane shares combined by a butterfly) wherever a nest has one; the emulation
     runs the lanes as 64 threads.  The order of a sum changes, hence the f32 bar instead of 1e-5."""
-    run_cases(shim_lib, {"ILANG_HIP_WAVE": "1", "ILANG_SHIM_CASES": "wave", "ILANG_SHIM_TOLERANCE": "1e-4"})
-    run_cases(shim_lib, {"ILANG_HIP_WAVE": "1", "ILANG_SHIM_TOLERANCE": "1e-4", "ILANG_HIP_UNCHECKED": "0"},
+    run_cases(shim_lib, {"ILANG_SHIM_WAVE": "1", "ILANG_SHIM_CASES": "wave", "ILANG_SHIM_TOLERANCE": "1e-4"})
+    run_cases(shim_lib, {"ILANG_SHIM_WAVE": "1", "ILANG_SHIM_TOLERANCE": "1e-4", "ILANG_HIP_UNCHECKED": "0"},
               names=["row sum 5x300", "fused matrix-vector product", "column max", "mlp with pair"])
 
 
@@ -73,7 +73,7 @@ def test_schedules_with_unsound_lowerings_cannot_fault(shim_lib):
     found by random schedules on this emulation).  The reference reads heap garbage there; the generated kernels
     check every access, so on a device this is a wrong result for a schedule that was wrong already, not a memory
     fault.  Unchecked, each of these hits a guard page."""
-    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"), ILANG_HIP_GENERATED_ONLY="1",
+    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"),
                ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
     code = """
 import sys
@@ -84,7 +84,9 @@ cases = [(">ij~j|i:4:2,j:4|jij'i'i''", "ij-j~ij|i:4:2,j:4|jij'i'i''1", (13, 10))
          ("+ij~j|i:8|ii'j", "ij-j~ij|i:8|ii'j1", (10, 9))]
 a, b, shape = cases[int(sys.argv[1])]
 x = np.random.default_rng(1).standard_normal(shape).astype(np.float32)
-out = ((I & i(a)) >> i(b)).exec_numpy(x)
+comp = (I & i(a)) >> i(b)
+comp.option("generated.only", 1)
+out = comp.exec_numpy(x)
 print("ran", out.shape == shape)
 """
     for n in range(3):
@@ -105,7 +107,7 @@ def test_fixed_workspace_entry_matches_on_the_cpu(shim_lib):
 def test_operands_that_disagree_on_a_shared_index_are_refused_before_any_launch(shim_lib):
     """A kernel takes each loop bound from one operand; another operand with a smaller extent for the same index
     would be read out of bounds (a GPU memory fault on the device, a guard-page hit here)."""
-    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"), ILANG_HIP_GENERATED_ONLY="1",
+    env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"),
                ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
     code = """
 import numpy as np

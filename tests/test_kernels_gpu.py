@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
+from conftest import gemm_kernel_knobs
 
 pytestmark = pytest.mark.gpu
 
@@ -25,8 +26,10 @@ def env():
     class Env:
         pass
 
+    from conftest import NativeWithKnobs
+
     e = Env()
-    e.torch, e.nat = torch, nat
+    e.torch, e.nat = torch, NativeWithKnobs(nat)
     e.stream = lambda: torch.cuda.current_stream().cuda_stream
     return e
 
@@ -112,13 +115,13 @@ def test_attention_f32_online_rescale_stress(env):
 
 @pytest.mark.parametrize("d", [64, 128, 36, 60, 96, 100, 124])
 @pytest.mark.parametrize("direct", [True, False])
-def test_attention_f32_direct_and_staged_kernels_vs_oracle(env, monkeypatch, d, direct):
+def test_attention_f32_direct_and_staged_kernels_vs_oracle(env, knobs, d, direct):
     """f32 operands with d == dv that is a multiple of 4 above 32 run the kernel that moves K/V tiles global -> LDS directly
-    (with its LDS rows padded when d is neither 64 nor 128), everything else (and ILANG_ATTN_NO_DIRECT=1) the
+    (with its LDS rows padded when d is neither 64 nor 128), everything else (and the launcher option attention.direct=0) the
     register-staged one: both against the oracle on one tile, partial tiles, several heads (more than the 8 XCDs),
     ragged query counts, negative and zero scales, and a longer key loop."""
     if not direct:
-        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+        knobs["attention.direct"] = 0
     for bh, nq, nk, scale in ((1, 128, 32, 1.0), (3, 200, 333, 0.11), (2, 77, 130, -0.2), (9, 130, 64, 0.0), (1, 1, 1, 1.0),
                               (2, 512, 1024, float(np.float32(1.0 / np.sqrt(d))))):
         q, k, v = (rnd((bh, n, d), sd) for sd, n in ((1, nq), (2, nk), (3, nk)))
@@ -164,15 +167,15 @@ def test_attention_bf16_vs_oracle(env, bh, nq, nk, d):
 
 @pytest.mark.parametrize("d", [8, 24, 40, 56, 72, 80, 96, 112, 120])
 @pytest.mark.parametrize("waves", ["4", "8", "staged"])
-def test_attention_bf16_head_sizes_between_the_kernel_sizes(env, monkeypatch, d, waves):
+def test_attention_bf16_head_sizes_between_the_kernel_sizes(env, knobs, d, waves):
     """d == dv that is a multiple of 8 but neither 64 nor 128 runs the direct-to-LDS kernels with LDS rows padded to
     64 or 128 columns (4 and 8 waves per workgroup forced in turn; "staged": the register-staged kernel these
     shapes used to take).  Short and long key loops (the steady state needs four full tiles), partial tiles, ragged
     query counts, more heads than XCDs, both output types."""
     if waves == "staged":
-        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+        knobs["attention.direct"] = 0
     else:
-        monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+        knobs["attention.waves"] = waves
     scale = float(np.float32(1.0 / np.sqrt(d)))
     for bh, nq, nk in ((1, 64, 64), (3, 200, 333), (9, 130, 700), (2, 300, 1024)):
         q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
@@ -227,18 +230,18 @@ def test_attention_bf16_head_sizes_above_128(env, d):
 
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("force", [None, "waves8", "q64", "staged"])
-def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
+def test_attention_bf16_every_kernel_vs_oracle(env, knobs, d, force):
     """The launcher picks between the direct-to-LDS kernel (4 or 8 waves per workgroup), the 64-queries-per-wave
     kernel (d = 64) and the register-staged kernel; force each of them on one ragged problem (7 full 64-key
     tiles + a partial one, so the steady-state loop, its drain and the masked tail all run)."""
     if force == "q64" and d != 64:
         pytest.skip("the 64-queries-per-wave kernel exists for d = 64 only")
     if force == "waves8":
-        monkeypatch.setenv("ILANG_ATTN_WAVES", "8")
+        knobs["attention.waves"] = "8"
     elif force == "q64":
-        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
+        knobs["attention.waves"] = "64"
     elif force == "staged":
-        monkeypatch.setenv("ILANG_ATTN_NO_DIRECT", "1")
+        knobs["attention.direct"] = 0
     bh, nq, nk = 2, 300, 450
     q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s, n in ((1, nq), (2, nk), (3, nk)))
     scale = float(np.float32(1.0 / np.sqrt(d)))
@@ -247,31 +250,31 @@ def test_attention_bf16_every_kernel_vs_oracle(env, monkeypatch, d, force):
     assert_close(gpu_attention(env, q, k, v, scale, bf16=True, out_bf16=True), ref, RTOL_BF16)
 
 
-def test_attention_bf16_workgroup_sizes_agree_bitwise(env, monkeypatch):
+def test_attention_bf16_workgroup_sizes_agree_bitwise(env, knobs):
     """A wave does the same arithmetic whether its workgroup has 4 or 8 waves."""
     bh, n, d = 16, 1024, 128
     q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s)) for s in (1, 2, 3))
-    monkeypatch.setenv("ILANG_ATTN_WAVES", "4")
+    knobs["attention.waves"] = "4"
     a = gpu_attention(env, q, k, v, 0.1, bf16=True)
-    monkeypatch.setenv("ILANG_ATTN_WAVES", "8")
+    knobs["attention.waves"] = "8"
     b = gpu_attention(env, q, k, v, 0.1, bf16=True)
     assert np.array_equal(a, b)
-    monkeypatch.setenv("ILANG_ATTN_WAVES", "3")
+    knobs["attention.waves"] = "3"
     t = env.torch
     x = t.zeros(1, 8, 128, device="cuda", dtype=t.bfloat16)
     rc = env.nat.core.i_hip_attention(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 1, 1, 8, 8, 128, 128,
                                       1.0, env.stream())
-    assert rc == -1 and "ILANG_ATTN_WAVES" in env.nat.last_error()
+    assert rc == -1 and "attention.waves" in env.nat.last_error()
 
 
 @pytest.mark.parametrize("q64", [False, True])
 @pytest.mark.parametrize("span", [20.0, 45.0, 90.0])
-def test_attention_bf16_reference_max_moves_slowly_and_fast(env, monkeypatch, span, q64):
+def test_attention_bf16_reference_max_moves_slowly_and_fast(env, knobs, span, q64):
     """Scores rise steadily along the keys by `span` nats in total over 10 tiles.  The direct kernel
     moves a row's reference max only when a tile exceeds it by 2^8: span 20 never reaches that after
     the first tile, 45 reaches it every other tile, 90 at every tile."""
     if q64:
-        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
+        knobs["attention.waves"] = "64"
     nq, nk, d = 64, 640, 64
     q = np.ones((1, nq, d), np.float32)
     k = oracle.to_bf16_f32((np.arange(nk, dtype=np.float32)[None, :, None] * np.ones((1, 1, d), np.float32))
@@ -283,12 +286,12 @@ def test_attention_bf16_reference_max_moves_slowly_and_fast(env, monkeypatch, sp
 
 @pytest.mark.parametrize("d", [64, 128, "64 (64 queries per wave)"])
 @pytest.mark.parametrize("jump_tile", [1, 6, 11])
-def test_attention_bf16_score_jump_overflows_the_stale_reference(env, monkeypatch, d, jump_tile):
+def test_attention_bf16_score_jump_overflows_the_stale_reference(env, knobs, d, jump_tile):
     """All scores are ~0 except in one key tile, where they are ~+300 nats: exp against the reference of the
     earlier tiles overflows to inf there.  The steady-state loop takes no row max; its row-sum guard has to
     catch this before the tile's PV product and move the reference.  Rows 32.. keep small scores throughout."""
     if d == "64 (64 queries per wave)":
-        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
+        knobs["attention.waves"] = "64"
         d = 64
     nq, nk = 64, 12 * 64 + 40
     q = np.zeros((1, nq, d), np.float32)
@@ -305,13 +308,13 @@ def test_attention_bf16_score_jump_overflows_the_stale_reference(env, monkeypatc
 
 @pytest.mark.parametrize("waves,d", [("4", 128), ("8", 128), ("64", 64)])
 @pytest.mark.parametrize("offset", [-300.0, -75.0, -60.0, 0.0, 25.0, 50.0, 60.0, 80.0])
-def test_attention_bf16_scores_far_from_zero(env, monkeypatch, waves, d, offset):
+def test_attention_bf16_scores_far_from_zero(env, knobs, waves, d, offset):
     """Every score of rows 0..95 is `offset` nats plus noise.  The steady state of these kernels takes exp of the score
     as it is, with no reference: within range (-75 .. 50) it must stay accurate, and where a tile's row sum
     leaves the range (60, 80) or the whole row underflows (-300) the workgroup has to notice and compute the item
     again with the running max.  The other rows keep scores near zero, next to the affected ones in the same
     workgroup; the last query tile is a partial one."""
-    monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+    knobs["attention.waves"] = waves
     nq, nk = 300, 7 * 64 + 10
     q = oracle.to_bf16_f32(rnd((2, nq, d), 1) * 0.5)
     k = oracle.to_bf16_f32(rnd((2, nk, d), 2) * 0.5)
@@ -325,12 +328,12 @@ def test_attention_bf16_scores_far_from_zero(env, monkeypatch, waves, d, offset)
 
 
 @pytest.mark.parametrize("d,waves", [(128, "8"), (64, "8"), (64, "64")])
-def test_attention_bf16_large_scores_error_growth(env, monkeypatch, d, waves):
+def test_attention_bf16_large_scores_error_growth(env, knobs, d, waves):
     """The direct kernels fold scale * log2(e) into Q, rounded to bf16 once more: a perturbation of the scores that
     grows with their magnitude.  Inputs x 1, x 2 (the recipe of the long-sequence configuration) and x 3 (scores of
     +-35 nats, far more peaked than attention): the error against the f64 closed form stays below 1e-2, 1.5e-2
     and 3e-2 of max |reference|; the last is looser than the 2e-2 bar of the other tests and states where it ends."""
-    monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+    knobs["attention.waves"] = waves
     bh, nq, nk = 2, 200, 1100
     for amp, bound in ((1.0, 1e-2), (2.0, 1.5e-2), (3.0, 3e-2)):
         q, k, v = (oracle.to_bf16_f32(rnd((bh, n, d), s) * np.float32(amp)) for s, n in ((1, nq), (2, nk), (3, nk)))
@@ -378,9 +381,9 @@ def test_attention_bf16_every_schedule_tile_vs_oracle(env, d, query_tile, key_ti
 
 
 @pytest.mark.parametrize("q64", [False, True])
-def test_attention_bf16_direct_negative_and_zero_scale(env, monkeypatch, q64):
+def test_attention_bf16_direct_negative_and_zero_scale(env, knobs, q64):
     if q64:
-        monkeypatch.setenv("ILANG_ATTN_WAVES", "64")
+        knobs["attention.waves"] = "64"
     q, k, v = (oracle.to_bf16_f32(rnd((2, n, 64), s)) for s, n in ((1, 70), (2, 400), (3, 400)))
     for scale in (-0.3, 0.0):
         ref = oracle.np_attention64(q, k, v, scale).astype(np.float32)
@@ -399,10 +402,10 @@ def test_attention_bf16_config4_slice_vs_oracle(env):
 
 
 @pytest.mark.parametrize("waves", ["8", "64"])
-def test_attention_bf16_long_sequence_rescale_stress(env, monkeypatch, waves):
+def test_attention_bf16_long_sequence_rescale_stress(env, knobs, waves):
     """Config 5 recipe (inputs x2.0, d=64) at N=8192: heavy running-max movement; the 8-wave kernel and the
     64-queries-per-wave kernel that the launcher picks at the full size."""
-    monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+    knobs["attention.waves"] = waves
     n, d = 8192, 64
     q, k, v = (oracle.to_bf16_f32(rnd((1, n, d), s) * 2.0) for s in (1, 2, 3))
     scale = float(np.float32(1.0 / np.sqrt(d)))
@@ -482,13 +485,13 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
                                       (3, 257, 255, 320)])
 @pytest.mark.parametrize("direct", ["256", "256w8", "128", "0"])
-def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
+def test_gemm_nt_bf16_every_kernel_vs_oracle(env, knobs, bh, m, n, k, direct):
     """The launcher picks between the 256 x 256 (four waves; "w8": the form with eight) and 128 x 128
     direct-to-LDS kernels and the register-staged kernel by problem size; force each of them on small ragged
     problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct[:3])
+    gemm_kernel_knobs(knobs, direct[:3])
     if direct.endswith("w8"):
-        monkeypatch.setenv("ILANG_GEMM_WAVES", "8")
+        knobs["gemm.waves"] = 8
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -503,12 +506,12 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, monkeypatch, bh, m, n, k, dire
                                       (1, 128, 128, 72)])
 @pytest.mark.parametrize("nn", [False, True])
 @pytest.mark.parametrize("tile", ["128", "256", "256w8"])
-def test_gemm_bf16_k_that_is_no_multiple_of_64(env, monkeypatch, bh, m, n, k, nn, tile):
+def test_gemm_bf16_k_that_is_no_multiple_of_64(env, knobs, bh, m, n, k, nn, tile):
     """k % 8 == 0 but k % 64 != 0: the direct kernels with a partial last slab (the lanes past k clear their LDS
     slots), both tile sizes (and both forms of the larger) forced here at small sizes; NT and NN, f32 and bf16 output."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile[:3])
+    gemm_kernel_knobs(knobs, tile[:3])
     if tile.endswith("w8"):
-        monkeypatch.setenv("ILANG_GEMM_WAVES", "8")
+        knobs["gemm.waves"] = 8
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -530,12 +533,12 @@ def test_gemm_bf16_k_that_is_no_multiple_of_64(env, monkeypatch, bh, m, n, k, nn
         assert t.equal(c16, cd.bfloat16())
 
 
-def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, monkeypatch):
+def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, knobs):
     """The four-wave form of the 256 x 256 tile spells its matrix instructions as inline assembly and carries its own
     wait states.  Its first matrix instructions multiply zeroed operands; issued too soon after the zeroing they read
     what the registers held before, which is visible when that was NaN: products of NaN operands run first here, so
     that the register file is full of NaN, then several small multi-batch products (many short-lived workgroups)."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", "256")
+    gemm_kernel_knobs(knobs, "256")
     t = env.torch
     poison = t.full((2048, 512), float("nan"), device="cuda", dtype=t.bfloat16)
     sink = t.empty(2048, 2048, device="cuda")
@@ -558,12 +561,12 @@ def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, monke
 
 
 @pytest.mark.parametrize("tile", [0, 128, 256])
-def test_gemm_nt_bf16_output_in_bf16(env, monkeypatch, tile):
+def test_gemm_nt_bf16_output_in_bf16(env, knobs, tile):
     """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
-    result rounded to bf16, bit for bit, for the register-staged kernel (ILANG_GEMM_DIRECT=0) and both tiles."""
+    result rounded to bf16, bit for bit, for the register-staged kernel (gemm.direct=0) and both tiles."""
     t = env.torch
     if tile == 0:
-        monkeypatch.setenv("ILANG_GEMM_DIRECT", "0")
+        gemm_kernel_knobs(knobs, "0")
     for bh, m, n, k in ((2, 300, 260, 128), (1, 512, 512, 576), (3, 1, 1, 64)):
         a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
         b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -606,10 +609,10 @@ def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 264, 128), (2, 600, 520, 192), (1, 1, 8, 256),
                                       (3, 257, 248, 320), (1, 130, 1000, 64)])
 @pytest.mark.parametrize("direct", ["256", "128"])
-def test_gemm_nn_bf16_vs_oracle(env, monkeypatch, bh, m, n, k, direct):
+def test_gemm_nn_bf16_vs_oracle(env, knobs, bh, m, n, k, direct):
     """Row-major right operand (c = a b, b [k, n]) on the direct kernels: 1 to 5 k-slabs, edge tiles on both
     axes (n a multiple of 8 only), several batches, both workgroup tiles."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
+    gemm_kernel_knobs(knobs, direct)
     t = env.torch
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, k, n), 2, "uniform"))
@@ -634,9 +637,9 @@ def test_gemm_nn_bf16_rejects_what_the_direct_kernels_cannot_read(env):
                                       # k a multiple of 4 but not of 32: a partial last slab
                                       (1, 256, 256, 40), (2, 300, 260, 100), (1, 100, 70, 4), (3, 257, 255, 1004), (1, 64, 64, 28)])
 @pytest.mark.parametrize("tile", ["256", "128"])
-def test_gemm_nt_f32_vs_oracle(env, monkeypatch, bh, m, n, k, tile):
+def test_gemm_nt_f32_vs_oracle(env, knobs, bh, m, n, k, tile):
     """f32 operands, f32 MFMA: the reference's own arithmetic type, against the scalar oracle at the f32 bar."""
-    monkeypatch.setenv("ILANG_GEMM_DIRECT", tile)
+    gemm_kernel_knobs(knobs, tile)
     t = env.torch
     a, b = rnd((bh, m, k), 1, "uniform"), rnd((bh, n, k), 2, "uniform")
     ad, bd = t.from_numpy(a).cuda(), t.from_numpy(b).cuda()

@@ -8,6 +8,8 @@ import random
 
 import pytest
 
+from conftest import gemm_kernel_knobs
+
 pytestmark = pytest.mark.gpu
 
 
@@ -21,14 +23,16 @@ def env():
     class Env:
         pass
 
+    from conftest import NativeWithKnobs
+
     e = Env()
-    e.torch, e.nat = torch, nat
+    e.torch, e.nat = torch, NativeWithKnobs(nat)
     e.stream = lambda: torch.cuda.current_stream().cuda_stream
     return e
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])
-def test_attention_bf16_random_shapes(env, monkeypatch, seed):
+def test_attention_bf16_random_shapes(env, knobs, seed):
     t, nat = env.torch, env.nat
     rng = random.Random(seed)
     for case in range(40):
@@ -39,9 +43,9 @@ def test_attention_bf16_random_shapes(env, monkeypatch, seed):
         waves = rng.choice([None, "4", "8"] + (["64"] if d == 64 else []))
         amp = rng.choice([0.5, 1.0, 2.0])
         if waves:
-            monkeypatch.setenv("ILANG_ATTN_WAVES", waves)
+            knobs["attention.waves"] = waves
         else:
-            monkeypatch.delenv("ILANG_ATTN_WAVES", raising=False)
+            knobs.pop("attention.waves", None)
         g = t.Generator(device="cuda").manual_seed(1000 * seed + case)
         q, k, v = ((amp * t.randn(bh, n, d, device="cuda", generator=g)).bfloat16() for n in (nq, nk, nk))
         scale = d ** -0.5
@@ -56,7 +60,7 @@ def test_attention_bf16_random_shapes(env, monkeypatch, seed):
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])
-def test_gemm_bf16_random_shapes(env, monkeypatch, seed):
+def test_gemm_bf16_random_shapes(env, knobs, seed):
     t, nat = env.torch, env.nat
     rng = random.Random(seed)
     for case in range(40):
@@ -69,9 +73,9 @@ def test_gemm_bf16_random_shapes(env, monkeypatch, seed):
             n = max(8, n // 8 * 8)
         direct = rng.choice([None, "256", "128"] + ([] if nn else ["0"]))
         if direct:
-            monkeypatch.setenv("ILANG_GEMM_DIRECT", direct)
+            gemm_kernel_knobs(knobs, direct)
         else:
-            monkeypatch.delenv("ILANG_GEMM_DIRECT", raising=False)
+            knobs.pop("gemm.tile", None); knobs.pop("gemm.direct", None)
         g = t.Generator(device="cuda").manual_seed(1000 * seed + case)
         a = (t.rand(bh, m, k, device="cuda", generator=g) * 2 - 1).bfloat16()
         b = (t.rand(*((bh, k, n) if nn else (bh, n, k)), device="cuda", generator=g) * 2 - 1).bfloat16()

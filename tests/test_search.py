@@ -4,7 +4,7 @@ import pytest
 
 import oracle
 from i_amd import Component as i
-from i_amd.search import Result, grid, search
+from i_amd.search import Result, grid, option_grid, search
 
 
 def test_grid_enumerates_split_strings():
@@ -16,6 +16,87 @@ def test_grid_enumerates_split_strings():
         primes = "i'i''" if "16:8" in split else "i'"
         comp = i(f"ik*jk~ijk | {split} | ji{primes}j'k") >> i(f"+ijk~ij | {split} | ji{primes}j'k0")
         assert "hand-written MFMA GEMM" in comp._code()
+
+
+def test_option_grid_enumerates_program_options():
+    assert option_grid({"gemm.k_parts": [1, 4], "gemm.waves": [4, 8]}) == [
+        {"gemm.k_parts": 1, "gemm.waves": 4}, {"gemm.k_parts": 1, "gemm.waves": 8},
+        {"gemm.k_parts": 4, "gemm.waves": 4}, {"gemm.k_parts": 4, "gemm.waves": 8}]
+    assert option_grid({}) == [{}]
+    # every name is one the compiled program knows; a wrong one or a wrong value is refused with its name
+    comp = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    for name, value in (("gemm.k_parts", 8), ("gemm.tile", 128), ("gemm.waves", 8), ("gemm.direct", 0), ("attention.kv_parts", 3),
+                        ("attention.waves", 64), ("attention.direct", 0), ("attention.f32_scale", 1), ("generated.only", 1),
+                        ("generated.wave", -1)):
+        comp.option(name, value)
+    for name, value, text in (("gemm.kparts", 2, "unknown program option"), ("gemm.tile", 64, "0, 128 or 256"),
+                              ("attention.waves", 3, "attention.waves"), ("gemm.k_parts", -1, "gemm.k_parts")):
+        with pytest.raises(RuntimeError, match=text):
+            comp.option(name, value)
+
+
+@pytest.mark.gpu
+def test_search_over_the_parts_of_a_split_loop():
+    """What a schedule has no spelling for is searched as program options: the number of parts the k loop of a product
+    with few output tiles (64 x 8192 x 8192) is cut into, and the number of parts of the keys of one head of 8192,
+    each ranked by device time with the C the reference backend emits as the referee (on a slice of the result)."""
+    import torch
+
+    from i_amd import I
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = (torch.rand(64, 8192, device="cuda", generator=g) * 2 - 1).bfloat16()
+    b = (torch.rand(8192, 8192, device="cuda", generator=g) * 2 - 1).bfloat16()
+
+    def mm_t(split):
+        return i(f"ik*jk~ijk | {split} | jii'j'k") >> i(f"+ijk~ij | {split} | jii'j'k0")
+
+    cols = slice(4000, 4032)
+
+    def referee(a_, b_):
+        comp = mm_t("i:16,j:16")
+        out = oracle.compile_component(comp.handle).run(a_.float().cpu().numpy(), np.ascontiguousarray(b_[cols].float().cpu().numpy()))
+        return torch.from_numpy(out).cuda()
+
+    ranked = search(mm_t, ["i:16,j:16"], inputs=(a, b), rtol=1e-2, referee=referee, repeats=7, view=lambda c: c[:, cols],
+                    options=option_grid({"gemm.k_parts": [1, 2, 4, 8, 16, 32]}))
+    assert all(r.failure is None for r in ranked), [(r.options, r.failure, r.error) for r in ranked]
+    assert len({r.options["gemm.k_parts"] for r in ranked}) >= 4 and ranked == sorted(ranked, key=lambda r: r.ms)
+    by = {r.options["gemm.k_parts"]: r for r in ranked}
+    assert "parts)" not in by[1].kernels and "(k in 8 parts)" in by[8].kernels
+    assert ranked[0].options["gemm.k_parts"] > 1 and ranked[0].ms < by[1].ms  # 32 output tiles for 256 CUs: some split wins
+    # the launcher's own choice (no option set) is within 25 % of the best of the search
+    own = search(mm_t, ["i:16,j:16"], inputs=(a, b), rtol=1e-2, referee=referee, repeats=7, view=lambda c: c[:, cols])[0]
+    assert own.ms <= 1.25 * ranked[0].ms, (own.ms, own.kernels, ranked[0].ms, ranked[0].options)
+
+    q, k, v = (torch.randn(1, 8192, 128, device="cuda", generator=g).bfloat16() for _ in range(3))
+    scale = torch.tensor(np.float32(128 ** -0.5), device="cuda")
+
+    def attn(split):
+        p = "b"
+        first = i(f"{p}ik*{p}jk~{p}ijk | {split} | {p}jii'j'k") >> i(f"+{p}ijk~{p}ij | {split} | {p}jii'j'k0")
+        sc = i(f"{p}ij*.~{p}ij | {split} | {p}ji0i'j'")
+        shift = (I & i(f">{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij-{p}i~{p}ij | {split} | {p}ji01i'j'")
+        ex = i(f"^{p}ij~{p}ij | {split} | {p}ji0i'j'")
+        norm = (I & i(f"+{p}ij~{p}i | {split} | {p}ji0i'j'")) >> i(f"{p}ij/{p}i~{p}ij | {split} | {p}ji01i'j'")
+        last = i(f"{p}ij*{p}jk~{p}ikj | {split} | {p}ji0i'kj'") >> i(f"+{p}ikj~{p}ik | {split} | {p}jii'kj'0")
+        return first >> sc >> shift >> ex >> norm >> last
+
+    rows = slice(5000, 5032)
+
+    def attn_referee(q_, k_, s_, v_):
+        comp = attn("i:16,j:16")
+        out = oracle.compile_component(comp.handle).run(np.ascontiguousarray(q_[:, rows].float().cpu().numpy()), k_.float().cpu().numpy(),
+                                                        np.float32(s_.item()), v_.float().cpu().numpy())
+        return torch.from_numpy(out).cuda()
+
+    ranked = search(attn, ["i:128,j:64"], inputs=(q, k, scale, v), rtol=2e-2, referee=attn_referee, repeats=7,
+                    view=lambda o: o[:, rows], options=option_grid({"attention.kv_parts": [1, 2, 4, 8, 16]}))
+    assert all(r.failure is None for r in ranked), [(r.options, r.failure, r.error) for r in ranked]
+    assert len({r.options["attention.kv_parts"] for r in ranked}) >= 4 and ranked == sorted(ranked, key=lambda r: r.ms)
+    by = {r.options["attention.kv_parts"]: r for r in ranked}
+    assert "keys in" not in by[1].kernels and "(keys in 4 parts)" in by[4].kernels
+    assert ranked[0].options["attention.kv_parts"] > 1 and ranked[0].ms < by[1].ms  # 64 query tiles for 256 CUs
 
 
 @pytest.mark.gpu

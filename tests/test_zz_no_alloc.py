@@ -100,7 +100,7 @@ def test_split_loops_keep_their_partial_results_in_the_workspace(torch, monkeypa
                  >> ((I & i(f">ij~i | {s} | ji0i'j'")) >> i(f"ij-i~ij | {s} | ji01i'j'")) >> i(f"^ij~ij | {s} | ji0i'j'")
                  >> ((I & i(f"+ij~i | {s} | ji0i'j'")) >> i(f"ij/i~ij | {s} | ji01i'j'"))
                  >> (i(f"ij*jk~ikj | {s} | ji0i'kj'") >> i(f"+ikj~ik | {s} | jii'kj'0")))
-    monkeypatch.setenv("ILANG_ATTN_KV_SPLITS", "3")
+    attention.option("attention.kv_parts", 3)
     for nq, nk, d in ((300, 2500, 128), (70, 1000, 64)):
         print("case split attention", (nq, nk, d), flush=True)
         q, k, v = (randn(torch, shape, seed, torch.bfloat16) for seed, shape in ((9, (nq, d)), (10, (nk, d)), (11, (nk, d))))
