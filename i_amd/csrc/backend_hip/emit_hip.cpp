@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <functional>
 #include <map>
 #include <set>
 #include <sstream>
@@ -202,14 +203,38 @@ void loop_ids(const Block<Param>& block, std::set<size_t>& ids) {
 // inside L becomes that variable, and it is stored back after L.  (As printed by the C backend the element
 // makes a round trip through memory in every iteration, which serialises the loop on the latency of that trip.)
 // Buffers of one kernel never overlap: a kernel's readonlys and writeables are disjoint sets of distinct buffers.
+// Loops in `parallel` are the work-item index space: their iterators are fixed inside a work-item, so an index that
+// one of them takes part in still names one element (a column sum with the row loop outside the column loop keeps
+// each work-item's column total in a register across the rows).  A parallel loop with a tail guard below the
+// loop in question is no such loop: the guard sits inside, and a load hoisted above it would run for the tail's
+// work-items too.
 // Result: loop id -> writeable indexes.
-void held_elements(const Block<Param>& block, std::map<size_t, std::vector<size_t>>& out) {
+void held_elements(const Block<Param>& block, const std::set<size_t>& parallel, std::map<size_t, std::vector<size_t>>& out) {
   for (const PAct& loop : block) {
     if (loop.kind != PAct::Loop) continue;
+    if (parallel.count(loop.id)) {
+      held_elements(loop.body, parallel, out);
+      continue;
+    }
     Uses u;
     collect(loop.body, u);
     std::set<size_t> inner{loop.id};
     loop_ids(loop.body, inner);
+    {
+      std::set<size_t> guarded;
+      std::vector<const Block<Param>*> todo{&loop.body};
+      while (!todo.empty()) {
+        const Block<Param>* b = todo.back();
+        todo.pop_back();
+        for (const PAct& a : *b)
+          if (a.kind == PAct::Loop) {
+            if (a.guard) guarded.insert(a.id);
+            todo.push_back(&a.body);
+          }
+      }
+      for (size_t id : parallel)
+        if (!guarded.count(id)) inner.erase(id);
+    }
     for (const Param& w : u.written) {
       const Access<Param>* first = nullptr;
       bool ok = w.writeable;
@@ -221,7 +246,7 @@ void held_elements(const Block<Param>& block, std::map<size_t, std::vector<size_
       for (size_t id : inner) ok = ok && first && !access_uses(*first, id);
       if (ok) out[loop.id].push_back(w.ind);
     }
-    held_elements(loop.body, out);
+    held_elements(loop.body, parallel, out);
   }
 }
 
@@ -476,7 +501,20 @@ struct Printer {
   std::set<std::string> parallel;  // iterator names handled by the work-item decomposition
   const std::map<size_t, std::vector<size_t>>* held = nullptr;  // loop id -> elements to hold in registers (held_elements)
   const std::vector<WaveLoop>* wave = nullptr;  // the wavefront-per-iteration form: loops spread over the lanes
+  const GridForm* grid = nullptr;               // the form with a loop in parts: `part` of `parts` takes its share of grid->loop
   int serial_depth = 0;                         // loops being printed as loops around the current statement
+  // In the form with a loop in parts every part accumulates into copies of the accumulated buffers that the
+  // launcher has filled with the reduction's identity: the nest's own initialisations of those buffers are dropped.
+  bool dropped_initialisation(const MStmt& s) const {
+    if (!grid || s.kind != MStmt::Set || !s.value || s.value->kind != MExpr::Scalar) return false;
+    std::string cap;
+    bool writeable = false;
+    size_t ind = 0;
+    if (!buffer_access(*s.dst, &cap, &writeable, &ind) || !writeable) return false;
+    for (const GridAccumulator& acc : grid->accumulators)
+      if (acc.writeable == ind) return true;
+    return false;
+  }
   static const char* identity_text(Op op) {
     return op == Op::Mul ? "1.0f" : op == Op::Max ? "(-INFINITY)" : op == Op::Min ? "INFINITY" : "0.0f";
   }
@@ -491,9 +529,10 @@ struct Printer {
   void uniform_statement_done(int depth) {
     if (wave && serial_depth == 0) line(depth, "ILANG_WAVE_SYNC();");
   }
-  static bool innermost(const std::vector<MStmt>& body) {
+  // no loop below that is printed as a loop (the parallel ones are the work-item's coordinates)
+  bool innermost(const std::vector<MStmt>& body) const {
     for (const MStmt& s : body)
-      if (s.kind == MStmt::Loop || !innermost(s.body)) return false;
+      if ((s.kind == MStmt::Loop && !parallel.count(s.ident)) || !innermost(s.body)) return false;
     return true;
   }
   void line(int depth, const std::string& s) { os << std::string(2 * depth, ' ') << s << "\n"; }
@@ -504,6 +543,7 @@ struct Printer {
     switch (s.kind) {
       case MStmt::Set: {
         std::string cap;
+        if (dropped_initialisation(s)) break;
         if (const std::string* local = held_local(*s.dst)) {
           line(depth, *local + " = " + expr_text(*s.value) + ";");
         } else if (g_checked_accesses && buffer_access(*s.dst, &cap)) {
@@ -546,12 +586,18 @@ struct Printer {
           const int d = mine.empty() ? depth : depth + 1;
           if (!mine.empty()) line(depth, "{");
           for (const Held& h : mine) {
+            // (in the form with a loop in parts an accumulated element starts as the reduction's identity: what its
+            // copy holds is not read, so the copies need no filling when every accumulator is held this way)
+            const GridAccumulator* fresh = nullptr;
+            if (grid && grid->held_accumulators)
+              for (const GridAccumulator& acc : grid->accumulators)
+                if (acc.writeable == h.ind) fresh = &acc;
             if (h.shared) {
               // the element as it is before the loop, and this lane's share of what the loop adds to it
-              line(d, "const float before_" + h.local + " = " + expr_text(*h.at) + ";");
+              line(d, "const float before_" + h.local + " = " + (fresh ? std::string(identity_text(fresh->op)) : expr_text(*h.at)) + ";");
               line(d, "float " + h.local + " = " + identity_text(h.op) + ";");
             } else {
-              line(d, "float " + h.local + " = " + expr_text(*h.at) + ";");
+              line(d, "float " + h.local + " = " + (fresh ? std::string(identity_text(fresh->op)) : expr_text(*h.at)) + ";");
             }
           }
           for (const Held& h : mine) g_held[h.ind] = h.local;
@@ -561,9 +607,20 @@ struct Printer {
           // an innermost loop that only accumulates into registers: unrolled, so that the loads of several
           // iterations are in flight at once (measured on row sums: 2.1 -> 3.8 TB/s in the wavefront form, 0.6 -> 1.0
           // with a work-item per row)
-          if ((spread || !mine.empty()) && innermost(s.body)) line(d, "#pragma unroll 4");
-          if (spread)
+          // part p takes a run of consecutive iterations of this loop (consecutive rows stay within a page)
+          const bool in_parts = grid && grid->loop == loop_id;
+          if (in_parts) {
+            line(d, "const size_t share_" + s.ident + " = (" + expr_text(*s.value) + " + parts - 1) / parts;");
+            line(d, "const size_t end_" + s.ident + " = (part + 1) * share_" + s.ident + " < " + expr_text(*s.value) + " ? (part + 1) * share_" +
+                        s.ident + " : " + expr_text(*s.value) + ";");
+          }
+          if ((spread || !mine.empty()) && innermost(s.body)) line(d, "#pragma unroll 8");
+          if (spread && in_parts)
+            line(d, "for (size_t " + s.ident + " = part * share_" + s.ident + " + lane; " + s.ident + " < end_" + s.ident + "; " + s.ident + " += 64) {");
+          else if (spread)
             line(d, "for (size_t " + s.ident + " = lane; " + s.ident + " < " + expr_text(*s.value) + "; " + s.ident + " += 64) {");
+          else if (in_parts)
+            line(d, "for (size_t " + s.ident + " = part * share_" + s.ident + "; " + s.ident + " < end_" + s.ident + "; ++" + s.ident + ") {");
           else
             line(d, "for (size_t " + s.ident + " = 0; " + s.ident + " < " + expr_text(*s.value) + "; ++" + s.ident + ") {");
           ++serial_depth;
@@ -609,7 +666,200 @@ const MStmt* find_loop(const std::vector<MStmt>& stmts, const std::string& iter)
   return nullptr;
 }
 
+// ------------------------------------------------------------------ one kernel per loop nest
+void visit_scalar_params(ScalarExpr<Param>& e, const std::function<void(Param&)>& f) {
+  if (e.kind == ScalarExpr<Param>::Acc) f(e.access.buffer);
+  for (auto& a : e.args) visit_scalar_params(a, f);
+}
+// every reference to a kernel parameter in a block: accesses, and the buffers whose extents bound the loops
+void visit_params(Block<Param>& block, const std::function<void(Param&)>& f) {
+  for (PAct& a : block) {
+    switch (a.kind) {
+      case PAct::Loop:
+        f(a.extent.source.buffer);
+        visit_params(a.body, f);
+        break;
+      case PAct::Init: f(a.write.buffer); break;
+      case PAct::Compute:
+      case PAct::Snapshot:
+        f(a.write.buffer);
+        for (auto& r : a.reads) f(r.buffer);
+        break;
+      case PAct::Scale:
+        f(a.write.buffer);
+        visit_scalar_params(a.factor, f);
+        break;
+    }
+  }
+}
+
+// The form of a nest with its outermost sequential loop in parts (GridForm), or nothing when the nest does not
+// qualify.  Walking down from the top of the body, through the parallel loops, the first sequential loop G is the
+// one in parts; on the way there may only be initialisations.  Under G there are only loops, initialisations
+// (checked for the first iteration of the loops they sit in) and Computes, and every Compute either stores into a
+// work-item-private buffer or accumulates (+, *, max, min) into a buffer that nothing under G reads: then part p
+// may run iterations p, p + parts, ... of G on a copy of each accumulated buffer that starts as the reduction's
+// identity, and the copies fold into the buffer afterwards, element by element, in part order.
+void grid_plan(const Block<Param>& body, const std::set<Param>& accumulating, const std::map<size_t, std::vector<size_t>>& held,
+               GenericPhase& phase) {
+  auto is_parallel = [&](size_t id) { return std::find(phase.parallel_loops.begin(), phase.parallel_loops.end(), id) != phase.parallel_loops.end(); };
+  auto is_private = [&](const Param& w) {
+    if (!w.writeable) return false;
+    for (const PrivateBuffer& pb : phase.privates)
+      if (pb.writeable == w.ind) return true;
+    return false;
+  };
+  std::set<Param> initialised_here;
+  const Block<Param>* block = &body;
+  const PAct* g = nullptr;
+  while (!g) {
+    const PAct* only = nullptr;
+    for (const PAct& a : *block) {
+      if (a.kind == PAct::Loop) {
+        if (only) return;
+        only = &a;
+      } else if (a.kind == PAct::Init) {
+        initialised_here.insert(a.write.buffer);
+      } else {
+        return;
+      }
+    }
+    if (!only) return;
+    if (is_parallel(only->id)) block = &only->body;
+    else g = only;
+  }
+  std::map<Param, Op> ops;
+  std::vector<const PAct*> computes;
+  std::vector<const Block<Param>*> todo{&g->body};
+  while (!todo.empty()) {
+    const Block<Param>* b = todo.back();
+    todo.pop_back();
+    for (const PAct& a : *b) {
+      if (a.kind == PAct::Loop) todo.push_back(&a.body);
+      else if (a.kind == PAct::Init) initialised_here.insert(a.write.buffer);
+      else if (a.kind == PAct::Compute) computes.push_back(&a);
+      else return;
+    }
+  }
+  for (const PAct* c : computes) {
+    const Param w = c->write.buffer;
+    if (is_private(w)) continue;
+    const bool known = c->op == Op::Add || c->op == Op::Mul || c->op == Op::Max || c->op == Op::Min;
+    if (!w.writeable || !accumulating.count(w) || !known) return;
+    auto [it, fresh] = ops.emplace(w, c->op);
+    if (!fresh && it->second != c->op) return;
+  }
+  if (ops.empty()) return;
+  for (const PAct* c : computes)
+    for (const auto& r : c->reads)
+      if (ops.count(r.buffer)) return;
+  for (const Param& w : initialised_here)
+    if (!ops.count(w)) return;  // (an initialisation of something that is no accumulator of this nest)
+  phase.grid.available = true;
+  phase.grid.loop = g->id;
+  phase.grid.extent = g->extent;
+  for (const auto& [w, op] : ops) phase.grid.accumulators.push_back({w.ind, op, initialised_here.count(w) != 0});
+  // every accumulator kept in a register across G (and nowhere else under it: held by G itself): the parts then
+  // never read their copies, they only store into them
+  const auto held_by_g = held.find(g->id);
+  phase.grid.held_accumulators = held_by_g != held.end();
+  for (const auto& [w, op] : ops)
+    phase.grid.held_accumulators = phase.grid.held_accumulators &&
+                                   std::find(held_by_g->second.begin(), held_by_g->second.end(), w.ind) != held_by_g->second.end();
+  // the wavefront form of the same: when the nest has one and G is its loop over (or around) the lanes
+  for (const WaveLoop& wl : phase.wave_loops)
+    if (wl.loop == g->id && !wl.accumulators.empty()) {
+      phase.grid.wave = true;
+      phase.grid.loop_is_spread = wl.spread == g->id;
+    }
+  if (phase.wave_loops.size() != 1) phase.grid.wave = false;
+}
+
 }  // namespace
+
+ExecPlan split_nests(const ExecPlan& plan, std::vector<size_t>* origin) {
+  ExecPlan out = plan;
+  out.kernels.clear();
+  out.exec.clear();
+  origin->clear();
+  std::vector<std::vector<size_t>> pieces_of(plan.kernels.size());   // new kernel ids per old kernel
+  std::vector<std::vector<std::vector<size_t>>> kept_reads, kept_writes;  // per new kernel: positions in the old lists
+  for (size_t k = 0; k < plan.kernels.size(); ++k) {
+    const Kernel<Param>& kernel = plan.kernels[k];
+    std::set<Param> initialised;
+    collect_initialized(kernel.body, initialised);
+    initialised.insert(kernel.accumulates.begin(), kernel.accumulates.end());
+    // a run of statements that are no loops goes with the loop after it when that loop writes what the run
+    // initialises (a scalar total and the loop that adds to it), otherwise it is a piece of its own
+    std::vector<std::pair<size_t, size_t>> ranges;
+    for (const auto& [first, last] : phase_ranges(kernel.body)) {
+      bool joined = false;
+      if (!ranges.empty() && first < last && kernel.body[first].kind == PAct::Loop) {
+        const auto [pf, pl] = ranges.back();
+        bool run = pf < pl;
+        std::set<Param> set_by_run;
+        for (size_t n = pf; n < pl; ++n) {
+          run = run && kernel.body[n].kind == PAct::Init;
+          set_by_run.insert(kernel.body[n].write.buffer);
+        }
+        if (run) {
+          Uses u;
+          collect_one(kernel.body[first], u);
+          for (const Param& w : u.written) joined = joined || set_by_run.count(w);
+        }
+      }
+      if (joined) ranges.back().second = last;
+      else ranges.push_back({first, last});
+    }
+    for (const auto& [first, last] : ranges) {
+      Kernel<Param> piece;
+      piece.body.assign(kernel.body.begin() + first, kernel.body.begin() + last);
+      std::set<Param> used;
+      visit_params(piece.body, [&](Param& p) { used.insert(p); });
+      std::vector<size_t> reads, writes;
+      std::map<Param, Param> renamed;
+      for (size_t r = 0; r < kernel.reads.size(); ++r)
+        if (ranges.size() == 1 || used.count(Param{false, r})) {
+          renamed[Param{false, r}] = Param{false, reads.size()};
+          reads.push_back(r);
+          piece.reads.push_back(kernel.reads[r]);
+        }
+      for (size_t w = 0; w < kernel.writes.size(); ++w)
+        if (ranges.size() == 1 || used.count(Param{true, w})) {
+          renamed[Param{true, w}] = Param{true, writes.size()};
+          writes.push_back(w);
+          piece.writes.push_back(kernel.writes[w]);
+        }
+      visit_params(piece.body, [&](Param& p) {
+        auto it = renamed.find(p);
+        if (it == renamed.end()) lower_error("kernel body names a buffer that is not in its lists");
+        p = it->second;
+      });
+      for (const Param& w : initialised)
+        if (renamed.count(w)) piece.accumulates.push_back(renamed[w]);
+      pieces_of[k].push_back(out.kernels.size());
+      origin->push_back(k);
+      out.kernels.push_back(std::move(piece));
+      kept_reads.push_back({reads});
+      kept_writes.push_back({writes});
+    }
+  }
+  for (const Step& step : plan.exec) {
+    if (step.kind != Step::Dispatch) {
+      out.exec.push_back(step);
+      continue;
+    }
+    for (size_t piece : pieces_of.at(step.id)) {
+      Step s;
+      s.kind = Step::Dispatch;
+      s.id = piece;
+      for (size_t r : kept_reads[piece][0]) s.reads.push_back(step.reads.at(r));
+      for (size_t w : kept_writes[piece][0]) s.writes.push_back(step.writes.at(w));
+      out.exec.push_back(std::move(s));
+    }
+  }
+  return out;
+}
 
 GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const std::vector<bool>& emit) {
   const char* unchecked = std::getenv("ILANG_HIP_UNCHECKED");
@@ -624,7 +874,7 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
   out.rank = rank;
 
   std::ostringstream src;
-  bool any = false;
+  bool any = false, any_grid = false;
   src << "// generated by the i gfx950 backend\n#include <hip/hip_runtime.h>\n#include <math.h>\n#include <stddef.h>\n\n";
   src << "#ifndef ILANG_WAVE_SYNC\n#define ILANG_WAVE_SYNC() __builtin_amdgcn_wave_barrier()\n#endif\n\n";
   src << "struct View { float* data; size_t shape[" << rank << "]; size_t layout[" << rank << "]; };\n\n";
@@ -637,68 +887,38 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
     info.n_writes = plan.kernels[k].writes.size();
     const Block<Param>& body = plan.kernels[k].body;
     const MFn& fn = module.kernels[k];
-    std::map<size_t, std::vector<size_t>> held;
-    held_elements(body, held);
-    // one statement of the module per action of the plan kernel (a trailing return aside)
     size_t fn_stmts = fn.body.size();
     while (fn_stmts > 0 && fn.body[fn_stmts - 1].kind == MStmt::Return) --fn_stmts;
-    // A body that is a sequence of top-level statements is split into phases (one per loop nest).  Default: the
-    // phases share one launch of one workgroup with barriers between them, provided some nest has parallel loops
-    // (otherwise the kernel stays a single work-item).  ILANG_HIP_PHASES=1: one launch per phase (CPU emulation only).
-    const char* want_phases = std::getenv("ILANG_HIP_PHASES");
-    const bool separate_launches = want_phases && want_phases[0] == '1';
-    auto ranges = phase_ranges(body);
-    if (fn_stmts != body.size()) ranges = {{0, body.size()}};  // no statement-by-statement correspondence: one phase
-    auto analyze_all = [&](const std::vector<std::pair<size_t, size_t>>& rs, std::vector<Block<Param>>& bodies,
-                           std::vector<GenericPhase>& phases) {
-      // buffers touched by more than one phase stay in memory
-      std::map<Param, size_t> touched;
-      bodies.clear();
-      phases.clear();
-      for (const auto& [first, last] : rs) {
-        bodies.emplace_back(body.begin() + first, body.begin() + last);
-        Uses u;
-        collect(bodies.back(), u);
-        std::set<Param> seen;
-        for (const auto* a : u.all) seen.insert(a->buffer);
-        for (const Param& b : seen) ++touched[b];
-      }
-      std::set<Param> shared;
-      for (const auto& [b, n] : touched)
-        if (n > 1) shared.insert(b);
-      for (size_t ph = 0; ph < rs.size(); ++ph) {
-        GenericPhase phase;
-        phase.name = rs.size() == 1 || !separate_launches ? info.name : info.name + "_p" + std::to_string(ph);
-        analyze(plan, k, bodies[ph], shared, phase);
-        phases.push_back(std::move(phase));
-      }
-    };
-    std::vector<Block<Param>> bodies;
-    std::vector<GenericPhase> phases;
-    analyze_all(ranges, bodies, phases);
-    bool cooperative = false;
-    if (ranges.size() > 1 && !separate_launches) {
-      for (const GenericPhase& ph : phases) cooperative |= !ph.parallel_loops.empty();
-      if (!cooperative) {  // nothing to spread over work-items: the whole body as one phase, one work-item
-        ranges = {{0, body.size()}};
-        analyze_all(ranges, bodies, phases);
-      }
-    }
-    info.cooperative = cooperative;
+    const std::vector<MStmt> stmts(fn.body.begin(), fn.body.begin() + fn_stmts);
+
+    GenericPhase phase;
+    phase.name = info.name;
+    analyze(plan, k, body, {}, phase);
+    std::map<size_t, std::vector<size_t>> held;
+    held_elements(body, std::set<size_t>(phase.parallel_loops.begin(), phase.parallel_loops.end()), held);
+    std::set<Param> initialized;
+    collect_initialized(body, initialized);
+    initialized.insert(plan.kernels[k].accumulates.begin(), plan.kernels[k].accumulates.end());
+    wave_plan(body, initialized, held, phase);
+    grid_plan(body, initialized, held, phase);
+    any_grid = any_grid || phase.grid.available;
 
     const size_t nr = std::max<size_t>(info.n_reads, 1), nw = std::max<size_t>(info.n_writes, 1);
     src << "struct Args_" << info.name << " { View readonlys[" << nr << "]; View writeables[" << nw << "]; };\n";
+    if (phase.grid.available)
+      src << "struct Args_" << info.name << "_g { View readonlys[" << nr << "]; View writeables[" << nw << "]; float* partial[" << nw
+          << "]; size_t parts; };\n";
     const Step* dispatch = nullptr;
     for (const Step& st : plan.exec)
       if (st.kind == Step::Dispatch && st.id == k) dispatch = &st;
+    auto rank_of = [&](BufferRef r) {
+      return (r.kind == BufferRef::Input ? plan.inputs.at(r.id) : r.kind == BufferRef::Intermediate ? plan.intermediates.at(r.id)
+                                                                                                   : plan.outputs.at(r.id)).layout.size();
+    };
     // element counts of the kernel's views, for the checked accesses: the product of the layout extents (a
     // work-item-private slice or array has the same layout as the buffer it stands for)
     auto emit_capacities = [&](const std::string& pad) {
       if (!g_checked_accesses) return;
-      auto rank_of = [&](BufferRef r) {
-        return (r.kind == BufferRef::Input ? plan.inputs.at(r.id) : r.kind == BufferRef::Intermediate ? plan.intermediates.at(r.id)
-                                                                                                     : plan.outputs.at(r.id)).layout.size();
-      };
       for (size_t b = 0; dispatch && b < dispatch->reads.size(); ++b) {
         src << pad << "const size_t cap_r" << b << " = (size_t)1";
         for (size_t d = 0; d < rank_of(dispatch->reads[b]); ++d) src << " * readonlys[" << b << "].layout[" << d << "]";
@@ -710,8 +930,8 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
         src << ";\n";
       }
     };
-    // work-item-private buffers of one phase: a local array, or this work-item's slice of a device buffer
-    auto emit_privates = [&](const GenericPhase& phase, const std::string& pad) {
+    // work-item-private buffers: a local array, or this work-item's slice of a device buffer
+    auto emit_privates = [&](const std::string& pad) {
       for (const PrivateBuffer& pb : phase.privates) {
         if (pb.is_static) {
           src << pad << "float priv" << pb.writeable << "[" << pb.static_size << "];\n";
@@ -723,12 +943,13 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
         }
       }
     };
-    // the statements of one phase spread over the work-items (wi_first, wi_stride); `depth` is the indentation
-    auto emit_spread = [&](const GenericPhase& phase, const std::vector<MStmt>& stmts, int depth, bool wave = false) {
+    // the nest spread over the work-items (wi_first, wi_stride); in_parts: over (work-item, part) pairs
+    auto emit_spread = [&](int depth, bool wave, bool in_parts) {
       const std::string pad(2 * depth, ' ');
       Printer pr;
       pr.held = &held;
       if (wave) pr.wave = &phase.wave_loops;
+      if (in_parts) pr.grid = &phase.grid;
       std::vector<std::string> iters;
       for (size_t id : phase.parallel_loops) iters.push_back("i" + std::to_string(id));
       for (const std::string& it : iters) {
@@ -739,88 +960,128 @@ GenericModule emit_generic_hip(const ExecPlan& plan, const Module& module, const
       }
       src << pad << "size_t wi_total = 1;\n";
       for (const std::string& it : iters) src << pad << "wi_total *= n_" << it << ";\n";
-      src << pad << "for (size_t wi = wi_first; wi < wi_total; wi += wi_stride) {\n";
-      src << pad << "  size_t wi_rest = wi;\n";
-      for (size_t t = iters.size(); t-- > 0;) {
-        src << pad << "  const size_t " << iters[t] << " = wi_rest % n_" << iters[t] << ";";
-        src << " wi_rest /= n_" << iters[t] << ";\n";
+      // The work-item index is a number in mixed radix (the extents of the parallel loops, the last one fastest; in
+      // the form with a loop in parts the part is one more digit in front).  Its digits are taken apart once, for the
+      // first index and for the stride, and then advanced digit by digit with carries: no division in the loop.
+      std::vector<std::string> digits;  // most significant first
+      if (in_parts) {
+        src << pad << "const size_t parts = args.parts;\n";
+        for (const GridAccumulator& acc : phase.grid.accumulators) {
+          src << pad << "const size_t part_cap" << acc.writeable << " = (size_t)1";
+          for (size_t d = 0; d < rank_of(dispatch->writes[acc.writeable]); ++d)
+            src << " * writeables[" << acc.writeable << "].layout[" << d << "]";
+          src << ";\n";
+        }
+        src << pad << "const size_t n_part = parts;\n";
+        digits.push_back("part");
       }
+      for (const std::string& it : iters) digits.push_back(it);
+      const std::string all = in_parts ? "wi_total * parts" : "wi_total";
+      src << pad << "if (" << all << " == 0) return;\n";
+      if (!digits.empty()) {
+        src << pad << "size_t wi_rest = wi_first < " << all << " ? wi_first : 0, step_rest = wi_stride;\n";
+        for (size_t t = digits.size(); t-- > 0;) {
+          src << pad << "size_t at_" << digits[t] << " = wi_rest % n_" << digits[t] << "; wi_rest /= n_" << digits[t] << ";\n";
+          src << pad << "const size_t step_" << digits[t] << " = step_rest % n_" << digits[t] << "; step_rest /= n_" << digits[t] << ";\n";
+        }
+      }
+      src << pad << "for (size_t wi = wi_first; wi < " << all << "; wi += wi_stride) {\n";
+      for (const std::string& dg : digits) src << pad << "  const size_t " << dg << " = at_" << dg << ";\n";
+      if (in_parts)  // this part's copy of every accumulated buffer stands where the buffer stood
+        for (const GridAccumulator& acc : phase.grid.accumulators)
+          src << pad << "  writeables[" << acc.writeable << "].data = args.partial[" << acc.writeable << "] + part * part_cap"
+              << acc.writeable << ";\n";
       pr.block(stmts, depth + 1);
       src << pr.os.str();
+      if (!digits.empty()) {
+        src << pad << "  {\n" << pad << "    size_t carry = 0;\n";
+        for (size_t t = digits.size(); t-- > 0;) {
+          src << pad << "    at_" << digits[t] << " += step_" << digits[t] << " + carry;\n";
+          src << pad << "    carry = at_" << digits[t] << " >= n_" << digits[t] << " ? 1 : 0;\n";
+          src << pad << "    if (carry) at_" << digits[t] << " -= n_" << digits[t] << ";\n";
+        }
+        src << pad << "  }\n";
+      }
       src << pad << "}\n";
     };
-    auto phase_stmts = [&](size_t ph) {
-      return std::vector<MStmt>(fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].first : 0),
-                                fn.body.begin() + (fn_stmts == body.size() ? ranges[ph].second : fn_stmts));
-    };
-    if (cooperative) {
-      src << "extern \"C\" __global__ void __launch_bounds__(" << GenericKernel::kCooperativeThreads << ") " << info.name
-          << "(Args_" << info.name << " args) {\n";
+    // forms: the nest as it is; _w: a wavefront per work-item; _g / _gw: either with the outermost sequential loop in parts
+    struct Form { bool wave, in_parts; const char* suffix; };
+    for (const Form form : {Form{false, false, ""}, Form{true, false, "_w"}, Form{false, true, "_g"}, Form{true, true, "_gw"}}) {
+      if (form.wave && !form.in_parts && phase.wave_loops.empty()) continue;
+      if (form.in_parts && (!phase.grid.available || (form.wave && !phase.grid.wave))) continue;
+      src << "extern \"C\" __global__ void __launch_bounds__(" << (form.wave ? GenericPhase::kWaveThreads : 64u) << ") " << phase.name
+          << form.suffix << "(Args_" << info.name << (form.in_parts ? "_g" : "") << " args) {\n";
       src << "  const View* readonlys = args.readonlys;\n";
       src << "  View writeables[" << nw << "];\n";
       src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
-      src << "  // one workgroup: every loop nest below is spread over its work-items, a barrier orders the nests\n";
-      src << "  const size_t wi_first = threadIdx.x;\n";
-      src << "  const size_t wi_stride = blockDim.x;\n";
+      if (form.wave) {
+        src << "  const size_t lane = threadIdx.x % 64;\n";
+        src << "  const size_t wi_first = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;\n";
+        src << "  const size_t wi_stride = ((size_t)gridDim.x * blockDim.x) / 64;\n";
+      } else {
+        src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
+        src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
+      }
       emit_capacities("  ");
-      for (size_t ph = 0; ph < ranges.size(); ++ph) {
-        if (ph > 0) src << "  __syncthreads();\n";
-        src << "  {\n";
-        emit_privates(phases[ph], "    ");
-        if (phases[ph].parallel_loops.empty()) {
-          src << "    if (wi_first == 0) {\n";
-          Printer pr;
-      pr.held = &held;
-          pr.block(phase_stmts(ph), 3);
-          src << pr.os.str();
-          src << "    }\n";
-        } else {
-          emit_spread(phases[ph], phase_stmts(ph), 2);
-        }
-        src << "  }\n";
+      emit_privates("  ");
+      if (phase.parallel_loops.empty() && !form.in_parts) {
+        src << "  if (wi_first != 0) return;\n";
+        Printer pr;
+        pr.held = &held;
+        if (form.wave) pr.wave = &phase.wave_loops;
+        pr.block(stmts, 1);
+        src << pr.os.str();
+      } else {
+        emit_spread(1, form.wave, form.in_parts);
       }
       src << "}\n\n";
-      for (auto& ph : phases) info.phases.push_back(std::move(ph));
-      continue;
     }
-    std::set<Param> initialized;
-    collect_initialized(body, initialized);
-    for (size_t ph = 0; ph < ranges.size(); ++ph) {
-      GenericPhase& phase = phases[ph];
-      wave_plan(bodies[ph], initialized, held, phase);
-      const std::vector<MStmt> stmts = phase_stmts(ph);
-      // wave: one wavefront per iteration of the parallel loops (<name>_w) instead of one work-item
-      for (const bool wave : {false, true}) {
-        if (wave && phase.wave_loops.empty()) continue;
-        src << "extern \"C\" __global__ void __launch_bounds__(" << (wave ? GenericPhase::kWaveThreads : 64u) << ") " << phase.name
-            << (wave ? "_w" : "") << "(Args_" << info.name << " args) {\n";
-        src << "  const View* readonlys = args.readonlys;\n";
-        src << "  View writeables[" << nw << "];\n";
-        src << "  for (int b = 0; b < " << nw << "; ++b) writeables[b] = args.writeables[b];\n";
-        if (wave) {
-          src << "  const size_t lane = threadIdx.x % 64;\n";
-          src << "  const size_t wi_first = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;\n";
-          src << "  const size_t wi_stride = ((size_t)gridDim.x * blockDim.x) / 64;\n";
-        } else {
-          src << "  const size_t wi_first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;\n";
-          src << "  const size_t wi_stride = (size_t)gridDim.x * blockDim.x;\n";
-        }
-        emit_capacities("  ");
-        emit_privates(phase, "  ");
-        if (phase.parallel_loops.empty()) {
-          src << "  if (wi_first != 0) return;\n";
-          Printer pr;
-          pr.held = &held;
-          if (wave) pr.wave = &phase.wave_loops;
-          pr.block(stmts, 1);
-          src << pr.os.str();
-        } else {
-          emit_spread(phase, stmts, 1, wave);
-        }
-        src << "}\n\n";
-      }
-      info.phases.push_back(std::move(phase));
-    }
+    info.phases.push_back(std::move(phase));
+  }
+  if (any_grid) {
+    // the two helpers of the form with a loop in parts: the parts' copies start as the reduction's identity, and
+    // fold into the accumulated buffer in part order (op: 0 +, 1 *, 2 max, 3 min; keep: the buffer's own value
+    // takes part, i.e. the nest did not initialise it)
+    src << "struct Args_" << kFillKernel << " { float* data; size_t count; float value; };\n";
+    src << "extern \"C\" __global__ void __launch_bounds__(256) " << kFillKernel << "(Args_" << kFillKernel << " args) {\n";
+    src << "  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < args.count; e += (size_t)gridDim.x * blockDim.x)\n";
+    src << "    args.data[e] = args.value;\n}\n\n";
+    src << "struct Args_" << kCombineKernel << " { const float* partial; float* data; size_t parts; size_t count; int op; int keep; };\n";
+    src << "extern \"C\" __global__ void __launch_bounds__(256) " << kCombineKernel << "(Args_" << kCombineKernel << " args) {\n";
+    src << "  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < args.count; e += (size_t)gridDim.x * blockDim.x) {\n";
+    src << "    float acc = args.partial[e];\n";
+    src << "    #pragma unroll 8\n";
+    src << "    for (size_t p = 1; p < args.parts; ++p) {\n";
+    src << "      const float v = args.partial[p * args.count + e];\n";
+    src << "      acc = args.op == 0 ? acc + v : args.op == 1 ? acc * v : args.op == 2 ? fmaxf(acc, v) : fminf(acc, v);\n";
+    src << "    }\n";
+    src << "    if (args.keep) {\n";
+    src << "      const float v = args.data[e];\n";
+    src << "      acc = args.op == 0 ? v + acc : args.op == 1 ? v * acc : args.op == 2 ? fmaxf(v, acc) : fminf(v, acc);\n";
+    src << "    }\n";
+    src << "    args.data[e] = acc;\n";
+    src << "  }\n}\n\n";
+    // the same for a few elements and many parts: a wavefront per element, its lanes over the parts
+    src << "extern \"C\" __global__ void __launch_bounds__(256) " << kCombineWaveKernel << "(Args_" << kCombineKernel << " args) {\n";
+    src << "  const size_t lane = threadIdx.x % 64;\n";
+    src << "  for (size_t e = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / 64; e < args.count; e += ((size_t)gridDim.x * blockDim.x) / 64) {\n";
+    src << "    float acc = args.op == 0 ? 0.0f : args.op == 1 ? 1.0f : args.op == 2 ? (-INFINITY) : INFINITY;\n";
+    src << "    #pragma unroll 8\n";
+    src << "    for (size_t p = lane; p < args.parts; p += 64) {\n";
+    src << "      const float v = args.partial[p * args.count + e];\n";
+    src << "      acc = args.op == 0 ? acc + v : args.op == 1 ? acc * v : args.op == 2 ? fmaxf(acc, v) : fminf(acc, v);\n";
+    src << "    }\n";
+    src << "    for (int lane_xor = 32; lane_xor > 0; lane_xor >>= 1) {\n";
+    src << "      const float v = __shfl_xor(acc, lane_xor);\n";
+    src << "      acc = args.op == 0 ? acc + v : args.op == 1 ? acc * v : args.op == 2 ? fmaxf(acc, v) : fminf(acc, v);\n";
+    src << "    }\n";
+    src << "    if (args.keep) {\n";
+    src << "      const float v = args.data[e];\n";
+    src << "      acc = args.op == 0 ? v + acc : args.op == 1 ? v * acc : args.op == 2 ? fmaxf(v, acc) : fminf(v, acc);\n";
+    src << "    }\n";
+    src << "    ILANG_WAVE_SYNC();\n";
+    src << "    if (lane == 0) args.data[e] = acc;\n";
+    src << "  }\n}\n\n";
   }
   if (any) out.source = src.str();
   return out;

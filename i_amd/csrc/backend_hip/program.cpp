@@ -1,6 +1,7 @@
 #include "program.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -39,9 +40,9 @@ std::string ref_name(BufferRef r) {
 // release cost the host 20 to 45 us a call here, several times the rest of the executor).  A call carves its
 // temporaries off the block; what does not fit is allocated as before, and at its end the call replaces the block
 // by one large enough for all it needed, up to ILANG_HIP_ARENA_MB (default 256; 0: no such block) per stream,
-// held until the process ends, for the first 16 streams that run programs.  A stream under capture, a second
-// call in flight on the same stream from another thread, and the emulated runtime (whose allocations are guarded
-// one by one) take the allocating path.
+// held until the process ends, for the first 16 streams that run programs.  A stream under capture and a second
+// call in flight on the same stream from another thread take the allocating path (and so does every call under
+// ILANG_HIP_ARENA_MB=0, which tools that guard allocations one by one use).
 struct Arena {
   void* base = nullptr;
   size_t capacity = 0;
@@ -609,20 +610,40 @@ ihip::Err generic_function(Program& p, const std::string& name, hipFunction_t* f
   return ihip::module_function(it->second, name.c_str(), fn);
 }
 
+// Into how many parts to deal out the outermost sequential loop of a generated nest (1: the nest as it is).
+// `total` counts the iterations of its parallel loops, `reduced` those of the loop in question, `wave` says which of
+// the two forms (a work-item or a wavefront per iteration) would run.  Parts pay when the parallel loops alone leave
+// most of the chip idle: enough of them for 16 wavefronts per compute unit, each part with at least 16 iterations of
+// a loop that a work-item runs by itself, 4 rounds of the 64 lanes when the loop in parts is the one over the lanes,
+// one iteration when the lanes run over a loop inside it; at most 4096, from 16 on a multiple of 8 and from 256 on
+// of 32 (the copies of buffers of 64 elements and more are then folded in two passes).
+size_t generated_parts(const ihip::KernelOptions& knobs, const GridForm& grid, bool wave, size_t total, size_t reduced) {
+  if (!grid.available || (wave && !grid.wave) || knobs.generated_parts == 1 || total == 0) return 1;
+  const size_t least = !wave ? 16 : grid.loop_is_spread ? 256 : 1;
+  size_t parts;
+  if (knobs.generated_parts > 1) {
+    parts = (size_t)knobs.generated_parts;
+  } else {
+    const size_t target = wave ? 4096 : 262144;  // wavefronts / work-items that fill the chip
+    if (total * 2 > target) return 1;
+    parts = std::min<size_t>(target / total, reduced / least);
+  }
+  parts = std::min<size_t>(std::min<size_t>(parts, 4096), std::max<size_t>(reduced, 1));
+  if (parts >= 256) parts = parts / 32 * 32;
+  else if (parts >= 16) parts = parts / 8 * 8;
+  return parts < 2 ? 1 : parts;
+}
+
 ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
   Program& p = run.p;
   const GenericKernel& gk = p.generic.kernels[k];
-  if (gk.name.empty()) return "kernel " + std::to_string(k) + " has no generated form";
-  // One launch per top-level loop nest (ILANG_HIP_PHASES=1 at compile time) is confined to the emulated runtime:
-  // its one run on a GPU ended in a memory fault whose cause has not been shown, so it must not reach a device.
-  if (gk.phases.size() > 1 && !gk.cooperative && !ihip::runtime_is_emulated())
-    return "kernel " + std::to_string(k) + " was compiled with ILANG_HIP_PHASES=1 (one launch per loop nest), which is "
-           "restricted to the CPU emulation of the runtime; unset it and compile again";
+  if (gk.name.empty() || gk.phases.size() != 1) return "kernel " + std::to_string(k) + " has no generated form";
+  const GenericPhase& ph = gk.phases[0];
   const size_t R = p.generic.rank;
   const size_t view_bytes = 8 + 16 * R;
   const size_t nr = std::max<size_t>(gk.n_reads, 1), nw = std::max<size_t>(gk.n_writes, 1);
   std::vector<unsigned char> args((nr + nw) * view_bytes, 0);
-  if (args.size() > 4000) return "kernel " + std::to_string(k) + " takes too many buffers for one launch";
+  if (args.size() + 8 * nw + 8 > 4000) return "kernel " + std::to_string(k) + " takes too many buffers for one launch";
 
   auto fill = [&](size_t slot, void* data, BufferRef r) {
     unsigned char* v = args.data() + slot * view_bytes;
@@ -636,88 +657,139 @@ ihip::Err launch_generic(Run& run, size_t k, const Step& dispatch) {
     if (ihip::Err e = run.read_f32(dispatch.reads[i], &ptr); !e.empty()) return e;
     fill(i, ptr, dispatch.reads[i]);
   }
-  // buffers that live in memory are the same for every phase
+  std::vector<void*> write_ptrs(dispatch.writes.size(), nullptr);
   for (size_t i = 0; i < dispatch.writes.size(); ++i) {
-    void* ptr = nullptr;
     if (!gk.is_private(i))
-      if (ihip::Err e = run.write_f32(dispatch.writes[i], &ptr); !e.empty()) return e;
-    fill(nr + i, ptr, dispatch.writes[i]);
+      if (ihip::Err e = run.write_f32(dispatch.writes[i], &write_ptrs[i]); !e.empty()) return e;
+    fill(nr + i, write_ptrs[i], dispatch.writes[i]);
   }
-
-  if (gk.cooperative) {
-    // one launch of one workgroup; every nest's work-item-private device buffers get one slice per work-item
-    run.notes.push_back("generated kernel " + gk.name + ": one workgroup of " + std::to_string(GenericKernel::kCooperativeThreads) +
-                        " work-items, " + std::to_string(gk.phases.size()) + " loop nests separated by barriers");
-    const size_t slots = GenericKernel::kCooperativeThreads;
-    for (const GenericPhase& ph : gk.phases)
-      for (const PrivateBuffer& pb : ph.privates) {
-        void* ptr = nullptr;
-        if (!pb.is_static) {
-          const size_t n = std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
-          if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
+  auto extent_of = [&](const Extent<Param>& e) {
+    const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
+    return run.extent(Extent<size_t>{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind});
+  };
+  run.notes.push_back("generated kernel " + gk.name);
+  size_t total = 1;
+  for (const auto& e : ph.parallel_extents) total *= extent_of(e);
+  if (total == 0) return {};
+  // The wavefront-per-iteration form (reduction loops spread over 64 lanes), when the nest has one: taken when
+  // the reduction is long enough to occupy the lanes and either consecutive lanes read consecutive elements
+  // or there are too few iterations to fill the chip with one work-item each.  Option generated.wave = 0 | 1 overrides.
+  bool wave = false;
+  if (!ph.wave_loops.empty()) {
+    const size_t reduced = extent_of(ph.wave_extent);
+    // (a nest with a form in parts fills the chip with work-items, whose lanes read along the parallel index)
+    wave = reduced >= 128 && (ph.wave_contiguous || (total < 65536 && !ph.grid.available));
+    if (run.knobs.generated_wave >= 0) wave = run.knobs.generated_wave == 1;
+  }
+  bool dynamic_private = false;  // (per-work-item slices of a device buffer are sized for the plain form's grid)
+  for (const PrivateBuffer& pb : ph.privates) dynamic_private = dynamic_private || !pb.is_static;
+  const size_t parts = dynamic_private ? 1 : generated_parts(run.knobs, ph.grid, wave, total, ph.grid.available ? extent_of(ph.grid.extent) : 0);
+  hipFunction_t fn;
+  if (parts > 1) {
+    // every part accumulates into a copy of its own of each accumulated buffer (filled with the reduction's
+    // identity first); ilang_combine folds the copies into the buffer afterwards
+    std::vector<size_t> counts;
+    size_t floats = 0;
+    for (const GridAccumulator& acc : ph.grid.accumulators) {
+      counts.push_back(std::max<size_t>(1, product(run.layout_of(dispatch.writes.at(acc.writeable)))));
+      floats += counts.back() * parts;
+    }
+    // How the copies fold.  A buffer of fewer than 64 elements: one pass, a wavefront per element with its lanes
+    // over the parts.  Larger ones: a work-item per element, and from 16 parts on in two passes (the copies, read as
+    // [parts / w][w * count], fold into w = 8 or 32 copies first), which puts w times as many work-items on the
+    // first pass.
+    const size_t width = parts >= 256 && parts % 32 == 0 ? 32 : parts >= 16 && parts % 8 == 0 ? 8 : 0;
+    size_t most = 0;
+    for (size_t c : counts)
+      if (c >= 64) most = std::max(most, c);
+    const bool two_passes = width != 0 && most != 0;
+    if (two_passes) floats += width * most;
+    void* partial = nullptr;
+    if (run.alloc_optional(&partial, floats * 4)) {
+      std::vector<unsigned char> gargs(args);
+      gargs.resize(args.size() + 8 * nw + 8, 0);
+      float* at = static_cast<float*>(partial);
+      struct FillArgs { float* data; size_t count; float value; };
+      struct CombineArgs { const float* partial; float* data; size_t parts; size_t count; int op; int keep; };
+      hipFunction_t fill_fn, combine_fn, combine_wave_fn;
+      if (ihip::Err e = generic_function(p, kFillKernel, &fill_fn); !e.empty()) return e;
+      if (ihip::Err e = generic_function(p, kCombineKernel, &combine_fn); !e.empty()) return e;
+      if (ihip::Err e = generic_function(p, kCombineWaveKernel, &combine_wave_fn); !e.empty()) return e;
+      std::vector<std::pair<CombineArgs, bool>> combines;  // (arguments, a wavefront per element)
+      float* const folded = static_cast<float*>(partial) + (floats - (two_passes ? width * most : 0));
+      for (size_t a = 0; a < ph.grid.accumulators.size(); ++a) {
+        const GridAccumulator& acc = ph.grid.accumulators[a];
+        std::memcpy(gargs.data() + args.size() + 8 * acc.writeable, &at, 8);
+        const float identity = acc.op == Op::Mul ? 1.0f : acc.op == Op::Max ? -INFINITY : acc.op == Op::Min ? INFINITY : 0.0f;
+        // (the parts store every element of their copies themselves when the accumulators live in registers and the
+        // buffer has no padding that no work-item owns)
+        const bool dense = product(run.shape_of(dispatch.writes.at(acc.writeable))) == counts[a];
+        if (!(ph.grid.held_accumulators && dense)) {
+          FillArgs fa{at, counts[a] * parts, identity};
+          const size_t fgrid = std::min<size_t>((fa.count + 255) / 256, 4096);
+          if (ihip::Err e = ihip::launch(fill_fn, (unsigned)fgrid, 1, 1, 256, &fa, sizeof(fa), run.stream); !e.empty()) return e;
         }
-        fill(nr + pb.writeable, ptr, dispatch.writes[pb.writeable]);
+        const int op = acc.op == Op::Add ? 0 : acc.op == Op::Mul ? 1 : acc.op == Op::Max ? 2 : 3;
+        float* const dst = static_cast<float*>(write_ptrs.at(acc.writeable));
+        if (counts[a] < 64) {
+          combines.push_back({{at, dst, parts, counts[a], op, acc.init_here ? 0 : 1}, true});
+        } else if (two_passes) {
+          combines.push_back({{at, folded, parts / width, width * counts[a], op, 0}, false});
+          combines.push_back({{folded, dst, width, counts[a], op, acc.init_here ? 0 : 1}, false});
+        } else {
+          combines.push_back({{at, dst, parts, counts[a], op, acc.init_here ? 0 : 1}, false});
+        }
+        at += counts[a] * parts;
       }
-    hipFunction_t fn;
-    if (ihip::Err e = generic_function(p, gk.name, &fn); !e.empty()) return e;
-    return ihip::launch(fn, 1, 1, 1, GenericKernel::kCooperativeThreads, args.data(), args.size(), run.stream);
+      std::memcpy(gargs.data() + args.size() + 8 * nw, &parts, 8);
+      const std::string name = ph.name + (wave ? "_gw" : "_g");
+      if (ihip::Err e = generic_function(p, name, &fn); !e.empty()) return e;
+      run.notes.back() += ", as " + name + ": the outermost sequential loop in " + std::to_string(parts) + " parts over " +
+                          (wave ? "wavefronts" : "work-items") + ", combined by " + kCombineKernel;
+      const size_t units = total * parts;
+      const unsigned per_group = wave ? GenericPhase::kWaveThreads / 64 : 64;
+      const size_t groups = std::min<size_t>((units + per_group - 1) / per_group, size_t(1) << 20);
+      if (ihip::Err e = ihip::launch(fn, (unsigned)groups, 1, 1, wave ? GenericPhase::kWaveThreads : 64, gargs.data(), gargs.size(), run.stream);
+          !e.empty())
+        return e;
+      for (const auto& [ca, by_wave] : combines) {
+        const size_t cgrid = std::min<size_t>(by_wave ? (ca.count + 3) / 4 : (ca.count + 255) / 256, 4096);
+        if (ihip::Err e = ihip::launch(by_wave ? combine_wave_fn : combine_fn, (unsigned)cgrid, 1, 1, 256, &ca, sizeof(ca), run.stream);
+            !e.empty())
+          return e;
+      }
+      return {};
+    }
   }
-  run.notes.push_back("generated kernel " + gk.name + (gk.phases.size() > 1 ? " in " + std::to_string(gk.phases.size()) + " launches" : ""));
-  // one launch per phase, in order on the stream
-  for (const GenericPhase& ph : gk.phases) {
-    size_t total = 1;
-    for (const auto& e : ph.parallel_extents) {
-      const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
-      Extent<size_t> resolved{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind};
-      total *= run.extent(resolved);
-    }
-    if (total == 0) continue;
-    // The wavefront-per-iteration form (reduction loops spread over 64 lanes), when the nest has one: taken when
-    // the reduction is long enough to occupy the lanes and either consecutive lanes read consecutive elements
-    // or there are too few iterations to fill the chip with one work-item each.  Option generated.wave = 0 | 1 overrides.
-    if (!ph.wave_loops.empty()) {
-      const auto& e = ph.wave_extent;
-      const BufferRef src = e.source.buffer.writeable ? dispatch.writes.at(e.source.buffer.ind) : dispatch.reads.at(e.source.buffer.ind);
-      const size_t reduced = run.extent(Extent<size_t>{plan_buffer(run.plan, src).shape.at(e.source.dim), e.kind});
-      bool wave = reduced >= 128 && (ph.wave_contiguous || total < 65536);
-      if (run.knobs.generated_wave >= 0) wave = run.knobs.generated_wave == 1;
-      if (wave) {
-        const size_t waves = std::min<size_t>(total, size_t(1) << 16);
-        const unsigned per_group = GenericPhase::kWaveThreads / 64;
-        for (const PrivateBuffer& pb : ph.privates) fill(nr + pb.writeable, nullptr, dispatch.writes[pb.writeable]);
-        hipFunction_t fn;
-        if (ihip::Err err = generic_function(p, ph.name + "_w", &fn); !err.empty()) return err;
-        run.notes.back() += ", as " + ph.name + "_w: one wavefront per iteration of the parallel loops";
-        if (ihip::Err err = ihip::launch(fn, (unsigned)((waves + per_group - 1) / per_group), 1, 1, GenericPhase::kWaveThreads,
-                                         args.data(), args.size(), run.stream);
-            !err.empty())
-          return err;
-        continue;
-      }
-    }
-    size_t threads = ph.parallel_loops.empty() ? 1 : total;
-    // dynamic private buffers cost memory per work-item slot: cap the slots
-    size_t slot_elems = 0;
-    for (const PrivateBuffer& pb : ph.privates)
-      if (!pb.is_static) slot_elems += std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
-    size_t max_threads = size_t(1) << 20;
-    if (slot_elems) max_threads = std::max<size_t>(64, std::min(max_threads, (size_t(1) << 28) / (slot_elems * 4)));
-    threads = std::min(threads, max_threads);
-    const unsigned grid = (unsigned)((threads + 63) / 64);
-    const size_t slots = (size_t)grid * 64;
-    for (const PrivateBuffer& pb : ph.privates) {
-      void* ptr = nullptr;
-      if (!pb.is_static) {
-        const size_t n = std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
-        if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
-      }
-      fill(nr + pb.writeable, ptr, dispatch.writes[pb.writeable]);
-    }
-    hipFunction_t fn;
-    if (ihip::Err e = generic_function(p, ph.name, &fn); !e.empty()) return e;
-    if (ihip::Err e = ihip::launch(fn, grid, 1, 1, 64, args.data(), args.size(), run.stream); !e.empty()) return e;
+  if (wave) {
+    const size_t waves = std::min<size_t>(total, size_t(1) << 16);
+    const unsigned per_group = GenericPhase::kWaveThreads / 64;
+    for (const PrivateBuffer& pb : ph.privates) fill(nr + pb.writeable, nullptr, dispatch.writes[pb.writeable]);
+    if (ihip::Err err = generic_function(p, ph.name + "_w", &fn); !err.empty()) return err;
+    run.notes.back() += ", as " + ph.name + "_w: one wavefront per iteration of the parallel loops";
+    return ihip::launch(fn, (unsigned)((waves + per_group - 1) / per_group), 1, 1, GenericPhase::kWaveThreads, args.data(), args.size(),
+                        run.stream);
   }
-  return {};
+  size_t threads = ph.parallel_loops.empty() ? 1 : total;
+  // dynamic private buffers cost memory per work-item slot: cap the slots
+  size_t slot_elems = 0;
+  for (const PrivateBuffer& pb : ph.privates)
+    if (!pb.is_static) slot_elems += std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+  size_t max_threads = size_t(1) << 20;
+  if (slot_elems) max_threads = std::max<size_t>(64, std::min(max_threads, (size_t(1) << 28) / (slot_elems * 4)));
+  threads = std::min(threads, max_threads);
+  const unsigned grid = (unsigned)((threads + 63) / 64);
+  const size_t slots = (size_t)grid * 64;
+  for (const PrivateBuffer& pb : ph.privates) {
+    void* ptr = nullptr;
+    if (!pb.is_static) {
+      const size_t n = std::max<size_t>(1, product(run.layout_of(dispatch.writes[pb.writeable])));
+      if (ihip::Err e = run.alloc(&ptr, n * slots * 4); !e.empty()) return e;
+    }
+    fill(nr + pb.writeable, ptr, dispatch.writes[pb.writeable]);
+  }
+  if (ihip::Err e = generic_function(p, ph.name, &fn); !e.empty()) return e;
+  return ihip::launch(fn, grid, 1, 1, 64, args.data(), args.size(), run.stream);
 }
 
 const Step* find_dispatch(const ExecPlan& plan, size_t k) {
@@ -773,8 +845,12 @@ std::string compile_program(const Component& component, Program** out) {
   p->recognized = recognize_kernels(p->low);
   p->same_extent = tied_extents(p->low.graph);
   if (p->recognized.size() != p->low.plan.kernels.size()) lower_error("kernel recognition lost track of the kernel list");
-  std::vector<bool> emit(p->low.plan.kernels.size(), true);
-  p->generic = emit_generic_hip(p->low.plan, p->module, emit);
+  // the generated form: one kernel per loop nest
+  std::vector<size_t> origin;
+  p->nest_plan = split_nests(p->low.plan, &origin);
+  p->nests_of.assign(p->low.plan.kernels.size(), {});
+  for (size_t n = 0; n < origin.size(); ++n) p->nests_of.at(origin[n]).push_back(n);
+  p->generic = emit_generic_hip(p->nest_plan, lower_exec_plan_to_module(p->nest_plan), std::vector<bool>(p->nest_plan.kernels.size(), true));
   bool needs_generated = false;
   for (const Recognized& r : p->recognized) needs_generated |= r.kind == Recognized::None;
   if (needs_generated)
@@ -787,7 +863,10 @@ std::string program_code(const Component& component) {
   const Lowered low = lower_component(component);
   const Module module = lower_exec_plan_to_module(low.plan);
   const auto rec = recognize_kernels(low);
-  const GenericModule gen = emit_generic_hip(low.plan, module, std::vector<bool>(low.plan.kernels.size(), true));
+  std::vector<size_t> origin;
+  const ExecPlan nest_plan = split_nests(low.plan, &origin);
+  const GenericModule gen = emit_generic_hip(nest_plan, lower_exec_plan_to_module(nest_plan), std::vector<bool>(nest_plan.kernels.size(), true));
+  (void)module;
   std::ostringstream os;
   os << "// 𝚒 gfx950 backend plan: " << low.plan.inputs.size() << " input(s), " << low.plan.intermediates.size()
      << " intermediate(s), " << low.plan.outputs.size() << " output(s), " << low.plan.kernels.size() << " kernel(s)\n";
@@ -820,26 +899,32 @@ std::string program_code(const Component& component) {
     for (BufferRef r : d->reads) os << " " << ref_name(r);
     os << "; writes";
     for (BufferRef r : d->writes) os << " " << ref_name(r);
-    if (gen.kernels[k].cooperative)
-      os << "\n//     one workgroup of " << GenericKernel::kCooperativeThreads << " work-items runs the " << gen.kernels[k].phases.size()
-         << " loop nests one after the other, a barrier between them";
-    for (size_t n = 0; n < gen.kernels[k].phases.size(); ++n) {
-      const GenericPhase& ph = gen.kernels[k].phases[n];
+    // the generated form: one kernel per loop nest of the kernel (their names are those of the source below)
+    size_t nests = 0;
+    for (size_t n = 0; n < origin.size(); ++n) nests += origin[n] == k;
+    for (size_t n = 0; n < origin.size(); ++n) {
+      if (origin[n] != k || gen.kernels[n].phases.empty()) continue;
+      const GenericPhase& ph = gen.kernels[n].phases[0];
+      const Step* nd = find_dispatch(nest_plan, n);
       os << "\n//     ";
-      if (gen.kernels[k].cooperative) os << "nest " << n << ", ";
-      else if (gen.kernels[k].phases.size() > 1) os << "launch " << ph.name << ", ";
+      if (nests > 1) os << "loop nest as kernel " << ph.name << ", ";
+      else os << "generated as " << ph.name << ", ";
       os << "work-items:";
       if (ph.parallel_loops.empty()) os << " 1 (no independent outer loop)";
       for (size_t id : ph.parallel_loops) os << " i" << id;
       if (!ph.privates.empty()) {
         os << "; work-item-private:";
         for (const auto& pb : ph.privates)
-          os << " " << ref_name(d->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
+          os << " " << ref_name(nd->writes[pb.writeable]) << (pb.is_static ? "[" + std::to_string(pb.static_size) + "]" : "[dynamic]");
       }
       if (!ph.wave_loops.empty()) {
         os << "\n//     " << ph.name << "_w, one wavefront per work-item of the above (long reductions): over its lanes";
         for (const WaveLoop& wl : ph.wave_loops) os << " i" << wl.loop;
       }
+      if (ph.grid.available)
+        os << "\n//     " << ph.name << "_g" << (ph.grid.wave ? " / " + ph.name + "_gw" : "") << ", loop i" << ph.grid.loop
+           << " in parts over groups of work-items (grids that the parallel loops alone leave mostly idle), the parts combined by "
+           << kCombineKernel;
     }
     os << "\n";
   }
@@ -913,15 +998,19 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
     if (hand[k]) {
       for (size_t id : hand_intermediates(p.recognized[k])) needed.insert(id);
     } else {
-      for (BufferRef r : d->reads)
-        if (r.kind == BufferRef::Intermediate) needed.insert(r.id);
-      for (size_t i = 0; i < d->writes.size(); ++i)
-        if (d->writes[i].kind == BufferRef::Intermediate && !p.generic.kernels[k].is_private(i)) needed.insert(d->writes[i].id);
+      for (size_t nest : p.nests_of[k]) {
+        const Step* nd = find_dispatch(p.nest_plan, nest);
+        if (!nd) return "kernel " + std::to_string(k) + ": a loop nest of it is never dispatched";
+        for (BufferRef r : nd->reads)
+          if (r.kind == BufferRef::Intermediate) needed.insert(r.id);
+        for (size_t i = 0; i < nd->writes.size(); ++i)
+          if (nd->writes[i].kind == BufferRef::Intermediate && !p.generic.kernels[nest].is_private(i)) needed.insert(nd->writes[i].id);
+      }
     }
   }
 
   std::unique_lock<std::mutex> arena_lock;
-  if (!workspace && !ihip::runtime_is_emulated()) {
+  if (!workspace) {
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
       (void)hipGetLastError();
@@ -954,7 +1043,19 @@ std::string execute(Program& p, const std::vector<DeviceTensor>& inputs, const s
       const size_t n = product(run.layout_of({BufferRef::Intermediate, step.id}));
       if (ihip::Err e = run.alloc(&run.intermediates[step.id], n * 4); !e.empty()) return finish(e);
     } else if (step.kind == Step::Dispatch) {
-      ihip::Err e = hand[step.id] ? launch_hand(run, p.recognized[step.id]) : launch_generic(run, step.id, step);
+      ihip::Err e;
+      if (hand[step.id]) {
+        e = launch_hand(run, p.recognized[step.id]);
+      } else {
+        // the generated form: the kernel's loop nests one after the other, each a kernel of its own (one line of the report)
+        std::string lines;
+        for (size_t nest : p.nests_of[step.id]) {
+          if (e = launch_generic(run, nest, *find_dispatch(p.nest_plan, nest)); !e.empty()) break;
+          lines += (lines.empty() ? "" : "; ") + run.notes.back();
+          run.notes.pop_back();
+        }
+        if (e.empty()) run.notes.push_back(p.nests_of[step.id].size() > 1 ? std::to_string(p.nests_of[step.id].size()) + " loop nests, a kernel each: " + lines : lines);
+      }
       if (!e.empty()) return finish("kernel f" + std::to_string(step.id) + ": " + e);
     }
   }

@@ -35,7 +35,11 @@ struct Program {
   // Groups of (input, dimension) pairs that one index symbol ties together, directly or through intermediate
   // results: their extents must agree, or some kernel would index an operand out of bounds.
   std::vector<std::vector<std::pair<size_t, size_t>>> same_extent;
-  GenericModule generic;               // source for every kernel (hand-written ones keep a generated twin)
+  // The generated form of the plan: every kernel cut into one kernel per loop nest (split_nests), the statement IR
+  // of those, and for each kernel of low.plan the kernels of nest_plan that stand for it, in order.
+  ic::ExecPlan nest_plan;
+  std::vector<std::vector<size_t>> nests_of;
+  GenericModule generic;               // source for every kernel of nest_plan (hand-written ones keep a generated twin)
   std::vector<char> image;             // built lazily unless some kernel can only run generated
   bool image_built = false;
   std::mutex mu;

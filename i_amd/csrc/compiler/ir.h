@@ -228,6 +228,10 @@ template <class B>
 struct Kernel {
   std::vector<B> reads, writes;
   Block<B> body;
+  // Buffers whose Computes accumulate (`dst = op(dst, reads...)`) although this body holds no Init of them: a
+  // backend that cuts a kernel's body into several kernels keeps the form of each Compute this way.  Empty in
+  // every plan the lowering passes produce.
+  std::vector<B> accumulates;
 };
 enum class BufferKind { Input, Intermediate, Output };
 struct Buffer {

@@ -325,6 +325,7 @@ Module lower_exec_plan_to_module(const ExecPlan& plan) {
       for (size_t d = 0; d < shape.size(); ++d) kl.semantic_dims.push_back({{Param{true, i}, d}, shape[d]});
     }
     collect_initialized(plan.kernels[k].body, kl.initialized);
+    kl.initialized.insert(plan.kernels[k].accumulates.begin(), plan.kernels[k].accumulates.end());
     m.kernels.push_back({"f" + std::to_string(k), MSignature::Kernel, kl.lower_block(plan.kernels[k].body)});
   }
   return m;

@@ -129,7 +129,7 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
   std::unique_lock<std::mutex> staging_lock;
   char* carve = nullptr;
   char *mirror = nullptr, *block_base = nullptr;  // mirror != nullptr: host data passes through the page-locked mirror
-  if (wanted <= staging_limit() && !ihip::runtime_is_emulated()) {
+  if (wanted <= staging_limit()) {
     if (Staging* block = staging_of_current_device()) {
       staging_lock = std::unique_lock<std::mutex>(block->busy, std::try_to_lock);
       if (staging_lock.owns_lock()) {

@@ -101,24 +101,19 @@ Err launch(hipFunction_t fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
   return check(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, 0, stream, nullptr, config), "hipModuleLaunchKernel");
 }
 
-bool runtime_is_emulated() {
-  static const bool emulated = dlsym(RTLD_DEFAULT, "ilang_hip_runtime_is_emulated") != nullptr;
-  return emulated;
-}
-
 DryRun::DryRun() { ++g_dry_run; }
 DryRun::~DryRun() { --g_dry_run; }
 
 // Stream-ordered temporaries come from a pool of the library's own, one per device, that keeps up to 1 GiB of
 // freed memory instead of handing it back to the system when the stream runs dry, which is what makes a
 // temporary cost tens of microseconds from the device's default pool.  The default pool and its settings, which
-// belong to the application, are left alone; without a pool of its own (the emulated runtime, a failed creation)
-// the library allocates from the default one.
+// belong to the application, are left alone; without a pool of its own (a runtime that has none to give: the
+// creation fails) the library allocates from the default one.
 Err temp_alloc(void** p, size_t bytes, hipStream_t stream) {
   *p = nullptr;
   if (bytes == 0) bytes = 4;
   hipMemPool_t pool = nullptr;
-  if (!runtime_is_emulated()) {
+  {
     std::lock_guard<std::mutex> lock(g_mu);
     int dev = 0;
     if (Err e = check(hipGetDevice(&dev), "hipGetDevice"); !e.empty()) return e;

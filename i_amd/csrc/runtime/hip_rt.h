@@ -28,10 +28,6 @@ void unload_module(hipModule_t mod);
 Err launch(hipFunction_t fn, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned block_x,
            const void* params, size_t params_size, hipStream_t stream);
 
-// True when the HIP entry points this library calls are the host emulation used by the CPU tests (which exports a
-// marker symbol), false with a real HIP runtime.
-bool runtime_is_emulated();
-
 // While one of these lives on a thread, launch() on that thread checks nothing in and enqueues nothing: the
 // executor walks a program once this way to add up the temporaries it would need.
 struct DryRun {

@@ -49,10 +49,13 @@ Err set_kernel_option(KernelOptions& o, const std::string& name, int value) {
   } else if (name == "generated.wave") {
     if (!one_of({-1, 0, 1})) return bad("-1 (the launcher decides), 0 or 1");
     o.generated_wave = value;
+  } else if (name == "generated.parts") {
+    if (value < 0 || value > 4096) return bad("0 (the launcher decides), 1 (never) or a number of parts up to 4096");
+    o.generated_parts = value;
   } else {
     return "unknown program option '" + name +
            "' (known: attention.f32_scale, attention.kv_parts, attention.waves, attention.direct, gemm.k_parts, gemm.waves, "
-           "gemm.tile, gemm.direct, generated.only, generated.wave)";
+           "gemm.tile, gemm.direct, generated.only, generated.wave, generated.parts)";
   }
   return {};
 }

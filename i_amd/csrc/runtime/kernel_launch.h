@@ -32,6 +32,7 @@ struct KernelOptions {
   int gemm_direct = 1;          // 0: the register-staged bf16 kernel instead of the direct-to-LDS ones
   int generated_only = 0;       // 1: every kernel of a program in its generated form
   int generated_wave = -1;      // wavefront-per-iteration form of generated reduction nests: -1 decides, 0 never, 1 wherever a nest has one
+  int generated_parts = 0;      // outermost sequential loop of a generated reduction nest in parts over workgroups: 0 decides, 1 never, n that many
   // two 64-bit counters in device memory to which the bf16 direct-to-LDS attention kernels add the time their
   // workgroups were resident, on the shader clock and on the constant 100 MHz clock (AttnParams::clock)
   unsigned long long* clock_ticks = nullptr;

@@ -131,6 +131,8 @@ int i_hip_attention_opt(const void* q, const void* k, const void* v, void* o,
  *   "gemm.direct"          1 (default) / 0: the register-staged bf16 product kernel
  *   "generated.only"       0 (default) / 1: every kernel in its generated form (no hand-written kernel)
  *   "generated.wave"       wavefront-per-iteration form of generated reduction nests: -1 (default) by extents, 0 never, 1 always
+ *   "generated.parts"      outermost sequential loop of a generated reduction nest in parts over workgroups (a sum to one
+ *                          element, a column sum of few columns): 0 (default) by extents, 1 never, n that many (at most 4096)
  * Returns 0, or -1 with the text in i_error() for an unknown name or a value the option does not take.  Takes
  * effect from the next i_exec*.
  */

@@ -2,7 +2,8 @@
 emulation of the HIP runtime (shim.cpp), and compares with the C the oracle backend emits for the same
 component.  Started as a subprocess by tests/test_generated_kernels_cpu.py with
 ILANG_CORE_LIB, ILANG_HIPCC, ILANG_NO_TORCH and ILANG_NO_DISK_CACHE set; ILANG_SHIM_WAVE=1 asks for the
-wavefront-per-iteration form of reduction nests (the program option generated.wave).
+wavefront-per-iteration form of reduction nests (the program option generated.wave), ILANG_SHIM_PARTS=n for
+reduction nests with their outermost sequential loop in n parts (generated.parts).
 Prints the case name before running it, so a crash (a guard page hit = out-of-bounds access) names its case."""
 import sys
 from pathlib import Path
@@ -89,7 +90,7 @@ CASES = {
     "column min": (lambda: i("<ij~j"), [(9, 14)]),
     "product reduction": (lambda: i("*ij~i"), [(6, 5)]),
     "rank-3 output": (lambda: i("ik*jk~ijk | i:7 | jii'k"), [(20, 6), (9, 6)]),
-    "column normalize (two nests, one workgroup)": (lambda: (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij"), [(37, 70)]),
+    "column normalize (two nests)": (lambda: (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij"), [(37, 70)]),
     "column max shift, split": (lambda: (I & i(">ij~j|i:8,j:4|ijj'i'")) >> i("ij-j~ij|i:8,j:4|1ijj'i'"), [(21, 9)]),
     "column max shift, i outermost": (lambda: (I & i(">ij~j||ij")) >> i("ij-j~ij||1ij"), [(21, 9)]),
     "column sum normalize, split j": (lambda: (I & i("+ij~j|j:4|ijj'")) >> i("ij/j~ij|j:4|1ijj'"), [(9, 21)]),
@@ -112,11 +113,19 @@ WAVE_CASES = ["naive attention ragged", "batched naive attention", "mm_t", "mm_t
               "sum over the two last axes"]
 
 
+# a sample for the runs that repeat the suite under another option: every kind of reduction nest, kernels of several
+# nests, fused kernels with private tiles
+SAMPLE_CASES = ["flash 33x17", "naive attention ragged", "softmax naive 20x37", "mm_t", "mm_t empty", "matmul fused init site", "column max",
+                "total", "fanout two outputs", "two-level split mm_t", "product reduction", "column normalize (two nests)",
+                "column sum normalize, split j", "mlp with pair", "row sum 5x300", "row max 3x130, split j", "fused matrix-vector product",
+                "sum over the two last axes"]
+
+
 # Components with a reduced vector staged at the root of its consumer are checked against NumPy as well: the emitted
 # C comes out of the same lowering, and the reference's lowering mis-addresses that vector when producer and
 # consumer number the shared index differently (fixed here, see compiler/stage_to_kernels.cpp lower_read).
 CLOSED_FORMS = {
-    "column normalize (two nests, one workgroup)": lambda x: x / x.sum(axis=0),
+    "column normalize (two nests)": lambda x: x / x.sum(axis=0),
     "column max shift, split": lambda x: x - x.max(axis=0),
     "column max shift, i outermost": lambda x: x - x.max(axis=0),
     "column sum normalize, split j": lambda x: x / x.sum(axis=0),
@@ -143,7 +152,8 @@ def main():
     import os
 
     noalloc = os.environ.get("ILANG_SHIM_NOALLOC") == "1"
-    names = sys.argv[1:] or (WAVE_CASES if os.environ.get("ILANG_SHIM_CASES") == "wave" else list(CASES))
+    which = os.environ.get("ILANG_SHIM_CASES")
+    names = sys.argv[1:] or (WAVE_CASES if which == "wave" else SAMPLE_CASES if which == "sample" else list(CASES))
     tolerance = float(os.environ.get("ILANG_SHIM_TOLERANCE", "1e-5"))
     failed = []
     for name in names:
@@ -153,6 +163,8 @@ def main():
         comp.option("generated.only", 1)
         if os.environ.get("ILANG_SHIM_WAVE") is not None:
             comp.option("generated.wave", int(os.environ["ILANG_SHIM_WAVE"]))
+        if os.environ.get("ILANG_SHIM_PARTS") is not None:
+            comp.option("generated.parts", int(os.environ["ILANG_SHIM_PARTS"]))
         inputs = [rnd(s, k + 1) for k, s in enumerate(shapes)]
         got = run_without_allocating(comp, inputs) if noalloc else comp.exec_numpy(*inputs)
         ref = oracle.compile_component(comp.handle).run(*inputs)

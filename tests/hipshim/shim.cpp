@@ -85,8 +85,6 @@ Err static_scratch(void** ptr) {
 }  // namespace ihip
 
 extern "C" {
-// what ihip::runtime_is_emulated() looks for
-__attribute__((visibility("default"))) int ilang_hip_runtime_is_emulated = 1;
 hipError_t hipGetDevice(int* dev) {
   *dev = 0;
   return hipSuccess;
@@ -96,7 +94,7 @@ hipError_t hipMalloc(void** p, size_t bytes) { return guarded_alloc(p, bytes); }
 hipError_t hipFree(void* p) { return guarded_free(p); }
 hipError_t hipMallocAsync(void** p, size_t bytes, hipStream_t) { return guarded_alloc(p, bytes); }
 hipError_t hipFreeAsync(void* p, hipStream_t) { return guarded_free(p); }
-// (the library asks ilang_hip_runtime_is_emulated first and creates no pool here; these only satisfy the linker)
+// (no pool of its own here: the creation fails and the library allocates without one)
 hipError_t hipGetLastError() { return hipSuccess; }
 hipError_t hipHostMalloc(void**, size_t, unsigned int) { return hipErrorNotSupported; }
 hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* status) {

@@ -14,6 +14,9 @@ import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
 SHIM = ROOT / "tests" / "hipshim"
+# the library's kept blocks (temporaries per stream, device copies of host operands) switched off: every buffer is
+# then an allocation of its own, with the emulation's guard pages around it
+ONE_ALLOCATION_EACH = {"ILANG_HIP_ARENA_MB": "0", "ILANG_HIP_STAGING_MB": "0"}
 
 
 @pytest.fixture(scope="module")
@@ -26,11 +29,10 @@ def shim_lib():
 
 def run_cases(shim_lib, extra_env, names=()):
     env = dict(os.environ)
-    env.pop("ILANG_HIP_PHASES", None)
     # ILANG_HIP_UNCHECKED: plain accesses instead of the bounds-checked ones the product emits, so that an access
     # outside a buffer still hits a guard page here and names a lowering that is not sound
     env.update({"ILANG_CORE_LIB": str(shim_lib), "ILANG_HIPCC": str(SHIM / "hostcc.py"),
-                "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1", "ILANG_HIP_UNCHECKED": "1"})
+                "ILANG_NO_TORCH": "1", "ILANG_NO_DISK_CACHE": "1", "ILANG_HIP_UNCHECKED": "1", **ONE_ALLOCATION_EACH})
     env.update(extra_env)
     r = subprocess.run([sys.executable, str(SHIM / "run_cases.py"), *names], env=env, capture_output=True, text=True, timeout=900)
     last = [l for l in r.stdout.splitlines() if l.startswith("CASE")][-1:] or ["(none started)"]
@@ -42,15 +44,23 @@ def test_generated_kernels_match_the_emitted_c_on_the_cpu(shim_lib):
     run_cases(shim_lib, {})
 
 
-def test_generated_kernels_split_into_phases_match_too(shim_lib):
-    """ILANG_HIP_PHASES=1: a kernel whose body is a sequence of loop nests becomes one launch per nest."""
-    run_cases(shim_lib, {"ILANG_HIP_PHASES": "1"})
+def test_reduction_nests_with_their_outer_loop_in_parts_match_too(shim_lib):
+    """The program option generated.parts (ILANG_SHIM_PARTS to the case runner) deals the outermost sequential loop of
+    every nest that only accumulates out over that many groups of work-items, each with copies of its own of the
+    accumulated buffers, and a second kernel folds the copies: 3 parts (one pass of the fold, ragged shares), 256
+    parts (two passes; most parts get no iteration at these sizes), both forms of a nest (a work-item or a wavefront
+    per iteration), and work-items last to first.  (3 parts on every case; the other settings on a few.)"""
+    run_cases(shim_lib, {"ILANG_SHIM_PARTS": "3", "ILANG_SHIM_TOLERANCE": "1e-4"})
+    few = ["total", "column max", "row sum 5x300", "column normalize (two nests)", "fused matrix-vector product", "mm_t"]
+    run_cases(shim_lib, {"ILANG_SHIM_PARTS": "16", "ILANG_SHIM_TOLERANCE": "1e-4", "ILANG_HIP_UNCHECKED": "0"}, names=few)
+    run_cases(shim_lib, {"ILANG_SHIM_PARTS": "256", "ILANG_SHIM_TOLERANCE": "1e-4"}, names=few[:4])
+    run_cases(shim_lib, {"ILANG_SHIM_PARTS": "5", "ILANG_SHIM_WAVE": "1", "ILANG_SHIM_TOLERANCE": "1e-4"}, names=few[:3] + ["sum over the two last axes"])
+    run_cases(shim_lib, {"ILANG_SHIM_PARTS": "4", "ILANG_SHIM_ORDER": "reverse", "ILANG_SHIM_TOLERANCE": "1e-4"}, names=few)
 
 
 def test_generated_kernels_do_not_depend_on_work_item_order(shim_lib):
     """Work-items run last to first: a dependency between work-items would change the result."""
-    run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse"})
-    run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_HIP_PHASES": "1"})
+    run_cases(shim_lib, {"ILANG_SHIM_ORDER": "reverse", "ILANG_SHIM_CASES": "sample"})
 
 
 def test_wavefront_form_of_reduction_nests_matches_too(shim_lib):
@@ -64,7 +74,7 @@ def test_wavefront_form_of_reduction_nests_matches_too(shim_lib):
 
 def test_checked_accesses_give_the_same_results(shim_lib):
     """The form the product emits by default: every access checked against its buffer's element count."""
-    run_cases(shim_lib, {"ILANG_HIP_UNCHECKED": "0"})
+    run_cases(shim_lib, {"ILANG_HIP_UNCHECKED": "0", "ILANG_SHIM_CASES": "sample"})
 
 
 def test_schedules_with_unsound_lowerings_cannot_fault(shim_lib):
@@ -74,7 +84,7 @@ def test_schedules_with_unsound_lowerings_cannot_fault(shim_lib):
     check every access, so on a device this is a wrong result for a schedule that was wrong already, not a memory
     fault.  Unchecked, each of these hits a guard page."""
     env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"),
-               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
+               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1", **ONE_ALLOCATION_EACH)
     code = """
 import sys
 import numpy as np
@@ -99,16 +109,17 @@ print("ran", out.shape == shape)
 
 def test_fixed_workspace_entry_matches_on_the_cpu(shim_lib):
     """i_exec_into_device_noalloc: every temporary comes out of one fixed block (here a guarded host block of the
-    product's size), in both launch modes; results must equal the emitted C as through the allocating entry."""
+    product's size), also with reduction loops in parts (whose copies are temporaries too); results must equal the
+    emitted C as through the allocating entry."""
     run_cases(shim_lib, {"ILANG_SHIM_NOALLOC": "1"})
-    run_cases(shim_lib, {"ILANG_SHIM_NOALLOC": "1", "ILANG_HIP_PHASES": "1"})
+    run_cases(shim_lib, {"ILANG_SHIM_NOALLOC": "1", "ILANG_SHIM_PARTS": "3", "ILANG_SHIM_TOLERANCE": "1e-4", "ILANG_SHIM_CASES": "sample"})
 
 
 def test_operands_that_disagree_on_a_shared_index_are_refused_before_any_launch(shim_lib):
     """A kernel takes each loop bound from one operand; another operand with a smaller extent for the same index
     would be read out of bounds (a GPU memory fault on the device, a guard-page hit here)."""
     env = dict(os.environ, ILANG_CORE_LIB=str(shim_lib), ILANG_HIPCC=str(SHIM / "hostcc.py"),
-               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1")
+               ILANG_NO_TORCH="1", ILANG_NO_DISK_CACHE="1", **ONE_ALLOCATION_EACH)
     code = """
 import numpy as np
 from i_amd import Component as i
@@ -132,27 +143,46 @@ print(i('ij+ij~ij').exec_numpy(ones(3, 2), ones(3, 2)).sum())
     assert r.stdout.split() == ["ok"] * 4 + ["12.0"], r.stdout
 
 
-def test_multi_nest_kernels_run_as_one_workgroup_by_default():
-    """A kernel whose body is a sequence of loop nests is one launch of one 1024-work-item workgroup with barriers
-    between the nests (the emulation runs such a workgroup as real threads); a body with nothing to spread over
-    work-items stays one work-item."""
+def test_generated_sources_compile_for_the_device():
+    """The emulation compiles the generated source with the host compiler, which does not see what only the device
+    compiler refuses (a pragma in the wrong place, a builtin spelled wrongly): hipcc cross-compiles the source of a
+    few components with every form of a nest for gfx950 here, without a GPU."""
+    import tempfile
+
+    from i_amd import Component as i, I
+
+    hipcc = Path(os.environ.get("ROCM_PATH", "/opt/rocm")) / "bin" / "hipcc"
+    if not hipcc.exists():
+        pytest.skip("no hipcc here")
+    s = "i:16,j:16"
+    comps = [i("+ij~."), i("+ij~j"), (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij"), i("+bij~b"), i(">ij~i|j:16|ijj'"),
+             i("ij*j~ij||ij") >> i("+ij~i||ij0"),
+             (I & i(f">ij~i|{s}|jii'j'")) >> i(f"ij-i~ij|{s}|1jii'j'"), i(f"ik*jk~ijk | {s} | jii'j'k") >> i(f"+ijk~ij | {s} | jii'j'k0")]
+    with tempfile.TemporaryDirectory() as tmp:
+        for n, comp in enumerate(comps):
+            code = comp._code()
+            src = Path(tmp) / f"c{n}.hip"
+            src.write_text(code[code.index("// generated by the i gfx950 backend"):])
+            r = subprocess.run([str(hipcc), "--genco", "--offload-arch=gfx950", "-O1", "-std=c++17", str(src), "-o", str(src) + ".hsaco"],
+                               capture_output=True, text=True, timeout=600)
+            assert r.returncode == 0, (n, r.stderr[-1500:])
+
+
+def test_every_loop_nest_of_a_kernel_is_a_kernel_of_its_own():
+    """A kernel whose body is a sequence of loop nests is generated as one kernel per nest, each with the buffers its
+    nest touches and a grid of its own; the initialisation of a scalar stays with the nest that accumulates into it.
+    Nests that only accumulate also get the form with their outermost sequential loop in parts."""
     env = dict(os.environ, ILANG_NO_TORCH="1")
-    env.pop("ILANG_HIP_PHASES", None)
     code = ("from i_amd import Component as i, I\n"
             "print(((I & i('+ij~j||ij')) >> i('ij/j~ij||1ij'))._code())\n"
+            "print('=====')\n"
             "print(i('+ij~.')._code())")
     out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300).stdout
-    assert "one workgroup of 1024 work-items runs the 2 loop nests one after the other, a barrier between them" in out
-    assert "nest 0, work-items: " in out and "nest 1, work-items: " in out
-    assert "void __launch_bounds__(1024) f0(Args_f0 args)" in out and out.count("__syncthreads();") == 1
-    assert "work-items: 1 (no independent outer loop)" in out
-
-
-def test_phase_plan_is_reported(shim_lib):
-    env = dict(os.environ, ILANG_HIP_PHASES="1", ILANG_NO_TORCH="1")
-    code = ("from i_amd import Component as i, I\n"
-            "c = (I & i('>ij~i|i:16,j:16|jii\\'j\\'')) >> i('ij-i~ij|i:16,j:16|1jii\\'j\\'')\n"
-            "print(c._code())")
-    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300).stdout
-    assert "launch f0_p0, work-items: i5 i6" in out and "launch f0_p1, work-items: i0 i1 i2 i3" in out
-    assert 'void __launch_bounds__(64) f0_p0(Args_f0 args)' in out
+    colnorm, total = out.split("=====")
+    assert "1 kernel(s)" in colnorm and "loop nest as kernel f0, work-items: i3" in colnorm and "loop nest as kernel f1, work-items: i0 i1" in colnorm
+    assert "f0_g, loop i2 in parts" in colnorm and "__syncthreads" not in colnorm
+    assert 'void __launch_bounds__(64) f0_g(Args_f0_g args)' in colnorm and "ilang_combine" in colnorm
+    # the column sums stay in a register across the rows: one load before the loop over i2 and one store after it
+    assert "float h0_i2 = " in colnorm
+    assert "generated as f0, work-items: 1 (no independent outer loop)" in total
+    assert "f0_g / f0_gw, loop i0 in parts" in total and "for (size_t i0 = part * share_i0; i0 < end_i0; ++i0)" in total
