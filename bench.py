@@ -417,6 +417,19 @@ def main():
         _, lib_ms = time_steps(torch, lambda: torch.matmul(a, bt_), short_steps, short_warmup)
         lib_ghz = clock_beside(lambda: torch.matmul(a, bt_), lib_ms)
 
+    # ------------------------------------------------------------------ the reference's own entry point: mm_t 4096^3 on
+    # host f32 buffers through i_exec_into (upload, f32 MFMA kernel, download, wait).  The operands cross PCIe in
+    # page-locked chunks that several host threads fill and empty while the chunk before is in flight.
+    host_c = np.empty((M, M), np.float32)
+    mm.into(host_c, a_host, b_host)
+    host_kernel = mm.report().split()[1]
+    host_calls = 5 if args.steps >= 20 else 1
+    t0 = time.perf_counter()
+    for _ in range(host_calls):
+        mm.into(host_c, a_host, b_host)
+    host_s = (time.perf_counter() - t0) / host_calls
+    host_err = float(np.abs(host_c[:64] - (a_host[:64].astype(np.float64) @ b_host.astype(np.float64).T)).max() / np.abs(host_c[:64]).max())
+
     if args.calibrate_copy:
         y.copy_(x)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
@@ -555,6 +568,11 @@ def main():
              "roofline": roof("mfma", f32_tflops, PEAK_F32_TFLOPS, "TFLOP/s", "flash_attention_B2_H32_N4096_d128_f32.md",
                               f32_kernel, f32_ms),
              "cpu_baseline": cpuf, "rel_err": errf},
+            {"workload": "mm_t f32 M=N=K=4096 through the host entry point i_exec_into (host f32 buffers in pageable memory: the "
+                         "reference's own ABI; PCIe-inclusive, never the headline)",
+             "value": 2.0 * M ** 3 / host_s / 1e12, "unit": "TFLOP/s", "ms_per_call": host_s * 1e3, "kernel": host_kernel,
+             "pcie_GBps": 3.0 * M * M * 4 / host_s / 1e9, "bytes_over_pcie": 3 * M * M * 4, "calls": host_calls,
+             "rel_err_against_f64": host_err},
             {"workload": f"flash_attention_fwd of one head, bf16 [1,{2 * N},{D}] (not a BASELINE configuration): 64 query "
                          "tiles of 128 rows for 256 CUs, so the keys of the head run in parts over workgroups",
              "value": one_flop / (one_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_call": one_ms, "launches": one_launches,

@@ -14,6 +14,7 @@
 #include "../../../include/i_hip.h"
 #include "../backend_hip/program.h"
 #include "../runtime/hip_rt.h"
+#include "../runtime/host_copy.h"
 #include "../runtime/static_scratch.h"
 #include "error.h"
 #include "handles.h"
@@ -75,8 +76,9 @@ std::vector<std::vector<size_t>> host_shapes(const ihipc::Program& p, const i_te
 // at most ILANG_HIP_STAGING_MB (default 1024; 0: every operand is allocated, copied and freed on its own).  Calls
 // whose operands fit 8 MiB go through a page-locked host mirror of the block as well: the inputs are gathered
 // there and cross in one asynchronous copy, the outputs come back in one, instead of a blocking copy from pageable
-// memory per operand.  A call that finds the block in use by another thread, or needs more, allocates as before;
-// so does the emulated runtime, whose allocations are guarded one by one.
+// memory per operand.  Larger operands cross in page-locked chunks that several host threads fill and empty while
+// the chunk before is in flight (runtime/host_copy.h).  A call that finds the block in use by another thread, or
+// needs more, allocates as before.
 struct Staging {
   void* base = nullptr;
   size_t capacity = 0;
@@ -182,7 +184,7 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
     }
     if (mirror) {
       if (n) std::memcpy(mirror + (static_cast<char*>(t.data) - block_base), inputs[i].data, n * 4);
-    } else if (ihip::Err e = ihip::h2d(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
+    } else if (ihip::Err e = ihip::upload_pipelined(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
       cleanup();
       return e;
     }
@@ -216,7 +218,7 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
     size_t n = 1;
     for (size_t d : out_shapes[o]) n *= d;
     if (n && !out_ptrs[o]) err = "output " + std::to_string(o) + " has no data";
-    else if (!mirror) err = ihip::d2h(out_ptrs[o], out[o].data, n * 4, stream);
+    else if (!mirror) err = ihip::download_pipelined(out_ptrs[o], out[o].data, n * 4, stream);
   }
   if (mirror && err.empty() && carve - block_base > (ptrdiff_t)input_bytes)
     err = ihip::d2h(mirror + input_bytes, block_base + input_bytes, (size_t)(carve - block_base) - input_bytes, stream);
@@ -380,6 +382,28 @@ int i_exec_into(const i_program* program, const i_tensor* inputs, size_t input_c
   if (input_count > 0 && !inputs) return fail("null inputs");
   if (output_count != ihipc::output_count(*program->inner)) return fail("wrong output count");
   if (output_count > 0 && !outputs) return fail("null outputs");
+  // An output whose extents the caller states is checked against what the program writes: a smaller buffer would be
+  // overrun on the host.  (The reference takes the caller's word, core/src/lib.rs:200-225; a tensor without a shape
+  // array is taken on trust here too.)
+  {
+    std::vector<std::vector<size_t>> written;
+    if (std::string e = ihipc::output_shapes(*program->inner, host_shapes(*program->inner, inputs, input_count), &written); !e.empty())
+      return fail(e);
+    for (size_t o = 0; o < output_count && o < written.size(); ++o) {
+      if (!outputs[o].shape) continue;
+      bool same = outputs[o].rank == written[o].size();
+      for (size_t d = 0; same && d < written[o].size(); ++d) same = outputs[o].shape[d] == written[o][d];
+      if (!same) {
+        auto text = [](const size_t* dims, size_t rank) {
+          std::string t = "[";
+          for (size_t d = 0; d < rank; ++d) t += (d ? ", " : "") + std::to_string(dims[d]);
+          return t + "]";
+        };
+        return fail("output " + std::to_string(o) + " has shape " + text(outputs[o].shape, outputs[o].rank) + ", the program writes " +
+                    text(written[o].data(), written[o].size()));
+      }
+    }
+  }
   std::vector<float*> out_ptrs;
   for (size_t o = 0; o < output_count; ++o) out_ptrs.push_back(outputs[o].data);
   const std::string err = run_host(*program->inner, inputs, input_count, out_ptrs);

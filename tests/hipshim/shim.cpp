@@ -110,6 +110,10 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKin
   return hipSuccess;
 }
 hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+// (no page-locked memory here, so the library never gets as far as the events of its chunked host copies)
+hipError_t hipEventCreateWithFlags(hipEvent_t*, unsigned) { return hipErrorNotSupported; }
+hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipErrorNotSupported; }
+hipError_t hipEventSynchronize(hipEvent_t) { return hipErrorNotSupported; }
 
 hipError_t hipModuleLoadData(hipModule_t* mod, const void* image) {
   const auto* eh = static_cast<const Elf64_Ehdr*>(image);

@@ -91,6 +91,22 @@ def test_exec_into_checks_output_count_before_touching_the_device():
     assert nat.last_error() == "null outputs"
 
 
+def test_exec_into_refuses_an_output_whose_stated_extents_are_not_what_the_program_writes():
+    """A caller that states the extents of its output buffer (i_tensor_mut.shape) and states them too small would
+    have its buffer overrun by the copy back to the host; the call is refused before anything runs.  The Python
+    frontend states the extents of every NumPy output."""
+    prog = i("+ij~i")
+    program = prog._compile()
+    x = np.zeros((4, 9), np.float32)
+    arr, keep = ilang._pack([ilang._operand(x, "input")], on_device=False)
+    for wrong in (np.zeros((3,), np.float32), np.zeros((4, 1), np.float32), np.zeros((5,), np.float32)):
+        out, keep_out = ilang._pack([ilang._operand(wrong, "output")], on_device=False)
+        assert core.i_exec_into(program, arr, 1, out, 1) == -1
+        assert "the program writes [4]" in nat.last_error() and "output 0 has shape" in nat.last_error()
+    with pytest.raises(RuntimeError, match="the program writes"):
+        prog.into(np.zeros((2,), np.float32), x)
+
+
 def test_identity_program_is_rejected_like_the_reference():
     # a program output that is a program input has no kernel to produce it
     with pytest.raises(RuntimeError) as err:
