@@ -49,6 +49,8 @@ core.i_hip_program_clock_probe.argtypes = [vp, vp]
 core.i_hip_program_clock_probe.restype = ctypes.c_int
 core.i_hip_shader_clock_probe.argtypes = [vp, ctypes.c_uint, vp]
 core.i_hip_shader_clock_probe.restype = ctypes.c_int
+core.i_hip_release_cached_memory.argtypes = []
+core.i_hip_release_cached_memory.restype = sz
 core.i_hip_program_option.argtypes = [vp, ctypes.c_char_p, ctypes.c_int]
 core.i_hip_program_option.restype = ctypes.c_int
 core.i_hip_program_report.argtypes = [vp]

@@ -46,19 +46,55 @@ std::string ref_name(BufferRef r) {
 struct Arena {
   void* base = nullptr;
   size_t capacity = 0;
+  size_t last_use = 0;  // (guarded by the table's mutex)
   std::mutex busy;  // held by the call that carves from it
 };
 
+// At most 16 (device, stream) pairs keep a block.  A stream beyond that takes the place of the pair that has gone
+// unused the longest (an application with a stream per request: its short-lived streams pass through, the
+// long-lived ones keep their blocks); an entry is never destroyed, so a call that holds one is never left without.
+struct ArenaTable {
+  std::mutex mu;
+  std::map<std::pair<int, hipStream_t>, std::unique_ptr<Arena>> arenas;
+  size_t clock = 0;
+};
+ArenaTable& arena_table() {
+  static ArenaTable* table = new ArenaTable();
+  return *table;
+}
+
 Arena* arena_of(hipStream_t stream) {
-  static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, std::unique_ptr<Arena>> arenas;
+  ArenaTable& t = arena_table();
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  const auto found = arenas.find({device, stream});
-  if (found != arenas.end()) return found->second.get();
-  if (arenas.size() >= 16) return nullptr;  // (an application with a stream per request: the later streams allocate)
-  return (arenas[{device, stream}] = std::make_unique<Arena>()).get();
+  std::lock_guard<std::mutex> lock(t.mu);
+  auto found = t.arenas.find({device, stream});
+  if (found == t.arenas.end()) {
+    if (t.arenas.size() < 16) {
+      found = t.arenas.emplace(std::make_pair(device, stream), std::make_unique<Arena>()).first;
+    } else {
+      auto oldest = t.arenas.end();
+      for (auto it = t.arenas.begin(); it != t.arenas.end(); ++it)
+        if (it->first.first == device && (oldest == t.arenas.end() || it->second->last_use < oldest->second->last_use)) oldest = it;
+      if (oldest == t.arenas.end()) return nullptr;
+      std::unique_lock<std::mutex> idle(oldest->second->busy, std::try_to_lock);
+      if (!idle.owns_lock()) return nullptr;  // (in use right now: this call allocates)
+      // what the old stream's last call left in the block may still be running: the block goes back stream-ordered
+      // on that stream when the stream still exists, else at once
+      if (oldest->second->base && hipFreeAsync(oldest->second->base, oldest->first.second) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(oldest->second->base);
+      }
+      oldest->second->base = nullptr;
+      oldest->second->capacity = 0;
+      idle.unlock();
+      std::unique_ptr<Arena> moved = std::move(oldest->second);
+      t.arenas.erase(oldest);
+      found = t.arenas.emplace(std::make_pair(device, stream), std::move(moved)).first;
+    }
+  }
+  found->second->last_use = ++t.clock;
+  return found->second.get();
 }
 
 size_t arena_limit() {
@@ -151,7 +187,7 @@ struct Run {
   // A temporary that a launch can do without (the parts of a split loop): with a workspace, which is small and whose
   // sizing pass only adds up, at most 20 MiB are taken for one, so that most of what fits unsplit still fits.
   bool alloc_optional(void** ptr, size_t bytes) {
-    if (workspace && bytes > (size_t(20) << 20)) return false;
+    if (workspace && (workspace->refuse_optional || bytes > (size_t(20) << 20))) return false;
     return alloc(ptr, bytes).empty();
   }
 
@@ -1092,10 +1128,26 @@ std::string last_report(Program& p) {
   return p.last_report;
 }
 
+size_t release_stream_blocks() {
+  ArenaTable& t = arena_table();
+  std::lock_guard<std::mutex> lock(t.mu);
+  size_t released = 0;
+  for (auto& [key, arena] : t.arenas) {
+    std::unique_lock<std::mutex> idle(arena->busy, std::try_to_lock);
+    if (!idle.owns_lock() || !arena->base) continue;
+    (void)hipFree(arena->base);  // (waits for what still runs on the device)
+    released += arena->capacity;
+    arena->base = nullptr;
+    arena->capacity = 0;
+  }
+  return released;
+}
+
 std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
-                            size_t* bytes) {
+                            size_t* bytes, bool refuse_optional) {
   ihip::DryRun nothing_is_launched;
   Workspace sizing;
+  sizing.refuse_optional = refuse_optional;
   sizing.base = reinterpret_cast<void*>(uintptr_t(256));  // never dereferenced: only has to be non-null
   const std::string err = execute(p, inputs, outputs, nullptr, &sizing);
   *bytes = sizing.used;

@@ -75,6 +75,9 @@ struct Workspace {
   void* base = nullptr;
   size_t limit = 0;
   size_t used = 0;
+  // temporaries that a launch can do without (the parts of a split loop) are not taken from the workspace at all:
+  // for operands whose mandatory temporaries fit it only without them
+  bool refuse_optional = false;
 };
 
 // Enqueue the program on `stream`.  All tensors live in device memory.
@@ -94,6 +97,10 @@ std::string last_report(Program& p);
 
 // What execute() with a workspace would take from it for these operands, in bytes.  Launches nothing.
 std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,
-                            size_t* bytes);
+                            size_t* bytes, bool refuse_optional = false);
+
+// Frees the blocks of device memory that execute() keeps per stream for temporaries (those not in use by a call at
+// this moment); returns the bytes released.
+size_t release_stream_blocks();
 
 }  // namespace ihipc

@@ -87,15 +87,44 @@ struct Staging {
 };
 constexpr size_t kPinnedBytes = size_t(8) << 20;
 
+struct StagingTable {
+  std::mutex mu;
+  std::map<int, std::unique_ptr<Staging>> blocks;
+};
+StagingTable& staging_table() {
+  static StagingTable* table = new StagingTable();
+  return *table;
+}
 Staging* staging_of_current_device() {
-  static std::mutex mu;
-  static std::map<int, std::unique_ptr<Staging>> blocks;
+  StagingTable& t = staging_table();
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  auto& block = blocks[device];
+  std::lock_guard<std::mutex> lock(t.mu);
+  auto& block = t.blocks[device];
   if (!block) block = std::make_unique<Staging>();
   return block.get();
+}
+
+// Frees the blocks that no call is using at this moment; returns the bytes released (device and page-locked).
+size_t release_staging_blocks() {
+  size_t released = 0;
+  StagingTable& t = staging_table();
+  std::lock_guard<std::mutex> lock(t.mu);
+  for (auto& [device, block] : t.blocks) {
+    std::unique_lock<std::mutex> idle(block->busy, std::try_to_lock);
+    if (!idle.owns_lock()) continue;
+    if (block->base) {
+      ihip::dev_free(block->base);
+      released += block->capacity;
+    }
+    if (block->pinned) {
+      (void)hipHostFree(block->pinned);
+      released += kPinnedBytes;
+    }
+    block->base = block->pinned = nullptr;
+    block->capacity = 0;
+  }
+  return released;
 }
 
 size_t staging_limit() {
@@ -472,17 +501,31 @@ int i_exec_into_device_noalloc(const i_program* program, const i_device_tensor* 
     void* base = nullptr;
     if (ihip::Err e = ihip::static_scratch(&base); !e.empty()) return fail(e);
     // size the temporaries first, so that a program that does not fit is refused before anything is enqueued
+    // (with the temporaries of split loops first; when that is too much, without them: the loops then run whole)
     size_t need = 0;
+    bool refuse_optional = false;
     if (std::string e = ihipc::workspace_bytes(*program->inner, in, out, &need); !e.empty()) return fail(e);
+    if (need > ihip::kStaticScratchBytes) {
+      refuse_optional = true;
+      if (std::string e = ihipc::workspace_bytes(*program->inner, in, out, &need, true); !e.empty()) return fail(e);
+    }
     if (need > ihip::kStaticScratchBytes)
       return fail("program needs " + std::to_string(need) + " bytes of temporaries for these operands, the static workspace holds " +
                   std::to_string(ihip::kStaticScratchBytes) + " (use i_exec_into_device)");
-    ihipc::Workspace ws{base, ihip::kStaticScratchBytes, 0};
+    ihipc::Workspace ws{base, ihip::kStaticScratchBytes, 0, refuse_optional};
     const std::string err = ihipc::execute(*program->inner, in, out, static_cast<hipStream_t>(stream), &ws);
     return err.empty() ? 0 : fail(err);
   } catch (const std::exception& e) {
     return fail(e.what());
   }
+}
+
+size_t i_hip_release_cached_memory(void) {
+  size_t released = ihipc::release_stream_blocks();
+  released += release_staging_blocks();
+  released += ihip::release_copy_chunks();
+  released += ihip::trim_temp_pool();
+  return released;
 }
 
 int i_hip_program_option(i_program* program, const char* name, int value) {

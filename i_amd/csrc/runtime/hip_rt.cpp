@@ -139,6 +139,20 @@ Err temp_alloc(void** p, size_t bytes, hipStream_t stream) {
   return check(hipMallocAsync(p, bytes, stream), "hipMallocAsync");
 }
 
+size_t trim_temp_pool() {
+  std::lock_guard<std::mutex> lock(g_mu);
+  size_t released = 0;
+  for (auto& [dev, dm] : g_builtin) {
+    if (!dm.pool) continue;
+    uint64_t before = 0, after = 0;
+    (void)hipMemPoolGetAttribute(dm.pool, hipMemPoolAttrReservedMemCurrent, &before);
+    if (hipMemPoolTrimTo(dm.pool, 0) != hipSuccess) (void)hipGetLastError();
+    (void)hipMemPoolGetAttribute(dm.pool, hipMemPoolAttrReservedMemCurrent, &after);
+    if (before > after) released += (size_t)(before - after);
+  }
+  return released;
+}
+
 Err dev_alloc(void** p, size_t bytes) {
   *p = nullptr;
   if (bytes == 0) bytes = 4;

@@ -41,6 +41,9 @@ Err dev_alloc(void** p, size_t bytes);
 // a temporary that hipFreeAsync(p, stream) gives back, from the library's own pool of the current device
 Err temp_alloc(void** p, size_t bytes, hipStream_t stream);
 void dev_free(void* p);
+// Hands the freed memory that the library's pools of temporaries hold back to the system; returns the bytes (0 when
+// the runtime cannot tell).
+size_t trim_temp_pool();
 Err h2d(void* dst, const void* src, size_t bytes, hipStream_t stream);
 Err d2h(void* dst, const void* src, size_t bytes, hipStream_t stream);
 Err sync(hipStream_t stream);

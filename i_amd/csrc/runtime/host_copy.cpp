@@ -101,13 +101,20 @@ struct Ring {
   }
 };
 
+struct RingTable {
+  std::mutex mu;
+  std::map<int, std::unique_ptr<Ring>> rings;
+};
+RingTable& ring_table() {
+  static RingTable* table = new RingTable();
+  return *table;
+}
 Ring* ring_of_current_device() {
-  static std::mutex mu;
-  static std::map<int, std::unique_ptr<Ring>> rings;
+  RingTable& t = ring_table();
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  auto& ring = rings[device];
+  std::lock_guard<std::mutex> lock(t.mu);
+  auto& ring = t.rings[device];
   if (!ring) ring = std::make_unique<Ring>();
   return ring.get();
 }
@@ -128,6 +135,26 @@ bool prepare(Ring* ring) {
 }
 
 }  // namespace
+
+size_t release_copy_chunks() {
+  RingTable& t = ring_table();
+  std::lock_guard<std::mutex> lock(t.mu);
+  size_t released = 0;
+  for (auto& [device, ring] : t.rings) {
+    std::unique_lock<std::mutex> idle(ring->busy, std::try_to_lock);
+    if (!idle.owns_lock() || !ring->ready) continue;
+    for (int c = 0; c < kChunks; ++c) {
+      (void)ring->settle(c);
+      (void)hipHostFree(ring->chunk[c]);
+      (void)hipEventDestroy(ring->landed[c]);
+      ring->chunk[c] = nullptr;
+      ring->landed[c] = nullptr;
+      released += kChunkBytes;
+    }
+    ring->ready = false;
+  }
+  return released;
+}
 
 Err upload_pipelined(void* dst, const void* src, size_t bytes, hipStream_t stream) {
   Ring* ring = bytes >= kPipelinedCopyBytes ? ring_of_current_device() : nullptr;

@@ -21,4 +21,7 @@ Err download_pipelined(void* dst, const void* src, size_t bytes, hipStream_t str
 // From this size on the two calls above pay (below it one plain copy does)
 constexpr size_t kPipelinedCopyBytes = size_t(8) << 20;
 
+// Frees the page-locked chunks of every device (those that no transfer is using at this moment); returns the bytes.
+size_t release_copy_chunks();
+
 }  // namespace ihip

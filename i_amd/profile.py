@@ -22,7 +22,10 @@ from collections import namedtuple
 KernelRow = namedtuple("KernelRow", "name calls total_us avg_us min_us max_us share lds_bytes workgroup")
 CounterRow = namedtuple("CounterRow", "kernel counter dispatches avg min max")
 
-_OURS = re.compile(r"^(attn_fwd_|gemm_n[nt]_|row_(softmax|shift|norm|exp|scaled_softmax)_|transpose_b(16|32)|convert_|f\d+(_p\d+)?$)")
+# every name the backend can launch: the hand-written kernels (kernels/kernels.hip), the generated kernels f<k> in
+# their forms (_w: a wavefront per iteration, _g / _gw: a loop in parts) and the helpers generated beside them
+_OURS = re.compile(r"^(attn_fwd_|attn_kv_merge$|gemm_n[nt]_|splitk_reduce$|row_(softmax|shift|norm|exp|scaled_softmax)_|transpose_b(16|32)$|"
+                   r"pad_rows_b(16|32)$|convert_|shader_clock_probe$|ilang_(fill|combine|combine_w)$|f\d+(_w|_g|_gw)?$)")
 
 
 def is_backend_kernel(name):

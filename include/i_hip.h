@@ -48,6 +48,15 @@ typedef struct {
  * kernels where a kernel has one and are widened on the device otherwise;
  * each output is written in its own dtype.  Output shapes, when given
  * (rank > 0), are checked against i_output_shapes.
+ *
+ * Precision of bf16 attention: by default the fused kernels fold scale * log2(e) into Q, rounded to bf16 once
+ * more, which saves one multiply per score (about 5 % of the time) and perturbs every score by about
+ * 2^-9.5 * |q . k| * scale nats.  At the magnitudes attention has (inputs of unit variance, scores within +-30
+ * nats) the result stays within 1e-2 of an f32 computation, relative to max |result|; at scores beyond about
+ * +-30 nats (inputs x 3) it leaves the 2e-2 bar of the reference comparison (up to 2.4e-2 measured).  Callers
+ * with such scores set i_hip_program_option(program, "attention.f32_scale", 1): the scale is then applied in f32
+ * to every score, the reference's own arithmetic (compiler/src/lower/exec_plan_to_module.rs:605-640), and the
+ * error stays below 1e-2 at any score magnitude.  f32 operands never fold anything.
  */
 int i_exec_into_device(const i_program* program,
                        const i_device_tensor* inputs, size_t input_count,
@@ -156,6 +165,18 @@ int i_hip_program_clock_probe(i_program* program, void* ticks);
  * work in question.  It occupies one wave slot of one compute unit while it sleeps.
  */
 int i_hip_shader_clock_probe(void* ticks, unsigned microseconds, void* stream);
+
+/*
+ * Memory that the library keeps from call to call, so that a call allocates nothing after the first of its kind: per
+ * (device, stream), for the 16 pairs used most recently, a block for temporaries (at most ILANG_HIP_ARENA_MB, default
+ * 256 MiB each); per device a block for the device copies of host operands (at most ILANG_HIP_STAGING_MB, default
+ * 1 GiB) with an 8 MiB page-locked mirror, four page-locked chunks of 8 MiB for large host operands, up to 1 GiB of
+ * freed temporaries in the library's own memory pool, and the fixed workspace of i_exec_into_device_noalloc
+ * (I_HIP_STATIC_WORKSPACE_BYTES, part of the loaded library).  This call frees all of it except the last, as far as
+ * no call is using it at the moment, and returns the bytes released; the next calls allocate again.  No counterpart
+ * in the reference, whose generated exec mallocs and frees on every call.
+ */
+size_t i_hip_release_cached_memory(void);
 
 /*
  * What the last i_exec* of this program dispatched, one line per kernel of the plan that i_code prints:

@@ -114,6 +114,10 @@ hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 hipError_t hipEventCreateWithFlags(hipEvent_t*, unsigned) { return hipErrorNotSupported; }
 hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipErrorNotSupported; }
 hipError_t hipEventSynchronize(hipEvent_t) { return hipErrorNotSupported; }
+hipError_t hipEventDestroy(hipEvent_t) { return hipErrorNotSupported; }
+hipError_t hipHostFree(void*) { return hipErrorNotSupported; }
+hipError_t hipMemPoolGetAttribute(hipMemPool_t, hipMemPoolAttr, void*) { return hipErrorNotSupported; }
+hipError_t hipMemPoolTrimTo(hipMemPool_t, size_t) { return hipErrorNotSupported; }
 
 hipError_t hipModuleLoadData(hipModule_t* mod, const void* image) {
   const auto* eh = static_cast<const Elf64_Ehdr*>(image);

@@ -108,6 +108,45 @@ def test_split_loops_keep_their_partial_results_in_the_workspace(torch, monkeypa
         assert "(keys in 3 parts)" in attention.report(), attention.report()
 
 
+def test_temporaries_that_a_launch_can_do_without_are_left_out_when_the_rest_only_fits_without_them(torch):
+    """An f32 product whose contracted extent is no multiple of 4: both operands are copied into temporaries with
+    padded rows (61.4 MiB here, which the kernels cannot run without), and its k loop would be split over workgroups
+    (partial products of a few MiB more, which they can).  Together that exceeds the fixed array; the call then
+    runs the loop whole instead of being refused, and a smaller problem afterwards splits again."""
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    for m, n, k, splits in ((64, 1900, 8190, False), (64, 300, 4102, True)):
+        print("case optional temporaries", (m, n, k), flush=True)
+        a, b = randn(torch, (m, k), 5), randn(torch, (n, k), 6)
+        out = torch.full((m, n), float("nan"), device="cuda")
+        assert call(nat.core.i_exec_into_device_noalloc, mm_t, [a, b], [out], torch) == 0, nat.last_error()
+        assert ("parts)" in mm_t.report()) == splits, mm_t.report()
+        ref = a.double() @ b.double().T
+        assert float((out.double() - ref).abs().max() / ref.abs().max()) <= 1e-4
+        whole = torch.full((m, n), float("nan"), device="cuda")
+        assert call(nat.core.i_exec_into_device, mm_t, [a, b], [whole], torch) == 0, nat.last_error()
+        assert "parts)" in mm_t.report(), mm_t.report()
+        assert float((out - whole).abs().max()) <= 1e-4 * float(ref.abs().max())
+
+
+def test_cached_memory_can_be_released_and_comes_back(torch):
+    """i_hip_release_cached_memory frees the blocks the library keeps from call to call (per-stream temporaries, the
+    device copies and page-locked chunks of host operands, its pool of freed temporaries); the calls after it
+    allocate again and give the same results."""
+    comp = softmax_naive()
+    x = randn(torch, (512, 1000), 7)
+    first = comp.exec_torch(x)
+    host = comp.exec_numpy(x.cpu().numpy())  # the host entry: a kept device block for the operands' copies
+    big = np.ones((2100, 1024), np.float32)  # 8.2 MiB: through the page-locked chunks
+    assert np.array_equal(i("ij+ij~ij").exec_numpy(big, big), big + big)
+    torch.cuda.synchronize()
+    released = nat.core.i_hip_release_cached_memory()
+    assert released >= (2 * 512 * 1000 * 4) + (4 << 23), released  # the softmax intermediates' block and the four 8 MiB chunks at least
+    assert nat.core.i_hip_release_cached_memory() == 0  # nothing left to give back
+    assert torch.equal(comp.exec_torch(x), first)
+    assert np.array_equal(comp.exec_numpy(x.cpu().numpy()), host)
+    assert np.array_equal(i("ij+ij~ij").exec_numpy(big, big), big + big)
+
+
 def test_both_device_entry_points_under_graph_capture(torch):
     """What the entry point that allocates nothing is for: captured into a HIP graph (after one eager call, which
     loads the code object and compiles the generated kernels) and replayed three times, with new input values,
