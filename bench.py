@@ -410,12 +410,18 @@ def main():
     # on the same operands as the mm_t line: a practical ceiling for dense bf16 on random data on this box, next to
     # which the MFMA lines can be read.  Not part of the product path; the shader clock under dense MFMA work on
     # random operands stays well below the 2.4 GHz the 2.5 PFLOP/s peak is quoted at.
-    lib_ms = lib_ghz = None
+    lib_ms = lib_ghz = lib32_ms = None
     if args.steps >= 20:
         bt_ = b.t()
         torch.matmul(a, bt_)
         _, lib_ms = time_steps(torch, lambda: torch.matmul(a, bt_), short_steps, short_warmup)
         lib_ghz = clock_beside(lambda: torch.matmul(a, bt_), lib_ms)
+        # the same product with an f32 result, which is what the mm_t line writes (twice the bytes stored)
+        try:
+            torch.mm(a, bt_, out_dtype=torch.float32)
+            _, lib32_ms = time_steps(torch, lambda: torch.mm(a, bt_, out_dtype=torch.float32), short_steps, short_warmup)
+        except (TypeError, RuntimeError):
+            lib32_ms = None
 
     # ------------------------------------------------------------------ the reference's own entry point: mm_t 4096^3 on
     # host f32 buffers through i_exec_into (upload, f32 MFMA kernel, download, wait).  The operands cross PCIe in
@@ -527,7 +533,11 @@ def main():
             "frac_of_peak": 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
             "shader_clock_ghz": lib_ghz,
             "frac_at_measured_clock": None if not lib_ghz else 2.0 * M ** 3 / (lib_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS * NOMINAL_GHZ / lib_ghz,
-            "shader_clock_source": "a one-wavefront kernel on a second stream beside a second batch of launches (i_hip_shader_clock_probe)"},
+            "shader_clock_source": "a one-wavefront kernel on a second stream beside a second batch of launches (i_hip_shader_clock_probe)",
+            "f32_out": None if lib32_ms is None else {
+                "workload": "the same product with an f32 result (torch.mm, out_dtype float32), as the mm_t line writes it",
+                "value": 2.0 * M ** 3 / (lib32_ms * 1e-3) / 1e12, "kernel_ms": lib32_ms,
+                "frac_of_peak": 2.0 * M ** 3 / (lib32_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}},
         "secondary": [
             {"workload": "row_softmax f32 [16384,4096] (BASELINE configs[1]); the steps rotate over 4 input/output pairs (2 GiB) so that nothing is re-read from the Infinity Cache", "value": sm_gbs, "unit": "GB/s",
              "roofline": roof("hbm", sm_gbs, PEAK_HBM_GBS, "GB/s", "row_softmax_16384x4096_f32.md", sm_kernel, sm_ms),

@@ -3,7 +3,6 @@
 // hipModuleGetFunction; each takes one parameter block by value (params.h).
 #include "attention_bf16.h"
 #include "attention_bf16_direct.h"
-#include "attention_bf16_q64.h"
 #include "attention_f32.h"
 #include "attention_f32_direct.h"
 #include "gemm_nt_bf16.h"
@@ -64,9 +63,9 @@ ATTN_BF16_DIRECT(256, 32, 4, 1, , false)
 ATTN_BF16_DIRECT_PAD(256, 32, 4, 1, , false)
 ATTN_BF16_DIRECT(256, 32, 4, 1, _f32scale, true)
 ATTN_BF16_DIRECT_PAD(256, 32, 4, 1, _f32scale, true)
-// d = 64 with 64 queries per wave (attention_bf16_q64.h): 8 waves, 512 query rows per workgroup, 32-key tiles
+// d = 64 with 64 queries per wave (two query blocks): 8 waves, 512 query rows per workgroup, 32-key tiles
 extern "C" __global__ void __launch_bounds__(512, 1) attn_fwd_bf16_d64_bn32_q64(AttnParams p) {
-  attn_fwd_bf16_q64_body<64, 32, 8>(p);
+  attn_fwd_bf16_direct_body<64, 32, 8, false, false, 2>(p);
 }
 
 #define ATTN_F32(DPAD, BN, NW)                                                             \
