@@ -39,7 +39,7 @@ struct PrivateBuffer {
 // A nest that does nothing but accumulate (sums, products, maxima, minima) under its outermost sequential loop
 // has a third form, <name>_g (and <name>_gw, the wavefront form of the same), for runs whose parallel loops alone
 // cannot fill the chip (a sum to a single element, a column sum of a few thousand columns): the iterations of
-// that loop are dealt out over `parts` groups of work-items, part p taking iterations p, p + parts, ...; every
+// that loop are dealt out over `parts` groups of work-items, part p taking a contiguous share of them; every
 // part accumulates into a copy of its own of each accumulated buffer (a temporary that the launcher fills with
 // the reduction's identity first), and a second kernel, ilang_combine, folds the copies into the buffer in part
 // order.  (GridForm below.)
