@@ -7,7 +7,9 @@
 // is the matrix instruction and what follows from it.  On operands that toggle the datapath (anything but constants) the chip sustains more
 // 16x16x32 MFMAs per second than 32x32x16 ones under its power limit, at the same operand traffic from LDS.
 //
-//   workgroup   WM x WN waves; a wave owns (BT / WM) x (BT / WN) of the tile as TM x TN accumulators of
+//   workgroup   WM x WN waves on a BTM x BTN tile of C (BTM rows of A against BTN rows of B; square but for the
+//               192 x 256 form, which is one full round of workgroups where 256 x 256 tiles leave a partly empty
+//               one: 3072^3, 6144^3); a wave owns (BTM / WM) x (BTN / WN) of the tile as TM x TN accumulators of
 //               16 x 16 (256 x 256 with 2 x 4 waves: 8 x 4 accumulators, 128 registers; with 2 x 2 waves, one per
 //               SIMD: 8 x 8 accumulators, the 256 registers of the accumulation file, a third fewer operand
 //               reads per matrix instruction; that form's matrix instructions are inline assembly, see kstep)
@@ -52,20 +54,23 @@
 #include "common.h"
 #include "params.h"
 
-template <int BT, int WM, int WN, bool EDGE, bool NN, bool KTAIL>
+template <int BTM, int BTN, int WM, int WN, bool EDGE, bool NN, bool KTAIL>
 __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* smem_base, uint32_t tm, uint32_t tn) {
   constexpr int RB = 128;            // bytes per slab row: 64 k of bf16
   constexpr int BK = 64;
   constexpr int NWAVES = WM * WN;
-  constexpr int TM = BT / WM / 16;   // 16-row fragments of A per wave
-  constexpr int TN = BT / WN / 16;   // 16-row fragments of B per wave
+  constexpr int TM = BTM / WM / 16;  // 16-row fragments of A per wave
+  constexpr int TN = BTN / WN / 16;  // 16-row fragments of B per wave
   constexpr int CH = RB / 16;        // 16-byte chunks per row
   constexpr int RPW = 64 / CH;       // rows per wave-load
-  constexpr int SLAB = BT * RB;
-  constexpr int WL = SLAB / 1024;    // wave-loads per slab
-  constexpr int WLW = WL / NWAVES;
-  static_assert(WL % NWAVES == 0 && NWAVES % 2 == 0 && TM >= 2 && TN >= 2, "slab shape");
-  char (*smem)[2][SLAB] = reinterpret_cast<char (*)[2][SLAB]>(smem_base);  // [buffer][A, B]
+  constexpr int SLAB_A = BTM * RB, SLAB_B = BTN * RB, SLABS = SLAB_A + SLAB_B;  // a buffer: the A slab, then the B slab
+  constexpr int WLW_A = SLAB_A / 1024 / NWAVES;  // wave-loads per slab and wave
+  constexpr int WLW_B = SLAB_B / 1024 / NWAVES;
+  constexpr int WLW = WLW_A > WLW_B ? WLW_A : WLW_B;
+  static_assert(SLAB_A % (1024 * NWAVES) == 0 && SLAB_B % (1024 * NWAVES) == 0 && NWAVES % 2 == 0 && TM >= 2 && TN >= 2, "slab shape");
+  static_assert(!NN || BTM == BTN, "the row-major right operand has square tiles only");
+  // slab `which` (0: A, 1: B) of buffer `buf`
+  auto slab = [&](int buf, int which) { return smem_base + buf * SLABS + which * SLAB_A; };
   // (the k loop split over workgroups: blockIdx.y counts (batch, split) pairs)
   const uint32_t nsplit = p.splits > 1 ? p.splits : 1u;
   const uint32_t batch = blockIdx.y / nsplit, split = blockIdx.y - batch * nsplit;
@@ -83,14 +88,14 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   const char* __restrict__ B = reinterpret_cast<const char*>(p.b) + (size_t)batch * p.n * row_bytes +
                                (NN ? (size_t)k_first * p.n * 2 : (size_t)k_first * 2);  // (NN: rows of B are k)
   char* __restrict__ C = reinterpret_cast<char*>(p.c) + (size_t)blockIdx.y * p.m * p.n * (p.out_bf16 ? 2 : 4);
-  const uint32_t m0 = tm * BT, n0 = tn * BT;
+  const uint32_t m0 = tm * BTM, n0 = tn * BTN;
 
   // ---- global -> LDS.  Wave-load w of a slab covers slab rows 8 w .. 8 w + 7; this lane's LDS slot is
   // (row 8 w + lane / 8, chunk lane % 8) and it fetches chunk (lane % 8) ^ ((row / 2) % 8) of that row.
   // w = wave + NWAVES it with NWAVES even, so (row / 2) % 8 = (4 (wave % 2) + lane / 16) % 8 for every `it`.
   const uint32_t lrow = lane / CH, lch = lane % CH;
   const uint32_t gch = lch ^ ((4 * (wave & 1) + lane / 16) % CH);
-  const uint32_t smem0 = lds_address(&smem[0][0][0]);
+  const uint32_t smem0 = lds_address(smem_base);
   // Per-lane byte offset of this lane's 16 bytes from the first row of its wave-load.  EDGE: from the tile's
   // first row, with the row clamped, recomputed at every request (held in registers it would cost 2 WLW of
   // them; the empty asm keeps the compiler from hoisting the values back out of the loop).
@@ -112,7 +117,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   // NN: wave-load w of a B slab covers slab rows (k) RPWN w .. + RPWN - 1; this lane's LDS slot is (row, chunk
   // lane % CHN) and it fetches chunk (lane % CHN) ^ 2 f(row) of that row.  Rounds of wave-loads are 16 rows apart,
   // which changes neither f(row) nor the clamp, so one per-lane offset serves every request.
-  constexpr int RBN = 2 * BT;         // bytes per row of an NN slab
+  constexpr int RBN = 2 * BTN;        // bytes per row of an NN slab
   constexpr int CHN = RBN / 16;       // chunks per row
   constexpr int RPWN = 1024 / RBN;    // rows per wave-load
   // (with four waves a round of wave-loads is 8 rows, and f(row) of a lane alternates between two values from one
@@ -138,32 +143,32 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   auto move = [&](const void* base, uint32_t voff, uint32_t lds_base, bool valid) {
     if constexpr (KTAIL) {
       if (valid) dma16(base, voff, lds_base);
-      else *reinterpret_cast<u32x4*>(&smem[0][0][0] + (lds_base - smem0) + 16 * lane) = u32x4{0, 0, 0, 0};
+      else *reinterpret_cast<u32x4*>(smem_base + (lds_base - smem0) + 16 * lane) = u32x4{0, 0, 0, 0};
     } else {
       dma16(base, voff, lds_base);
     }
   };
-  // request r of the 2 WLW that bring slab s into `buf`; `tail`: slab s may be the partial one (KTAIL)
+  // request r of the WLW_A + WLW_B that bring slab s into `buf` (A first); `tail`: slab s may be the partial one (KTAIL)
   auto request = [&](uint32_t s, int buf, int r, auto tail) {
-    const int it = r % WLW;
+    const int it = r < WLW_A ? r : r - WLW_A;
     const uint32_t w = wave + NWAVES * it;
     const size_t k_byte = (size_t)s * RB;
-    const uint32_t to_a = smem0 + (2 * buf + 0) * SLAB + w * 1024, to_b = smem0 + (2 * buf + 1) * SLAB + w * 1024;
+    const uint32_t to_a = smem0 + buf * SLABS + w * 1024, to_b = smem0 + buf * SLABS + SLAB_A + w * 1024;
     const bool whole = !KTAIL || !decltype(tail)::value || s + 1 < nslabs;  // the slab lies inside k
     const bool valid = whole || gch < tail_chunks;         // ... or this lane's chunk of a K-contiguous row does
-    if (r >= WLW && NN) {
+    if (r >= WLW_A && NN) {
       const bool valid_row = whole || (w * RPWN + lane / CHN) < 8 * tail_chunks;
       move(b_tile + ((size_t)s * BK + NN_ROUND * it) * brow_bytes, boff_nn[NN_ROUND == 8 ? it % 2 : 0], to_b, valid_row);
     } else if constexpr (EDGE) {
-      if (r < WLW) move(a_tile + k_byte, row_offset(it, lim_a), to_a, valid);
+      if (r < WLW_A) move(a_tile + k_byte, row_offset(it, lim_a), to_a, valid);
       else move(b_tile + k_byte, row_offset(it, lim_b), to_b, valid);
     } else if constexpr (TM * TN > 32) {
       // (one wave per SIMD: nothing hides the scalar address arithmetic of a request, so the wave-loads differ in
       // a per-lane offset kept in a register each, and the base moves once per slab)
-      if (r < WLW) move(a_tile + k_byte, voff_it[it], to_a, valid);
+      if (r < WLW_A) move(a_tile + k_byte, voff_it[it], to_a, valid);
       else move(b_tile + k_byte, voff_it[it], to_b, valid);
     } else {
-      if (r < WLW) move(a_tile + k_byte + it * it_stride, voff0, to_a, valid);
+      if (r < WLW_A) move(a_tile + k_byte + it * it_stride, voff0, to_a, valid);
       else move(b_tile + k_byte + it * it_stride, voff0, to_b, valid);
     }
   };
@@ -209,29 +214,29 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   }
 
 #pragma unroll
-  for (int r = 0; r < 2 * WLW; ++r) request(0, 0, r, std::true_type{});
+  for (int r = 0; r < WLW_A + WLW_B; ++r) request(0, 0, r, std::true_type{});
   dma_wait_all();
   __syncthreads();
 
   bf16x8 a[TM], b0[TN], b1[TN];
   auto load_a = [&](int buf, int ks, int i) {
-    a[i] = *reinterpret_cast<const bf16x8*>(&smem[buf][0][0] + a_rows + i * 16 * RB + addr[ks]);
+    a[i] = *reinterpret_cast<const bf16x8*>(slab(buf, 0) + a_rows + i * 16 * RB + addr[ks]);
   };
   auto load_b = [&](int buf, int ks, int j, bf16x8 (&b)[TN]) {
     if constexpr (NN) {
       uint32_t first = baddr0;
       asm volatile("" : "+v"(first));  // (keeps the TN addresses from being hoisted into registers of their own)
-      const char* ba = &smem[buf][1][0] + 32 * ks * RBN + (first ^ (32u * j));
+      const char* ba = slab(buf, 1) + 32 * ks * RBN + (first ^ (32u * j));
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ba + 4 * RBN));
       b[j] = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     } else {
-      b[j] = *reinterpret_cast<const bf16x8*>(&smem[buf][1][0] + b_rows + j * 16 * RB + addr[ks]);
+      b[j] = *reinterpret_cast<const bf16x8*>(slab(buf, 1) + b_rows + j * 16 * RB + addr[ks]);
     }
   };
   // One k-step: TM x TN MFMAs on (a, bc) while a is refilled in place and bn is filled with the operands of
   // k-step `ks` of buffer `buf`; `reqs` says whether the slab requests of this trip ride on it.
-  constexpr int NREQ = 2 * WLW, NSLOT = TM * TN;
+  constexpr int NREQ = WLW_A + WLW_B, NSLOT = TM * TN;
   auto kstep = [&](bf16x8 (&bc)[TN], bf16x8 (&bn)[TN], int buf, int ks, bool refill, auto reqs, uint32_t s_req, int req_buf,
                    auto tail) {
 #pragma unroll
@@ -340,12 +345,12 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   }
 }
 
-template <int BT, int WM, int WN, bool NN = false, bool KTAIL = false>
+template <int BTM, int WM, int WN, bool NN = false, bool KTAIL = false, int BTN = BTM>
 __device__ __forceinline__ void gemm_nt_mfma16_body(const GemmParams& p) {
-  __shared__ __attribute__((aligned(1024))) char smem[4 * BT * 128];  // [buffer][A, B][BT rows][128 bytes]
+  __shared__ __attribute__((aligned(1024))) char smem[2 * (BTM + BTN) * 128];  // [buffer][A: BTM rows, B: BTN rows][128 bytes]
   // ---- tile of this workgroup
   uint32_t tm, tn;
   if (!gemm_tile_of_workgroup(blockIdx.x, blockIdx.y, p.tiles_m, p.tiles_n, tm, tn)) return;
-  if ((tm + 1) * BT <= p.m && (tn + 1) * BT <= p.n) gemm_nt_mfma16_tile<BT, WM, WN, false, NN, KTAIL>(p, smem, tm, tn);
-  else gemm_nt_mfma16_tile<BT, WM, WN, true, NN, KTAIL>(p, smem, tm, tn);
+  if ((tm + 1) * BTM <= p.m && (tn + 1) * BTN <= p.n) gemm_nt_mfma16_tile<BTM, BTN, WM, WN, false, NN, KTAIL>(p, smem, tm, tn);
+  else gemm_nt_mfma16_tile<BTM, BTN, WM, WN, true, NN, KTAIL>(p, smem, tm, tn);
 }

@@ -117,6 +117,15 @@ extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_dir
 extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x256x64_direct_ktail_w4(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 2, false, true>(p);
 }
+// 192 rows of A against 256 rows of B, four waves of 96 x 128 (6 x 8 accumulators): for sizes whose 256 x 256 tiles
+// leave a partly empty last round of workgroups (3072^3: 192 of these fill three quarters of the CUs at once,
+// where 144 tiles of 256 x 256 fill 56 %; 6144^3: three full rounds instead of 2.25)
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_192x256x64_direct_w4(GemmParams p) {
+  gemm_nt_mfma16_body<192, 2, 2, false, false, 256>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_192x256x64_direct_ktail_w4(GemmParams p) {
+  gemm_nt_mfma16_body<192, 2, 2, false, true, 256>(p);
+}
 extern "C" __global__ void __launch_bounds__(256, 1) gemm_nn_bf16_256x256x64_direct_w4(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 2, true>(p);
 }

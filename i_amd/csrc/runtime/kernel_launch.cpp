@@ -40,7 +40,7 @@ Err set_kernel_option(KernelOptions& o, const std::string& name, int value) {
     if (!one_of({0, 4, 8})) return bad("0, 4 or 8");
     o.gemm_waves = value;
   } else if (name == "gemm.tile") {
-    if (!one_of({0, 128, 256})) return bad("0, 128 or 256");
+    if (!one_of({0, 128, 192, 256})) return bad("0, 128, 192 (192 x 256) or 256");
     o.gemm_tile = value;
   } else if (name == "gemm.direct") {
     o.gemm_direct = value != 0;
@@ -307,6 +307,24 @@ static unsigned pick_direct_tile(size_t t256, size_t t128) {
   return e256 >= e128 ? 256 : 128;
 }
 
+// A model of a launch's time in us, by which the 192 x 256 tile is weighed against the one chosen above: a fixed
+// part (launch, first slab, the store of C), plus the slabs of the k loop times the time of a slab for a full round
+// of workgroups (1.5 us on a 256 x 256 tile, 1.154 on 192 x 256, 0.95 on two 128 x 128 tiles per CU), times the
+// rounds, a partly empty round counting for 0.55 + half of its fill (fewer busy CUs run a higher clock and share
+// L2 and the fabric among fewer); less than one round of 128-tiles is cheaper still (one workgroup per CU).
+// Fitted to cubes from 1792 to 8192, where it is within 5 % of the measured times of all three tiles but for the
+// 192 x 256 tile from 7168 on, which it flatters by 8 %: that tile has to win by 8 % to be taken.  It is taken at
+// 3072^3 (64 against 71 us), 4608^3 (170 against 190) and 6144^3 (344 against 382), and nowhere from 5120 to 5632
+// or from 6400 on.
+static double direct_tile_time(unsigned tile, size_t tiles, size_t slabs) {
+  const double slots = tile == 128 ? 512.0 : 256.0;
+  const double slab_us = tile == 128 ? 0.95 : tile == 192 ? 1.154 : 1.5;
+  const double r = (double)tiles / slots, whole = std::floor(r), part = r - whole;
+  double rounds = whole + (part > 0.0 ? std::min(1.0, 0.55 + 0.5 * part) : 0.0);
+  if (tile == 128 && r <= 1.0) rounds = std::min(1.0, 0.25 + 0.85 * r);
+  return (tile == 128 ? 9.0 : 12.0) + rounds * (double)slabs * slab_us;
+}
+
 Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t m, size_t n, size_t k,
                         hipStream_t stream, size_t tile_m, size_t tile_n, LaunchNote* note, DType out_dtype,
                         const KernelOptions& knobs) {
@@ -326,29 +344,37 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   //                    128-tile kernel: 4.3 against 5.9 us at 128 x 128 x 64, 9.4 against 17.0 at 128 x 128 x 1024)
   // (k that is no multiple of 64: their _ktail forms, the last slab partial)
   // and the register-staged 128 x 128 kernel beyond their offset ranges (k > 2^22, more than 65535 batches).
-  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; knobs.gemm_tile = 256 | 128 and
+  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; knobs.gemm_tile = 256 | 192 | 128 and
   // knobs.gemm_direct = 0 force a kernel so that tests and searches can reach each of them at small sizes.
   {
     const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
-    unsigned tile = 128;  // (0: register-staged kernel)
-    if (k >= 512 && t256 >= 64) tile = pick_direct_tile(t256, t128);
+    const size_t t192 = ((m + 191) / 192) * ((n + 255) / 256) * bh;
+    unsigned tile = 128;  // rows of A per tile (192: against 256 rows of B; 0: register-staged kernel)
+    if (k >= 512 && t256 >= 64) {
+      tile = pick_direct_tile(t256, t128);
+      const size_t slabs = (k + 63) / 64;
+      if (1.08 * direct_tile_time(192, t192, slabs) < direct_tile_time(tile, tile == 256 ? t256 : t128, slabs)) tile = 192;
+    }
     if (tile_m == 256 && tile_n == 256) tile = 256;
-    if (tile_m == 128 && tile_n == 128 && tile == 256) tile = 128;
+    if (tile_m == 192 && tile_n == 256) tile = 192;
+    if (tile_m == 128 && tile_n == 128 && tile != 128) tile = 128;
     if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
     if (!knobs.gemm_direct) tile = 0;
     const bool ktail = k % 64 != 0;
     if (tile && k <= (size_t(1) << 22) && bh <= 65535) {
+      const unsigned across = tile == 192 ? 256 : tile;  // rows of B per tile
       p.tiles_m = (uint32_t)((m + tile - 1) / tile);
-      p.tiles_n = (uint32_t)((n + tile - 1) / tile);
+      p.tiles_n = (uint32_t)((n + across - 1) / across);
       const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
       // the 256 x 256 tile runs with four waves of 128 x 128 (knobs.gemm_waves = 8: the form with eight of 128 x 64,
-      // kept for comparison: equal on one round of tiles, 5-10 % behind on several)
-      const bool w4 = tile == 256 && knobs.gemm_waves != 8;
-      const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : "gemm_nt_bf16_128x128x64_direct") +
+      // kept for comparison: equal on one round of tiles, 5-10 % behind on several); 192 x 256 with four of 96 x 128
+      const bool w4 = tile == 192 || (tile == 256 && knobs.gemm_waves != 8);
+      const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : tile == 192 ? "gemm_nt_bf16_192x256x64_direct"
+                                                                                           : "gemm_nt_bf16_128x128x64_direct") +
                                (ktail ? "_ktail" : "") + (w4 ? "_w4" : "");
-      if (note) *note = LaunchNote{name, tile, tile};
+      if (note) *note = LaunchNote{name, tile, across};
       if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
       return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
     }
@@ -447,7 +473,7 @@ static unsigned gemm_nn_tile(size_t bh, size_t m, size_t n, size_t k, size_t til
   unsigned tile = t256 >= 128 ? pick_direct_tile(t256, t128) : 128;
   if (tile_m == 256 && tile_n == 256) tile = 256;
   if (tile_m == 128 && tile_n == 128) tile = 128;
-  if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
+  if (knobs.gemm_tile) tile = knobs.gemm_tile == 192 ? 256u : (unsigned)knobs.gemm_tile;  // (192 x 256 exists for bf16 NT products only)
   if (!knobs.gemm_direct) tile = 0;  // (no register-staged form of this product: callers transpose and use the NT kernels)
   return tile;
 }
@@ -548,7 +574,7 @@ Err launch_gemm_nt_f32(const float* a, const float* b, float* c, size_t bh, size
   // 256 x 256 tiles when they fill at least half of the CUs, 128 x 128 tiles otherwise
   const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh;
   unsigned tile = t256 >= 128 ? 256 : 128;
-  if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
+  if (knobs.gemm_tile) tile = knobs.gemm_tile == 192 ? 256u : (unsigned)knobs.gemm_tile;  // (192 x 256 exists for bf16 NT products only)
   // the k loop in parts over workgroups (gemm_nt_f32_split_k says when): partial products in the caller's temporary
   if (splits > 1) {
     if (!partial) return "gemm_nt f32 kernel: a split needs its temporary";

@@ -26,7 +26,8 @@ def golden():
 
 
 def gemm_kernel_knobs(knobs, which):
-    """`which` names one product kernel: "256" / "128" (the direct kernels' workgroup tile), "0" (register-staged)."""
+    """`which` names one product kernel: "256" / "192" (192 x 256) / "128" (the direct kernels' workgroup tile), "0"
+    (register-staged)."""
     knobs.pop("gemm.tile", None)
     knobs.pop("gemm.direct", None)
     if str(which) == "0":

@@ -526,7 +526,7 @@ def test_config4_attention_slice_vs_oracle(torch):
 
 def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
     """The i split of the attention schedule picks the workgroup size (128 or 256 query rows) and the
-    i, j splits of mm_t pick the 128 x 128 or 256 x 256 kernel; the variants agree (attention bitwise)."""
+    i, j splits of mm_t pick the 128 x 128, 192 x 256 or 256 x 256 kernel; the variants agree (attention bitwise)."""
     B, H, N, D = 1, 4, 1024, 128
     q, k, v = (torch.from_numpy(oracle.to_bf16_f32(rnd((B, H, N, D), s))).cuda().bfloat16() for s in (1, 2, 3))
     sd = torch.tensor(np.float32(1.0 / np.sqrt(D)), device="cuda")
@@ -540,6 +540,19 @@ def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
     ref = a.float() @ b.float().T
     assert (c128 - ref).abs().max() <= 1e-3 * ref.abs().max()
     assert (c256 - ref).abs().max() <= 1e-3 * ref.abs().max()
+    m192 = i("ik*jk~ijk | i:192,j:256 | jii'j'k") >> i("+ijk~ij | i:192,j:256 | jii'j'k0")
+    c192 = m192.exec_torch(a, b)
+    assert "gemm_nt_bf16_192x256x64_direct_w4" in m192.report(), m192.report()
+    assert "the schedule tile selects the kernel" in m192._code()
+    assert torch.equal(c192, c256)  # the same sums in the same order, whatever the tile
+    # the launcher's own choice: a size whose 256 x 256 tiles leave a partly empty round takes the 192 x 256 tile
+    g = torch.Generator(device="cuda").manual_seed(4)
+    a, b = ((torch.rand(3072, 1024, device="cuda", generator=g) * 2 - 1).bfloat16() for _ in range(2))
+    free = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    c = free.exec_torch(a, b)
+    assert "192x256" in free.report(), free.report()
+    ref = a.float() @ b.float().T
+    assert (c - ref).abs().max() <= 1e-5 * ref.abs().max()
 
 
 def test_few_heads_under_a_long_key_loop_split_the_keys_of_a_head_over_workgroups(torch, monkeypatch):

@@ -484,9 +484,9 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
                                       (3, 257, 255, 320)])
-@pytest.mark.parametrize("direct", ["256", "256w8", "128", "0"])
+@pytest.mark.parametrize("direct", ["256", "256w8", "192", "128", "0"])
 def test_gemm_nt_bf16_every_kernel_vs_oracle(env, knobs, bh, m, n, k, direct):
-    """The launcher picks between the 256 x 256 (four waves; "w8": the form with eight) and 128 x 128
+    """The launcher picks between the 256 x 256 (four waves; "w8": the form with eight), 192 x 256 and 128 x 128
     direct-to-LDS kernels and the register-staged kernel by problem size; force each of them on small ragged
     problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
     gemm_kernel_knobs(knobs, direct[:3])
@@ -505,10 +505,11 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, knobs, bh, m, n, k, direct):
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 8), (1, 300, 264, 40), (2, 600, 520, 136), (1, 1, 8, 200), (3, 257, 256, 1000),
                                       (1, 128, 128, 72)])
 @pytest.mark.parametrize("nn", [False, True])
-@pytest.mark.parametrize("tile", ["128", "256", "256w8"])
+@pytest.mark.parametrize("tile", ["128", "192", "256", "256w8"])
 def test_gemm_bf16_k_that_is_no_multiple_of_64(env, knobs, bh, m, n, k, nn, tile):
     """k % 8 == 0 but k % 64 != 0: the direct kernels with a partial last slab (the lanes past k clear their LDS
-    slots), both tile sizes (and both forms of the larger) forced here at small sizes; NT and NN, f32 and bf16 output."""
+    slots), every tile size (and both forms of the largest) forced here at small sizes; NT and NN (which has no
+    192 x 256 tile and takes 256 x 256 for it), f32 and bf16 output."""
     gemm_kernel_knobs(knobs, tile[:3])
     if tile.endswith("w8"):
         knobs["gemm.waves"] = 8
@@ -538,12 +539,12 @@ def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, knobs
     wait states.  Its first matrix instructions multiply zeroed operands; issued too soon after the zeroing they read
     what the registers held before, which is visible when that was NaN: products of NaN operands run first here, so
     that the register file is full of NaN, then several small multi-batch products (many short-lived workgroups)."""
-    gemm_kernel_knobs(knobs, "256")
     t = env.torch
     poison = t.full((2048, 512), float("nan"), device="cuda", dtype=t.bfloat16)
     sink = t.empty(2048, 2048, device="cuda")
     core = env.nat.core
     for rep in range(6):
+        gemm_kernel_knobs(knobs, "256" if rep % 2 == 0 else "192")  # (192 x 256: the other four-wave tile)
         env.nat.check(core.i_hip_gemm_nt_bf16(poison.data_ptr(), poison.data_ptr(), sink.data_ptr(), 1, 2048, 2048, 512, env.stream()))
         for bh, m, n, k in ((3, 677, 61, 128), (4, 512, 61, 128), (3, 677, 60, 256), (2, 300, 264, 64)):
             g = t.Generator(device="cuda").manual_seed(100 * rep + m)
@@ -560,13 +561,14 @@ def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, knobs
             assert float((cn.double() - ref[:, :, : n // 8 * 8]).abs().max()) <= 1e-2 * float(ref.abs().max()), (rep, bh, m, n, k)
 
 
-@pytest.mark.parametrize("tile", [0, 128, 256])
+@pytest.mark.parametrize("tile", [0, 128, 192, 256])
 def test_gemm_nt_bf16_output_in_bf16(env, knobs, tile):
     """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
-    result rounded to bf16, bit for bit, for the register-staged kernel (gemm.direct=0) and both tiles."""
+    result rounded to bf16, bit for bit, for the register-staged kernel (gemm.direct=0) and every tile."""
     t = env.torch
     if tile == 0:
         gemm_kernel_knobs(knobs, "0")
+    tile_n = 256 if tile == 192 else tile
     for bh, m, n, k in ((2, 300, 260, 128), (1, 512, 512, 576), (3, 1, 1, 64)):
         a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
         b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -575,15 +577,15 @@ def test_gemm_nt_bf16_output_in_bf16(env, knobs, tile):
         c16 = t.full((bh, m, n), float("nan"), device="cuda", dtype=t.bfloat16)
         core = env.nat.core
         env.nat.check(core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), c32.data_ptr(), env.nat.F32, bh, m, n, k,
-                                                  tile, tile, env.stream()))
+                                                  tile, tile_n, env.stream()))
         env.nat.check(core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), c16.data_ptr(), env.nat.BF16, bh, m, n, k,
-                                                  tile, tile, env.stream()))
+                                                  tile, tile_n, env.stream()))
         t.cuda.synchronize()
         assert t.equal(c16, c32.bfloat16())
         assert_close(c32.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
-@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("tile", [128, 192, 256])
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
     """The direct kernels store four columns per lane when C allows it; a C that starts one element past a
@@ -597,8 +599,8 @@ def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
     cd = whole[1:-1]
     assert cd.data_ptr() % 16 != 0
     env.nat.check(env.nat.core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(),
-                                                      env.nat.BF16 if out_bf16 else env.nat.F32, bh, m, n, k, tile, tile,
-                                                      env.stream()))
+                                                      env.nat.BF16 if out_bf16 else env.nat.F32, bh, m, n, k, tile,
+                                                      256 if tile == 192 else tile, env.stream()))
     t.cuda.synchronize()
     assert whole[0].item() == -7.0 and whole[-1].item() == -7.0
     ref = oracle.mm_t(a, b)

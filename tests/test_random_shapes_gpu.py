@@ -71,7 +71,7 @@ def test_gemm_bf16_random_shapes(env, knobs, seed):
         k = rng.choice([64, 128, 192, 320, 512, 1024]) if (nn or rng.random() < 0.7) else 8 * rng.randint(1, 60)
         if nn:
             n = max(8, n // 8 * 8)
-        direct = rng.choice([None, "256", "128"] + ([] if nn else ["0"]))
+        direct = rng.choice([None, "256", "128"] + ([] if nn else ["0", "192"]))
         if direct:
             gemm_kernel_knobs(knobs, direct)
         else:
