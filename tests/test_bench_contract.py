@@ -49,12 +49,21 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert cpu["kind"] == "port" and cpu["form"].startswith("emitted-c") and cpu["cores"] == 1 and cpu["value"] > 0 and cpu["sample"] and cpu["host_cpu"]
     assert rec["pre_warmup_launches"] == 41 and rec["rel_err"] <= 2e-2
     assert rec["roofline"]["kernel"] == "attn_fwd_bf16_d128_bn64_direct_w8"
+    # the clock the kernel counted for itself, and the committed profile's cycles at that clock against the measured time
+    assert 1.0 < roof["shader_clock_ghz"] < 2.6
+    assert abs(roof["frac_at_measured_clock"] - roof["frac"] * 2.4 / roof["shader_clock_ghz"]) < 1e-9
+    assert 0.85 < roof["kernel_ms_measured_over_predicted"] < 1.2
+    assert rec["library_gemm_probe"] is None  # (timed from 20 steps on)
     second = rec["secondary"]
-    assert len(second) == 7
-    one_head = second[6]  # (one head on its own: its keys in parts over workgroups, beside the same call unsplit)
+    assert len(second) == 8
+    host = second[6]  # (the host entry point: PCIe-inclusive, never the headline)
+    assert "i_exec_into" in host["workload"] and host["pcie_GBps"] > 0 and host["rel_err_against_f64"] <= 1e-4
+    one_head = second[7]  # (one head on its own: its keys in parts over workgroups, beside the same call unsplit)
     assert "(keys in " in one_head["launches"] and one_head["ms_per_call_unsplit"] > 0 and one_head["rel_err_against_unsplit"] <= 2e-3
     for entry, bar in zip(second, (1e-4, 1e-4, 2e-2, 2e-2, 1e-4, 1e-4)):
         assert entry["cpu_baseline"]["value"] > 0 and entry["rel_err"] <= bar, entry["workload"]
+    c5 = second[3]
+    assert c5["second_bound"]["binds"] in ("mfma", "valu") and 0.5 < c5["second_bound"]["frac_of_sum_of_bounds_at_measured_clock"] < 1.3
     f32_line = second[5]
     assert f32_line["dtype"] == "f32" and f32_line["roofline"]["peak"] == 157.3
     assert f32_line["roofline"]["kernel"] == "attn_fwd_f32_d128_bn32_direct"

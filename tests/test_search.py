@@ -29,7 +29,7 @@ def test_option_grid_enumerates_program_options():
                         ("attention.waves", 64), ("attention.direct", 0), ("attention.f32_scale", 1), ("generated.only", 1),
                         ("generated.wave", -1)):
         comp.option(name, value)
-    for name, value, text in (("gemm.kparts", 2, "unknown program option"), ("gemm.tile", 64, "0, 128 or 256"),
+    for name, value, text in (("gemm.kparts", 2, "unknown program option"), ("gemm.tile", 64, "0, 128, 192 .192 x 256. or 256"),
                               ("attention.waves", 3, "attention.waves"), ("gemm.k_parts", -1, "gemm.k_parts")):
         with pytest.raises(RuntimeError, match=text):
             comp.option(name, value)
