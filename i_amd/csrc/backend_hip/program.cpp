@@ -925,11 +925,11 @@ std::string program_code(const Component& component) {
       const bool attn = rec[k].kind == Recognized::Attention;
       const bool known = attn ? (((ti == 64 || ti == 128 || ti == 256) && (tj == 32 || tj == 64)) || (ti == 512 && tj == 32))
                               : ((ti == 128 && tj == 128) || (ti == 256 && tj == 256) ||
-                                 (ti == 192 && tj == 256 && rec[k].kind == Recognized::GemmNT));
+                                 (ti + tj == 448 && (ti == 192 || ti == 256) && rec[k].kind == Recognized::GemmNT));
       os << "\n//     " << (known ? "the schedule tile selects the kernel with that workgroup tile where the operands allow it"
                                    : "no hand-written kernel has this tile: the launcher picks one by problem size")
          << (attn ? " (attention tiles: 64 / 128 / 256 query rows x 32 / 64 keys, 512 x 32 at d = 64)"
-                  : " (GEMM tiles: 128 x 128, 256 x 256; 192 x 256 for a K-contiguous right operand)")
+                  : " (GEMM tiles: 128 x 128, 256 x 256; 192 x 256 and 256 x 192 for a K-contiguous right operand)")
          << "; i_hip_program_report names the kernel that ran";
     }
     os << "\n//     reads";

@@ -8,8 +8,8 @@
 // 16x16x32 MFMAs per second than 32x32x16 ones under its power limit, at the same operand traffic from LDS.
 //
 //   workgroup   WM x WN waves on a BTM x BTN tile of C (BTM rows of A against BTN rows of B; square but for the
-//               192 x 256 form, which is one full round of workgroups where 256 x 256 tiles leave a partly empty
-//               one: 3072^3, 6144^3); a wave owns (BTM / WM) x (BTN / WN) of the tile as TM x TN accumulators of
+//               192 x 256 and 256 x 192 forms, which are one full round of workgroups where 256 x 256 tiles leave a
+//               partly empty one: 3072^3, 6144^3); a wave owns (BTM / WM) x (BTN / WN) of the tile as TM x TN accumulators of
 //               16 x 16 (256 x 256 with 2 x 4 waves: 8 x 4 accumulators, 128 registers; with 2 x 2 waves, one per
 //               SIMD: 8 x 8 accumulators, the 256 registers of the accumulation file, a third fewer operand
 //               reads per matrix instruction; that form's matrix instructions are inline assembly, see kstep)
@@ -187,7 +187,7 @@ __device__ __forceinline__ void gemm_nt_mfma16_tile(const GemmParams& p, char* s
   const uint32_t jj = (lane >> 2) & 3, qq = lane & 3;
   // (fragment j of the wave is unit wn TN + j = (wn TN) ^ j of the row, TN being a power of two that j stays below:
   // the fragment's address is the first one's with 32 j XOR-ed in, one instruction instead of TN registers)
-  static_assert((TN & (TN - 1)) == 0, "fragments per wave");
+  static_assert(!NN || (TN & (TN - 1)) == 0, "fragments per wave");
   const uint32_t baddr0 = NN ? (8 * g + jj) * RBN + 32 * ((uint32_t)(wn * TN) ^ (jj | ((g & 1) << 2))) + 8 * qq : 0u;
 
   f32x4 acc[TM][TN];

@@ -126,6 +126,13 @@ extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_192x256x64_dir
 extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_192x256x64_direct_ktail_w4(GemmParams p) {
   gemm_nt_mfma16_body<192, 2, 2, false, true, 256>(p);
 }
+// ... and 256 rows of A against 192 rows of B (four waves of 128 x 96), for the same sizes when it is n that 256 cuts badly
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x192x64_direct_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2, false, false, 192>(p);
+}
+extern "C" __global__ void __launch_bounds__(256, 1) gemm_nt_bf16_256x192x64_direct_ktail_w4(GemmParams p) {
+  gemm_nt_mfma16_body<256, 2, 2, false, true, 192>(p);
+}
 extern "C" __global__ void __launch_bounds__(256, 1) gemm_nn_bf16_256x256x64_direct_w4(GemmParams p) {
   gemm_nt_mfma16_body<256, 2, 2, true>(p);
 }

@@ -42,6 +42,9 @@ Err set_kernel_option(KernelOptions& o, const std::string& name, int value) {
   } else if (name == "gemm.tile") {
     if (!one_of({0, 128, 192, 256})) return bad("0, 128, 192 (192 x 256) or 256");
     o.gemm_tile = value;
+  } else if (name == "gemm.tile_n") {
+    if (!one_of({0, 128, 192, 256})) return bad("0 (what goes with gemm.tile), 128, 192 (256 x 192) or 256");
+    o.gemm_tile_n = value;
   } else if (name == "gemm.direct") {
     o.gemm_direct = value != 0;
   } else if (name == "generated.only") {
@@ -55,7 +58,7 @@ Err set_kernel_option(KernelOptions& o, const std::string& name, int value) {
   } else {
     return "unknown program option '" + name +
            "' (known: attention.f32_scale, attention.kv_parts, attention.waves, attention.direct, gemm.k_parts, gemm.waves, "
-           "gemm.tile, gemm.direct, generated.only, generated.wave, generated.parts)";
+           "gemm.tile, gemm.tile_n, gemm.direct, generated.only, generated.wave, generated.parts)";
   }
   return {};
 }
@@ -344,39 +347,46 @@ Err launch_gemm_nt_bf16(const void* a, const void* b, void* c, size_t bh, size_t
   //                    128-tile kernel: 4.3 against 5.9 us at 128 x 128 x 64, 9.4 against 17.0 at 128 x 128 x 1024)
   // (k that is no multiple of 64: their _ktail forms, the last slab partial)
   // and the register-staged 128 x 128 kernel beyond their offset ranges (k > 2^22, more than 65535 batches).
-  // The schedule's i, j splits (256 x 256 or 128 x 128) decide when given; knobs.gemm_tile = 256 | 192 | 128 and
+  // The schedule's i, j splits (256 x 256, 192 x 256, 256 x 192 or 128 x 128) decide when given; knobs.gemm_tile
+  // = 256 | 192 | 128 (with knobs.gemm_tile_n = 192 for 256 x 192) and
   // knobs.gemm_direct = 0 force a kernel so that tests and searches can reach each of them at small sizes.
   {
     const size_t t256 = ((m + 255) / 256) * ((n + 255) / 256) * bh, t128 = ((m + 127) / 128) * ((n + 127) / 128) * bh;
-    const size_t t192 = ((m + 191) / 192) * ((n + 255) / 256) * bh;
-    unsigned tile = 128;  // rows of A per tile (192: against 256 rows of B; 0: register-staged kernel)
+    // the two rectangular tiles: 192 rows of A against 256 of B, or 256 against 192, whichever leaves fewer tiles
+    const size_t t192m = ((m + 191) / 192) * ((n + 255) / 256) * bh, t192n = ((m + 255) / 256) * ((n + 191) / 192) * bh;
+    unsigned tile = 128, across = 0;  // rows of A and of B per tile (across 0: as many as of A; tile 0: register-staged kernel)
     if (k >= 512 && t256 >= 64) {
       tile = pick_direct_tile(t256, t128);
       const size_t slabs = (k + 63) / 64;
-      if (1.08 * direct_tile_time(192, t192, slabs) < direct_tile_time(tile, tile == 256 ? t256 : t128, slabs)) tile = 192;
+      if (1.08 * direct_tile_time(192, std::min(t192m, t192n), slabs) < direct_tile_time(tile, tile == 256 ? t256 : t128, slabs)) {
+        tile = t192m <= t192n ? 192 : 256;
+        across = t192m <= t192n ? 256 : 192;
+      }
     }
-    if (tile_m == 256 && tile_n == 256) tile = 256;
-    if (tile_m == 192 && tile_n == 256) tile = 192;
-    if (tile_m == 128 && tile_n == 128 && tile != 128) tile = 128;
-    if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile;
+    if (tile_m == 128 && tile_n == 128) tile = 128, across = 0;
+    if ((tile_m == 256 || tile_m == 192) && (tile_n == 256 || tile_n == 192) && tile_m + tile_n >= 448) tile = (unsigned)tile_m, across = (unsigned)tile_n;
+    if (knobs.gemm_tile) tile = (unsigned)knobs.gemm_tile, across = (unsigned)knobs.gemm_tile_n;
+    if (!across) across = tile == 192 ? 256 : tile;
+    if (tile == 192 && across != 256) return "gemm_nt kernel: a 192-row tile goes with 256 columns";
+    if (tile == 128 && across != 128) return "gemm_nt kernel: a 128-row tile goes with 128 columns";
+    if (tile == 256 && across != 256 && across != 192) return "gemm_nt kernel: a 256-row tile goes with 256 or 192 columns";
     if (!knobs.gemm_direct) tile = 0;
     const bool ktail = k % 64 != 0;
     if (tile && k <= (size_t(1) << 22) && bh <= 65535) {
-      const unsigned across = tile == 192 ? 256 : tile;  // rows of B per tile
       p.tiles_m = (uint32_t)((m + tile - 1) / tile);
       p.tiles_n = (uint32_t)((n + across - 1) / across);
       const size_t grid = (size_t(p.tiles_m) * p.tiles_n + 7) / 8 * 8;  // the tiles in 8 equal runs, one per XCD
       if (grid > kMaxGrid) return "gemm_nt kernel: grid too large";
       hipFunction_t fn;
       // the 256 x 256 tile runs with four waves of 128 x 128 (knobs.gemm_waves = 8: the form with eight of 128 x 64,
-      // kept for comparison: equal on one round of tiles, 5-10 % behind on several); 192 x 256 with four of 96 x 128
-      const bool w4 = tile == 192 || (tile == 256 && knobs.gemm_waves != 8);
-      const std::string name = std::string(tile == 256 ? "gemm_nt_bf16_256x256x64_direct" : tile == 192 ? "gemm_nt_bf16_192x256x64_direct"
-                                                                                           : "gemm_nt_bf16_128x128x64_direct") +
+      // kept for comparison: equal on one round of tiles, 5-10 % behind on several); the rectangular ones with four
+      // of 96 x 128 or 128 x 96
+      const bool w4 = tile + across == 448 || (tile == 256 && knobs.gemm_waves != 8);
+      const std::string name = "gemm_nt_bf16_" + std::to_string(tile) + "x" + std::to_string(across) + "x64_direct" +
                                (ktail ? "_ktail" : "") + (w4 ? "_w4" : "");
       if (note) *note = LaunchNote{name, tile, across};
       if (Err e = builtin_function(name.c_str(), &fn); !e.empty()) return e;
-      return launch(fn, (unsigned)grid, (unsigned)bh, 1, tile == 256 && !w4 ? 512 : 256, &p, sizeof(p), stream);
+      return launch(fn, (unsigned)grid, (unsigned)bh, 1, w4 || tile == 128 ? 256 : 512, &p, sizeof(p), stream);
     }
   }
   p.tiles_m = (uint32_t)((m + 127) / 128);

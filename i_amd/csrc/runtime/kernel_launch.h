@@ -28,7 +28,8 @@ struct KernelOptions {
   int attention_direct = 1;     // 0: the register-staged kernels instead of the direct-to-LDS ones
   int gemm_k_parts = 0;         // k loop of a product in parts over workgroups: 0 the launcher decides, 1 never, n that many
   int gemm_waves = 0;           // waves of the 256 x 256 tile: 0 decides (four), 4, 8
-  int gemm_tile = 0;            // workgroup tile of the direct kernels: 0 decides, 128, 256
+  int gemm_tile = 0;            // workgroup tile of the direct kernels, rows of A: 0 decides, 128, 192 (x 256), 256
+  int gemm_tile_n = 0;          // ... rows of B: 0 what goes with gemm_tile, 192 with gemm_tile 256 for 256 x 192
   int gemm_direct = 1;          // 0: the register-staged bf16 kernel instead of the direct-to-LDS ones
   int generated_only = 0;       // 1: every kernel of a program in its generated form
   int generated_wave = -1;      // wavefront-per-iteration form of generated reduction nests: -1 decides, 0 never, 1 wherever a nest has one

@@ -137,6 +137,8 @@ int i_hip_attention_opt(const void* q, const void* k, const void* v, void* o,
  *   "gemm.k_parts"         k loop of a product in parts over workgroups: 0 (default) by a model of the time, 1 never, n
  *   "gemm.tile"            workgroup tile of the direct product kernels: 0 (default) by schedule tile and size, 128, 256,
  *                          192 (192 x 256: bf16 products with a K-contiguous right operand; the others take 256)
+ *   "gemm.tile_n"          columns of that tile when gemm.tile is given: 0 (default) what goes with it, 192 with
+ *                          gemm.tile = 256 for the 256 x 192 tile (same products as 192 x 256)
  *   "gemm.waves"           waves of the 256 x 256 tile: 0 (default: four), 4, 8
  *   "gemm.direct"          1 (default) / 0: the register-staged bf16 product kernel
  *   "generated.only"       0 (default) / 1: every kernel in its generated form (no hand-written kernel)

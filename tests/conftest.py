@@ -26,12 +26,16 @@ def golden():
 
 
 def gemm_kernel_knobs(knobs, which):
-    """`which` names one product kernel: "256" / "192" (192 x 256) / "128" (the direct kernels' workgroup tile), "0"
-    (register-staged)."""
-    knobs.pop("gemm.tile", None)
-    knobs.pop("gemm.direct", None)
-    if str(which) == "0":
+    """`which` names one product kernel: "256" / "192" (192 x 256) / "256x192" / "128" (the direct kernels' workgroup
+    tile; a trailing "w8" is not part of the name), "0" (register-staged)."""
+    which = str(which)
+    which = which[:-2] if which.endswith("w8") else which
+    for name in ("gemm.tile", "gemm.tile_n", "gemm.direct"):
+        knobs.pop(name, None)
+    if which == "0":
         knobs["gemm.direct"] = 0
+    elif "x" in which:
+        knobs["gemm.tile"], knobs["gemm.tile_n"] = (int(v) for v in which.split("x"))
     else:
         knobs["gemm.tile"] = int(which)
 

@@ -545,6 +545,8 @@ def test_schedule_tiles_select_kernel_variants_with_equal_results(torch):
     assert "gemm_nt_bf16_192x256x64_direct_w4" in m192.report(), m192.report()
     assert "the schedule tile selects the kernel" in m192._code()
     assert torch.equal(c192, c256)  # the same sums in the same order, whatever the tile
+    m256x192 = i("ik*jk~ijk | i:256,j:192 | jii'j'k") >> i("+ijk~ij | i:256,j:192 | jii'j'k0")
+    assert torch.equal(m256x192.exec_torch(a, b), c256) and "gemm_nt_bf16_256x192x64_direct_w4" in m256x192.report()
     # the launcher's own choice: a size whose 256 x 256 tiles leave a partly empty round takes the 192 x 256 tile
     g = torch.Generator(device="cuda").manual_seed(4)
     a, b = ((torch.rand(3072, 1024, device="cuda", generator=g) * 2 - 1).bfloat16() for _ in range(2))

@@ -484,12 +484,12 @@ def test_gemm_nt_bf16_vs_oracle(env, bh, m, n, k):
 
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 64), (1, 300, 260, 128), (2, 600, 520, 192), (1, 1, 1, 256),
                                       (3, 257, 255, 320)])
-@pytest.mark.parametrize("direct", ["256", "256w8", "192", "128", "0"])
+@pytest.mark.parametrize("direct", ["256", "256w8", "192", "256x192", "128", "0"])
 def test_gemm_nt_bf16_every_kernel_vs_oracle(env, knobs, bh, m, n, k, direct):
     """The launcher picks between the 256 x 256 (four waves; "w8": the form with eight), 192 x 256 and 128 x 128
     direct-to-LDS kernels and the register-staged kernel by problem size; force each of them on small ragged
     problems with 1 to 5 k-slabs, edge tiles on both axes and several batches."""
-    gemm_kernel_knobs(knobs, direct[:3])
+    gemm_kernel_knobs(knobs, direct)
     if direct.endswith("w8"):
         knobs["gemm.waves"] = 8
     t = env.torch
@@ -505,12 +505,12 @@ def test_gemm_nt_bf16_every_kernel_vs_oracle(env, knobs, bh, m, n, k, direct):
 @pytest.mark.parametrize("bh,m,n,k", [(1, 256, 256, 8), (1, 300, 264, 40), (2, 600, 520, 136), (1, 1, 8, 200), (3, 257, 256, 1000),
                                       (1, 128, 128, 72)])
 @pytest.mark.parametrize("nn", [False, True])
-@pytest.mark.parametrize("tile", ["128", "192", "256", "256w8"])
+@pytest.mark.parametrize("tile", ["128", "192", "256x192", "256", "256w8"])
 def test_gemm_bf16_k_that_is_no_multiple_of_64(env, knobs, bh, m, n, k, nn, tile):
     """k % 8 == 0 but k % 64 != 0: the direct kernels with a partial last slab (the lanes past k clear their LDS
     slots), every tile size (and both forms of the largest) forced here at small sizes; NT and NN (which has no
     192 x 256 tile and takes 256 x 256 for it), f32 and bf16 output."""
-    gemm_kernel_knobs(knobs, tile[:3])
+    gemm_kernel_knobs(knobs, tile)
     if tile.endswith("w8"):
         knobs["gemm.waves"] = 8
     t = env.torch
@@ -544,7 +544,7 @@ def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, knobs
     sink = t.empty(2048, 2048, device="cuda")
     core = env.nat.core
     for rep in range(6):
-        gemm_kernel_knobs(knobs, "256" if rep % 2 == 0 else "192")  # (192 x 256: the other four-wave tile)
+        gemm_kernel_knobs(knobs, ("256", "192", "256x192")[rep % 3])  # (the three four-wave tiles)
         env.nat.check(core.i_hip_gemm_nt_bf16(poison.data_ptr(), poison.data_ptr(), sink.data_ptr(), 1, 2048, 2048, 512, env.stream()))
         for bh, m, n, k in ((3, 677, 61, 128), (4, 512, 61, 128), (3, 677, 60, 256), (2, 300, 264, 64)):
             g = t.Generator(device="cuda").manual_seed(100 * rep + m)
@@ -561,14 +561,14 @@ def test_gemm_four_wave_form_does_not_read_what_registers_held_before(env, knobs
             assert float((cn.double() - ref[:, :, : n // 8 * 8]).abs().max()) <= 1e-2 * float(ref.abs().max()), (rep, bh, m, n, k)
 
 
-@pytest.mark.parametrize("tile", [0, 128, 192, 256])
+@pytest.mark.parametrize("tile", [0, 128, 192, 256, (256, 192)])
 def test_gemm_nt_bf16_output_in_bf16(env, knobs, tile):
     """bf16 output: the kernels round their f32 sums to nearest-even on the way out, so the result equals the f32
     result rounded to bf16, bit for bit, for the register-staged kernel (gemm.direct=0) and every tile."""
     t = env.torch
     if tile == 0:
         gemm_kernel_knobs(knobs, "0")
-    tile_n = 256 if tile == 192 else tile
+    tile, tile_n = tile if isinstance(tile, tuple) else (tile, 256 if tile == 192 else tile)
     for bh, m, n, k in ((2, 300, 260, 128), (1, 512, 512, 576), (3, 1, 1, 64)):
         a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
         b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
@@ -585,13 +585,14 @@ def test_gemm_nt_bf16_output_in_bf16(env, knobs, tile):
         assert_close(c32.cpu().numpy(), oracle.mm_t(a, b), RTOL_BF16)
 
 
-@pytest.mark.parametrize("tile", [128, 192, 256])
+@pytest.mark.parametrize("tile", [128, 192, 256, (256, 192)])
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
     """The direct kernels store four columns per lane when C allows it; a C that starts one element past a
     16-byte boundary takes the element-wise stores instead.  The elements before and after C stay untouched."""
     t = env.torch
     bh, m, n, k = 2, 300, 260, 128
+    tile, tile_n = tile if isinstance(tile, tuple) else (tile, 256 if tile == 192 else tile)
     a = oracle.to_bf16_f32(rnd((bh, m, k), 1, "uniform"))
     b = oracle.to_bf16_f32(rnd((bh, n, k), 2, "uniform"))
     ad, bd = t.from_numpy(a).cuda().bfloat16(), t.from_numpy(b).cuda().bfloat16()
@@ -600,7 +601,7 @@ def test_gemm_nt_bf16_output_not_16_byte_aligned(env, out_bf16, tile):
     assert cd.data_ptr() % 16 != 0
     env.nat.check(env.nat.core.i_hip_gemm_nt_bf16_ex(ad.data_ptr(), bd.data_ptr(), cd.data_ptr(),
                                                       env.nat.BF16 if out_bf16 else env.nat.F32, bh, m, n, k, tile,
-                                                      256 if tile == 192 else tile, env.stream()))
+                                                      tile_n, env.stream()))
     t.cuda.synchronize()
     assert whole[0].item() == -7.0 and whole[-1].item() == -7.0
     ref = oracle.mm_t(a, b)

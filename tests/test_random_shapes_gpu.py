@@ -71,11 +71,11 @@ def test_gemm_bf16_random_shapes(env, knobs, seed):
         k = rng.choice([64, 128, 192, 320, 512, 1024]) if (nn or rng.random() < 0.7) else 8 * rng.randint(1, 60)
         if nn:
             n = max(8, n // 8 * 8)
-        direct = rng.choice([None, "256", "128"] + ([] if nn else ["0", "192"]))
+        direct = rng.choice([None, "256", "128"] + ([] if nn else ["0", "192", "256x192"]))
         if direct:
             gemm_kernel_knobs(knobs, direct)
         else:
-            knobs.pop("gemm.tile", None); knobs.pop("gemm.direct", None)
+            knobs.pop("gemm.tile", None); knobs.pop("gemm.tile_n", None); knobs.pop("gemm.direct", None)
         g = t.Generator(device="cuda").manual_seed(1000 * seed + case)
         a = (t.rand(bh, m, k, device="cuda", generator=g) * 2 - 1).bfloat16()
         b = (t.rand(*((bh, k, n) if nn else (bh, n, k)), device="cuda", generator=g) * 2 - 1).bfloat16()
