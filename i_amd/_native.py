@@ -55,6 +55,8 @@ core.i_hip_program_option.argtypes = [vp, ctypes.c_char_p, ctypes.c_int]
 core.i_hip_program_option.restype = ctypes.c_int
 core.i_hip_program_report.argtypes = [vp]
 core.i_hip_program_report.restype = vp
+core.i_hip_program_row_slices.argtypes = [vp, ctypes.POINTER(ctypes.c_ubyte), ctypes.c_size_t]
+core.i_hip_program_row_slices.restype = ctypes.c_int
 core.i_hip_gemm_nt_bf16.argtypes = [vp, vp, vp, sz, sz, sz, sz, vp]
 core.i_hip_gemm_nt_bf16.restype = ctypes.c_int
 core.i_hip_gemm_nt_bf16_ex.argtypes = [vp, vp, vp, ctypes.c_int, sz, sz, sz, sz, sz, sz, vp]

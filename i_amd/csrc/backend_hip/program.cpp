@@ -868,6 +868,68 @@ std::vector<std::vector<std::pair<size_t, size_t>>> tied_extents(const Graph<Nod
   return {groups.begin(), groups.end()};
 }
 
+// See row_sliceable() in the header.  The dimension sets are those of tied_extents above, kept per symbol of every
+// node: a symbol stands for the (input, dimension) pairs of the operand dimensions it indexes, and a result
+// dimension for those of its output symbol.
+bool row_slices_of(const Graph<Node>& graph, std::vector<char>* sliced) {
+  using Dims = std::set<std::pair<size_t, size_t>>;
+  std::vector<std::vector<Dims>> result_dims(graph.nodes.size()), symbol_dims(graph.nodes.size());
+  std::vector<char> state(graph.nodes.size(), 0);
+  std::function<void(size_t)> visit = [&](size_t n) {
+    if (state[n] != 0) return;
+    state[n] = 1;
+    const GNode<Node>& g = graph.nodes[n];
+    const Node& node = g.inner;
+    std::vector<Dims>& of_symbol = symbol_dims[n];
+    of_symbol.assign(node.rank, {});
+    for (size_t o = 0; o < node.inputs.size() && o < g.inputs.size(); ++o) {
+      const Source& src = g.inputs[o];
+      if (!src.is_input && src.id < graph.nodes.size()) visit(src.id);
+      for (size_t pos = 0; pos < node.inputs[o].size(); ++pos) {
+        const size_t symbol = node.inputs[o][pos];
+        if (symbol >= of_symbol.size()) continue;
+        if (src.is_input) of_symbol[symbol].insert({src.id, pos});
+        else if (src.id < graph.nodes.size() && pos < result_dims[src.id].size())
+          of_symbol[symbol].insert(result_dims[src.id][pos].begin(), result_dims[src.id][pos].end());
+      }
+    }
+    for (size_t symbol : node.output) result_dims[n].push_back(symbol < of_symbol.size() ? of_symbol[symbol] : Dims{});
+    state[n] = 2;
+  };
+  for (size_t n = 0; n < graph.nodes.size(); ++n) visit(n);
+  // the leading index: the same for every output, and first dimensions of inputs only
+  Dims leading;
+  if (graph.outputs.empty()) return false;
+  for (size_t o = 0; o < graph.outputs.size(); ++o) {
+    const Source& out = graph.outputs[o];
+    if (out.is_input || out.id >= graph.nodes.size() || result_dims[out.id].empty()) return false;
+    if (o == 0) leading = result_dims[out.id][0];
+    else if (result_dims[out.id][0] != leading) return false;
+  }
+  if (leading.empty()) return false;
+  for (const auto& [input, pos] : leading)
+    if (pos != 0 || input >= graph.inputs) return false;
+  auto tied = [&](const Dims& d) {
+    for (const auto& pair : d)
+      if (leading.count(pair)) return true;
+    return false;
+  };
+  // no expression reduces over it, none has it under two names
+  for (size_t n = 0; n < graph.nodes.size(); ++n) {
+    const Node& node = graph.nodes[n].inner;
+    size_t names = 0;
+    for (size_t symbol = 0; symbol < symbol_dims[n].size(); ++symbol) {
+      if (!tied(symbol_dims[n][symbol])) continue;
+      ++names;
+      if (std::find(node.output.begin(), node.output.end(), symbol) == node.output.end()) return false;
+    }
+    if (names > 1) return false;
+  }
+  sliced->assign(graph.inputs, 0);
+  for (const auto& pair : leading) (*sliced)[pair.first] = 1;
+  return true;
+}
+
 }  // namespace
 
 Program::~Program() {
@@ -880,6 +942,7 @@ std::string compile_program(const Component& component, Program** out) {
   p->module = lower_exec_plan_to_module(p->low.plan);
   p->recognized = recognize_kernels(p->low);
   p->same_extent = tied_extents(p->low.graph);
+  p->row_sliceable = row_slices_of(p->low.graph, &p->row_sliced);
   if (p->recognized.size() != p->low.plan.kernels.size()) lower_error("kernel recognition lost track of the kernel list");
   // the generated form: one kernel per loop nest
   std::vector<size_t> origin;
@@ -967,6 +1030,11 @@ std::string program_code(const Component& component) {
   }
   os << "\n" << gen.source;
   return os.str();
+}
+
+bool row_sliceable(const Program& p, std::vector<char>* sliced) {
+  if (p.row_sliceable && sliced) *sliced = p.row_sliced;
+  return p.row_sliceable;
 }
 
 size_t output_count(const Program& p) { return p.low.plan.count; }
@@ -1122,6 +1190,11 @@ std::string set_clock_probe(Program& p, void* ticks) {
   std::lock_guard<std::mutex> lock(p.mu);
   p.options.clock_ticks = static_cast<unsigned long long*>(ticks);
   return {};
+}
+
+void append_to_report(Program& p, const std::string& line) {
+  std::lock_guard<std::mutex> lock(p.mu);
+  p.last_report += line;
 }
 
 std::string last_report(Program& p) {

@@ -35,6 +35,10 @@ struct Program {
   // Groups of (input, dimension) pairs that one index symbol ties together, directly or through intermediate
   // results: their extents must agree, or some kernel would index an operand out of bounds.
   std::vector<std::vector<std::pair<size_t, size_t>>> same_extent;
+  // Whether the program can be run on its leading index in slices (row_slices_of); sliced[i]: input i is cut along
+  // its first dimension with the outputs, the other inputs are needed whole by every slice.
+  bool row_sliceable = false;
+  std::vector<char> row_sliced;
   // The generated form of the plan: every kernel cut into one kernel per loop nest (split_nests), the statement IR
   // of those, and for each kernel of low.plan the kernels of nest_plan that stand for it, in order.
   ic::ExecPlan nest_plan;
@@ -67,6 +71,13 @@ std::string output_shapes(const Program& p, const std::vector<std::vector<size_t
                           std::vector<std::vector<size_t>>* shapes);
 size_t input_count(const Program& p);
 size_t input_rank(const Program& p, size_t input);
+// Whether every output's first dimension is an index that the program only ever maps over: one that stands for the
+// first dimension of some inputs (`sliced`, one flag per input) and for no other dimension of any input, that no
+// expression sums (or otherwise reduces) over, and that no expression uses twice under different names.  Rows
+// r0 .. r1 of the outputs are then what the program computes from rows r0 .. r1 of the sliced inputs and all of
+// the others, so a caller may run it slice by slice (the host entry points do, to have the kernels of one slice
+// run while the next is on its way to the device).
+bool row_sliceable(const Program& p, std::vector<char>* sliced);
 
 // Caller-provided device memory for a program's temporaries (intermediates of multi-kernel plans, dtype
 // staging, transposed operands, per-work-item slices of generated kernels).  `used` counts what one
@@ -94,6 +105,8 @@ std::string set_option(Program& p, const std::string& name, int value);
 std::string set_clock_probe(Program& p, void* ticks);
 // The kernels the last execute() of this program dispatched, one per line.
 std::string last_report(Program& p);
+// One more line for that report (the host entry points note a call that ran in slices).
+void append_to_report(Program& p, const std::string& line);
 
 // What execute() with a workspace would take from it for these operands, in bytes.  Launches nothing.
 std::string workspace_bytes(Program& p, const std::vector<DeviceTensor>& inputs, const std::vector<DeviceTensor>& outputs,

@@ -135,6 +135,112 @@ size_t staging_limit() {
   return limit;
 }
 
+// The stream that the operands of a call in slices are uploaded on (one per device, created on first use and kept;
+// not synchronised with the default stream, on which the kernels run); nullptr when there is none to be had.
+hipStream_t upload_stream_of_current_device() {
+  static std::mutex mu;
+  static std::map<int, hipStream_t>* streams = new std::map<int, hipStream_t>();
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = streams->find(device);
+  if (it != streams->end()) return it->second;
+  hipStream_t made = nullptr;
+  if (hipStreamCreateWithFlags(&made, hipStreamNonBlocking) != hipSuccess) {
+    (void)hipGetLastError();
+    made = nullptr;
+  }
+  (*streams)[device] = made;
+  return made;
+}
+
+// A call in slices (large operands of a program that only maps over its leading index, ihipc::row_sliceable): the
+// inputs that every slice needs whole are uploaded first; then, slice after slice, the rows of the other inputs go
+// up on the upload stream and the program is enqueued on `stream` behind them for just those rows, so the kernels
+// of one slice run while the next is on the link; the outputs come down when the last slice has run.  Returns
+// false when the call is not taken in slices (nothing has been enqueued then).
+constexpr size_t kSlicedCallBytes = size_t(64) << 20;  // what crosses the link in slices, at least
+constexpr size_t kSliceBytes = size_t(32) << 20;       // ... and per slice, about
+bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::vector<ihipc::DeviceTensor>& in,
+                        const std::vector<ihipc::DeviceTensor>& out, hipStream_t stream, std::string* err) {
+  std::vector<char> sliced;
+  if (!ihipc::row_sliceable(p, &sliced) || sliced.size() != in.size() || out.empty() || out[0].shape.empty()) return false;
+  const size_t rows = out[0].shape[0];
+  auto row_bytes = [](const ihipc::DeviceTensor& t) {
+    size_t n = 4;
+    for (size_t d = 1; d < t.shape.size(); ++d) n *= t.shape[d];
+    return n;
+  };
+  size_t moving = 0, whole = 0;
+  for (size_t i = 0; i < in.size(); ++i) {
+    if (sliced[i] && (in[i].shape.empty() || in[i].shape[0] != rows)) return false;
+    (sliced[i] ? moving : whole) += row_bytes(in[i]) * (in[i].shape.empty() ? 1 : in[i].shape[0]);
+  }
+  for (const ihipc::DeviceTensor& t : out) {
+    if (t.shape.empty() || t.shape[0] != rows) return false;
+    moving += row_bytes(t) * rows;
+  }
+  if (rows < 2 || moving < kSlicedCallBytes || moving < whole) return false;
+  const size_t slices = std::min<size_t>(std::min<size_t>(8, rows), std::max<size_t>(2, moving / kSliceBytes));
+  const size_t each = (rows + slices - 1) / slices;
+  hipStream_t up = upload_stream_of_current_device();
+  if (!up) return false;
+  std::vector<hipEvent_t> landed(slices, nullptr);
+  for (hipEvent_t& e : landed)
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      for (hipEvent_t made : landed)
+        if (made) (void)hipEventDestroy(made);
+      return false;
+    }
+  auto fail = [&](const std::string& what) {
+    *err = what;
+    (void)hipStreamSynchronize(up);
+    (void)ihip::sync(stream);
+    for (hipEvent_t e : landed) (void)hipEventDestroy(e);
+    return true;
+  };
+  // (the device copies may still be read by the kernels of the call before this one on `stream`: the kept block
+  // is handed from call to call only after a wait for `stream`, so nothing is in flight there)
+  for (size_t i = 0; i < in.size(); ++i)
+    if (!sliced[i]) {
+      const size_t bytes = row_bytes(in[i]) * (in[i].shape.empty() ? 1 : in[i].shape[0]);
+      if (ihip::Err e = ihip::upload_pipelined(in[i].data, inputs[i].data, bytes, up); !e.empty()) return fail(e);
+    }
+  for (size_t s = 0; s < slices; ++s) {
+    const size_t r0 = std::min(rows, s * each), r1 = std::min(rows, r0 + each);
+    if (r0 == r1) break;
+    std::vector<ihipc::DeviceTensor> in_s(in), out_s(out);
+    for (size_t i = 0; i < in.size(); ++i) {
+      if (!sliced[i]) continue;
+      const size_t at = r0 * row_bytes(in[i]), bytes = (r1 - r0) * row_bytes(in[i]);
+      in_s[i].data = static_cast<char*>(in[i].data) + at;
+      in_s[i].shape[0] = r1 - r0;
+      if (ihip::Err e = ihip::upload_pipelined(in_s[i].data, static_cast<const char*>(static_cast<const void*>(inputs[i].data)) + at, bytes, up);
+          !e.empty())
+        return fail(e);
+    }
+    for (size_t o = 0; o < out.size(); ++o) {
+      out_s[o].data = static_cast<char*>(out[o].data) + r0 * row_bytes(out[o]);
+      out_s[o].shape[0] = r1 - r0;
+    }
+    if (hipEventRecord(landed[s], up) != hipSuccess || hipStreamWaitEvent(stream, landed[s], 0) != hipSuccess)
+      return fail("hipStreamWaitEvent failed");
+    std::string e;
+    try {
+      e = ihipc::execute(p, in_s, out_s, stream);
+    } catch (const std::exception& ex) {
+      e = ex.what();
+    }
+    if (!e.empty()) return fail(e);
+  }
+  // (the events may be destroyed once recorded and waited for: the waits stay in the stream)
+  for (hipEvent_t e : landed) (void)hipEventDestroy(e);
+  ihipc::append_to_report(p, "host: operands in " + std::to_string((rows + each - 1) / each) + " slices of " + std::to_string(each) +
+                                 " rows, the kernels above are those of the last slice\n");
+  return true;
+}
+
 // Host entry: upload f32 operands, run, download, wait.  Mirrors the
 // blocking behaviour of the reference's exec (core/src/lib.rs:200-225).
 std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_count, const std::vector<float*>& out_ptrs) {
@@ -211,12 +317,7 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
       cleanup();
       return e;
     }
-    if (mirror) {
-      if (n) std::memcpy(mirror + (static_cast<char*>(t.data) - block_base), inputs[i].data, n * 4);
-    } else if (ihip::Err e = ihip::upload_pipelined(t.data, inputs[i].data, n * 4, stream); !e.empty()) {
-      cleanup();
-      return e;
-    }
+    if (mirror && n) std::memcpy(mirror + (static_cast<char*>(t.data) - block_base), inputs[i].data, n * 4);
     in.push_back(std::move(t));
   }
   const size_t input_bytes = carve ? (size_t)(carve - block_base) : 0;  // (the inputs lie first in the block)
@@ -238,10 +339,18 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
     out.push_back(std::move(t));
   }
   std::string err;
-  try {
-    err = ihipc::execute(p, in, out, stream);
-  } catch (const std::exception& e) {
-    err = e.what();
+  // large operands: in slices when the program allows it, else one after the other and then the program
+  if (mirror || !run_host_in_slices(p, inputs, in, out, stream, &err)) {
+    for (size_t i = 0; !mirror && err.empty() && i < input_count; ++i) {
+      size_t n = 1;
+      for (size_t d : in_shapes[i]) n *= d;
+      err = ihip::upload_pipelined(in[i].data, inputs[i].data, n * 4, stream);
+    }
+    try {
+      if (err.empty()) err = ihipc::execute(p, in, out, stream);
+    } catch (const std::exception& e) {
+      err = e.what();
+    }
   }
   for (size_t o = 0; err.empty() && o < out.size(); ++o) {
     size_t n = 1;
@@ -539,6 +648,21 @@ int i_hip_program_clock_probe(i_program* program, void* ticks) {
   if (!program) return fail("null program");
   const std::string err = ihipc::set_clock_probe(*program->inner, ticks);
   return err.empty() ? 0 : fail(err);
+}
+
+int i_hip_program_row_slices(const i_program* program, unsigned char* sliced, size_t capacity) {
+  if (!program) {
+    icore::set_error("null program");
+    return -1;
+  }
+  std::vector<char> flags;
+  if (!ihipc::row_sliceable(*program->inner, &flags)) return 0;
+  if (sliced && capacity < flags.size()) {
+    icore::set_error("the program has " + std::to_string(flags.size()) + " inputs");
+    return -1;
+  }
+  for (size_t i = 0; sliced && i < flags.size(); ++i) sliced[i] = flags[i] ? 1 : 0;
+  return (int)flags.size();
 }
 
 char* i_hip_program_report(const i_program* program) {

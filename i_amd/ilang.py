@@ -323,6 +323,16 @@ class Component:
         nat.check(core.i_hip_program_clock_probe(self._compile(), None if ticks is None else ticks.data_ptr()))
         return self
 
+    def row_slices(self):
+        """Whether the program may be run on its outputs' first index slice by slice (``i_hip_program_row_slices``):
+        None if it has to run whole, else one flag per input, True for the inputs that are cut along their first
+        dimension with the outputs and False for those that every slice needs whole."""
+        flags = (ctypes.c_ubyte * 256)()
+        n = core.i_hip_program_row_slices(self._compile(), flags, 256)
+        if n < 0:
+            nat.check(n)
+        return None if n == 0 else [bool(flags[k]) for k in range(n)]
+
     def report(self):
         """The kernels the last run dispatched, one line per kernel of the plan (``i_hip_program_report``)."""
         text = nat.check_ptr(core.i_hip_program_report(self._compile()))

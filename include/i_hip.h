@@ -189,6 +189,21 @@ size_t i_hip_release_cached_memory(void);
 char* i_hip_program_report(const i_program* program);
 
 /*
+ * Whether the program only ever maps over the first index of its outputs: that index is the first dimension of some
+ * of the inputs and no other dimension of any, no expression reduces over it, and none uses it under two names.
+ * Rows r0 .. r1 of every output are then what the program computes from rows r0 .. r1 of those inputs and all of
+ * the others, so the program may be run slice by slice.  Returns the number of the program's inputs (at least 1)
+ * and sets sliced[i] to 1 for the inputs that are cut with the outputs and to 0 for those every slice needs whole
+ * (sliced may be NULL; else `capacity` entries, at least as many as the program has inputs), 0 if the program has
+ * to run whole, -1 + i_error on a bad argument.  i_exec and i_exec_into use it themselves: calls
+ * that move 64 MiB and more in such rows go up, run and come down in up to 8 slices, the kernels of one slice under
+ * the transfer of the next (i_hip_program_report then says so).  A slice is computed by the kernels the launchers
+ * pick for its shape, which may add up sums in another order than the whole would (within the parity bars).  No
+ * counterpart in the reference, which runs on the host.
+ */
+int i_hip_program_row_slices(const i_program* program, unsigned char* sliced, size_t capacity);
+
+/*
  * mm_t,  c[bh,m,n] = sum_k a[bh,m,k] * b[bh,n,k]  with bf16 a, b and f32 c:
  * the fused kernel for  i("ik*jk~ijk") >> i("+ijk~ij ... k0")  (README.md:16;
  * same nest as annotated-flashattn.c:57-89).  Requires k % 8 == 0.

@@ -107,6 +107,32 @@ def test_exec_into_refuses_an_output_whose_stated_extents_are_not_what_the_progr
         prog.into(np.zeros((2,), np.float32), x)
 
 
+def test_which_programs_may_run_on_their_rows_in_slices():
+    """i_hip_program_row_slices: the first index of the outputs has to be one that the program only maps over."""
+    mm_t = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    assert mm_t.row_slices() == [True, False]                      # rows of A and of C; all of B for every slice
+    assert (i("ik*kj~ijk") >> i("+ijk~ij")).row_slices() == [True, False]
+    softmax = (I & i(">ij~i")) >> i("ij-i~ij") >> i("^ij~ij") >> (I & i("+ij~i")) >> i("ij/i~ij")
+    assert softmax.row_slices() == [True]                          # the reductions are over j
+    s = "i:16,j:16"
+    attn = (i(f"bhik*bhjk~bhijk | {s} | bhjii'j'k") >> i(f"+bhijk~bhij | {s} | bhjii'j'k0") >> i(f"bhij*.~bhij | {s} | bhji0i'j'")
+            >> (I & i(f">bhij~bhi | {s} | bhji0i'j'")) >> i(f"bhij-bhi~bhij | {s} | bhji01i'j'") >> i(f"^bhij~bhij | {s} | bhji0i'j'")
+            >> (I & i(f"+bhij~bhi | {s} | bhji0i'j'")) >> i(f"bhij/bhi~bhij | {s} | bhji01i'j'")
+            >> i(f"bhij*bhjk~bhikj | {s} | bhji0i'kj'") >> i(f"+bhikj~bhik | {s} | bhjii'kj'0"))
+    assert attn.row_slices() == [True, True, False, True]          # Q, K, V by batch; the scale whole
+    assert i("+ij~i").row_slices() == [True] and i("^ij~ij").row_slices() == [True]
+    # summed over, second dimension of the input, or under two names in one expression: whole
+    assert i("+ij~j").row_slices() is None and i("+ij~.").row_slices() is None and i("ij~ji").row_slices() is None
+    assert ((I & i("+ij~j||ij")) >> i("ij/j~ij||1ij")).row_slices() is None
+    gram = (I & I) >> i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    assert gram.row_slices() is None
+    # arguments
+    flags = (ctypes.c_ubyte * 1)()
+    assert nat.core.i_hip_program_row_slices(None, flags, 1) == -1 and "null program" in nat.last_error()
+    assert nat.core.i_hip_program_row_slices(mm_t._compile(), flags, 1) == -1 and "2 inputs" in nat.last_error()
+    assert nat.core.i_hip_program_row_slices(mm_t._compile(), None, 0) == 2
+
+
 def test_identity_program_is_rejected_like_the_reference():
     # a program output that is a program input has no kernel to produce it
     with pytest.raises(RuntimeError) as err:

@@ -241,6 +241,55 @@ def test_config3_mm_t_bf16_device(torch):
     close(c[:, cols].cpu().numpy(), oracle.mm_t(a, b[cols]), RTOL_BF16)
 
 
+def test_large_host_calls_run_in_slices(torch):
+    """The reference's own entry point (host f32 arrays) with operands of tens of MiB: a program that only maps over
+    the first index of its outputs runs slice by slice, the rows of one slice on the link while the kernels of the
+    slice before run.  Row softmax, attention (all of Q, K, V and O cut along the batch) and mm_t (A and C in
+    slices, B whole) against the device entry on the same operands; programs that sum over that index, or use it
+    under two names, stay whole and stay right."""
+    g = np.random.default_rng(7)
+
+    def on_device(comp, *ins):
+        return comp.exec_torch(*(torch.from_numpy(np.asarray(x)).cuda() for x in ins)).cpu().numpy()
+
+    x = g.standard_normal((16384, 1024), dtype=np.float32)                      # 64 MiB in, 64 MiB out
+    sm = softmax_rowstaged()
+    y = np.empty_like(x)
+    sm.into(y, x)
+    assert "host: operands in 4 slices of 4096 rows" in sm.report(), sm.report()
+    assert np.array_equal(y, on_device(sm, x))                                   # rows do not know how many there are
+    q, k, v = (g.standard_normal((4, 8, 1024, 128), dtype=np.float32) for _ in range(3))  # 16 MiB each
+    attn = flash("i:128,j:32", prefix="bh", scaled=True)
+    scale = np.float32(128 ** -0.5)
+    o = np.empty_like(q)
+    attn.into(o, q, k, scale, v)
+    assert "host: operands in 2 slices of 2 rows" in attn.report(), attn.report()
+    close(o, on_device(attn, q, k, scale, v), 1e-6)
+    a = g.uniform(-1, 1, (4100, 2048)).astype(np.float32)                        # 32 MiB, in slices
+    b = g.uniform(-1, 1, (4096, 2048)).astype(np.float32)                        # 32 MiB, whole
+    mm = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    c = np.empty((4100, 4096), np.float32)                                       # 64 MiB, in slices
+    mm.into(c, a, b)
+    assert "host: operands in 3 slices of 1367 rows" in mm.report(), mm.report()
+    close(c, on_device(mm, a, b), 1e-5)  # (a slice may take another kernel than the whole: sums in another order)
+    rows = np.r_[0:4, 1365:1369, 4096:4100]
+    close(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64).T, RTOL_F32)
+    # the first index summed over: whole
+    xs = np.abs(x[:, :1024]) + 0.1
+    colnorm = (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij")
+    yn = np.empty_like(xs)
+    colnorm.into(yn, xs)
+    assert "host:" not in colnorm.report()
+    close(yn, xs / xs.sum(0, dtype=np.float64), RTOL_F32)
+    # the first index under two names in one expression: one input as both operands of a product
+    gram = (I & I) >> i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
+    z = g.uniform(-1, 1, (4096, 1024)).astype(np.float32)
+    got = np.empty((4096, 4096), np.float32)                                     # 64 MiB out
+    gram.into(got, z)
+    assert "host:" not in gram.report()
+    close(got[:16], z[:16].astype(np.float64) @ z.astype(np.float64).T, RTOL_F32)
+
+
 def test_bf16_operands_that_start_off_a_16_byte_boundary(torch):
     """Every bf16 kernel moves 16 bytes per lane (the direct ones straight from global memory into LDS).  Operands
     that are views starting one element (2 bytes) into their allocation are copied into aligned temporaries by the
