@@ -7,8 +7,10 @@
 #include <algorithm>
 #include <map>
 #include <memory>
+#include <condition_variable>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../../include/i_hip.h"
@@ -135,34 +137,38 @@ size_t staging_limit() {
   return limit;
 }
 
-// The stream that the operands of a call in slices are uploaded on (one per device, created on first use and kept;
-// not synchronised with the default stream, on which the kernels run); nullptr when there is none to be had.
-hipStream_t upload_stream_of_current_device() {
+// The two streams beside the call's own that a call in slices uses: `which` 0 carries the uploads, 1 the downloads
+// (one each per device, created on first use and kept; not synchronised with the default stream, on which the
+// kernels run); nullptr when there is none to be had.
+hipStream_t side_stream_of_current_device(int which) {
   static std::mutex mu;
   static std::map<int, hipStream_t>* streams = new std::map<int, hipStream_t>();
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(mu);
-  auto it = streams->find(device);
+  auto it = streams->find(2 * device + which);
   if (it != streams->end()) return it->second;
   hipStream_t made = nullptr;
   if (hipStreamCreateWithFlags(&made, hipStreamNonBlocking) != hipSuccess) {
     (void)hipGetLastError();
     made = nullptr;
   }
-  (*streams)[device] = made;
+  (*streams)[2 * device + which] = made;
   return made;
 }
 
 // A call in slices (large operands of a program that only maps over its leading index, ihipc::row_sliceable): the
 // inputs that every slice needs whole are uploaded first; then, slice after slice, the rows of the other inputs go
 // up on the upload stream and the program is enqueued on `stream` behind them for just those rows, so the kernels
-// of one slice run while the next is on the link; the outputs come down when the last slice has run.  Returns
-// false when the call is not taken in slices (nothing has been enqueued then).
+// of one slice run while the next is on the link; a second host thread brings the rows of the outputs down on the
+// download stream as soon as their slice has run, beside the uploads of the slices after it (the link carries both
+// directions at once).  Returns false when the call is not taken in slices (nothing has been enqueued then); true
+// with the outputs in host memory, or with *err set.
 constexpr size_t kSlicedCallBytes = size_t(64) << 20;  // what crosses the link in slices, at least
 constexpr size_t kSliceBytes = size_t(32) << 20;       // ... and per slice, about
 bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::vector<ihipc::DeviceTensor>& in,
-                        const std::vector<ihipc::DeviceTensor>& out, hipStream_t stream, std::string* err) {
+                        const std::vector<ihipc::DeviceTensor>& out, const std::vector<float*>& out_ptrs, hipStream_t stream,
+                        std::string* err) {
   std::vector<char> sliced;
   if (!ihipc::row_sliceable(p, &sliced) || sliced.size() != in.size() || out.empty() || out[0].shape.empty()) return false;
   const size_t rows = out[0].shape[0];
@@ -176,28 +182,81 @@ bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::ve
     if (sliced[i] && (in[i].shape.empty() || in[i].shape[0] != rows)) return false;
     (sliced[i] ? moving : whole) += row_bytes(in[i]) * (in[i].shape.empty() ? 1 : in[i].shape[0]);
   }
-  for (const ihipc::DeviceTensor& t : out) {
-    if (t.shape.empty() || t.shape[0] != rows) return false;
-    moving += row_bytes(t) * rows;
+  for (size_t o = 0; o < out.size(); ++o) {
+    if (out[o].shape.empty() || out[o].shape[0] != rows || !out_ptrs[o]) return false;
+    moving += row_bytes(out[o]) * rows;
   }
   if (rows < 2 || moving < kSlicedCallBytes || moving < whole) return false;
-  const size_t slices = std::min<size_t>(std::min<size_t>(8, rows), std::max<size_t>(2, moving / kSliceBytes));
-  const size_t each = (rows + slices - 1) / slices;
-  hipStream_t up = upload_stream_of_current_device();
-  if (!up) return false;
-  std::vector<hipEvent_t> landed(slices, nullptr);
-  for (hipEvent_t& e : landed)
-    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+  const size_t wanted = std::min<size_t>(std::min<size_t>(8, rows), std::max<size_t>(2, moving / kSliceBytes));
+  const size_t each = (rows + wanted - 1) / wanted, slices = (rows + each - 1) / each;
+  hipStream_t up = side_stream_of_current_device(0), down = side_stream_of_current_device(1);
+  int device = 0;
+  if (!up || !down || hipGetDevice(&device) != hipSuccess) return false;
+  std::vector<hipEvent_t> landed(slices, nullptr), done(slices, nullptr);
+  auto destroy_events = [&] {
+    for (hipEvent_t e : landed)
+      if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : done)
+      if (e) (void)hipEventDestroy(e);
+  };
+  for (size_t s = 0; s < slices; ++s)
+    if (hipEventCreateWithFlags(&landed[s], hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&done[s], hipEventDisableTiming) != hipSuccess) {
       (void)hipGetLastError();
-      for (hipEvent_t made : landed)
-        if (made) (void)hipEventDestroy(made);
+      destroy_events();
       return false;
     }
-  auto fail = [&](const std::string& what) {
-    *err = what;
-    (void)hipStreamSynchronize(up);
-    (void)ihip::sync(stream);
-    for (hipEvent_t e : landed) (void)hipEventDestroy(e);
+  // the downloads: slice s once the main thread says that it has been enqueued (or that nothing more will be)
+  std::mutex mu;
+  std::condition_variable changed;
+  size_t enqueued = 0;
+  bool stop = false;
+  std::string down_err;
+  auto bring_down = [&] {
+    (void)hipSetDevice(device);
+    for (size_t s = 0; s < slices; ++s) {
+      {
+        std::unique_lock<std::mutex> lock(mu);
+        changed.wait(lock, [&] { return enqueued > s || stop; });
+        if (enqueued <= s) return;
+      }
+      if (hipStreamWaitEvent(down, done[s], 0) != hipSuccess) {
+        down_err = "hipStreamWaitEvent failed";
+        return;
+      }
+      const size_t r0 = s * each, r1 = std::min(rows, r0 + each);
+      for (size_t o = 0; o < out.size(); ++o) {
+        const size_t at = r0 * row_bytes(out[o]), bytes = (r1 - r0) * row_bytes(out[o]);
+        if (ihip::Err e = ihip::download_pipelined(reinterpret_cast<char*>(out_ptrs[o]) + at, static_cast<const char*>(out[o].data) + at, bytes, down);
+            !e.empty()) {
+          down_err = e;
+          return;
+        }
+      }
+    }
+  };
+  std::thread helper;
+  try {
+    helper = std::thread(bring_down);
+  } catch (const std::exception&) {
+    destroy_events();
+    return false;
+  }
+  auto finish = [&](const std::string& what, bool all_enqueued) {
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      stop = !all_enqueued;
+      if (all_enqueued) enqueued = slices;
+    }
+    changed.notify_all();
+    helper.join();
+    *err = !what.empty() ? what : down_err;
+    if (!err->empty()) {
+      (void)hipStreamSynchronize(up);
+      (void)hipStreamSynchronize(down);
+      (void)ihip::sync(stream);
+    }
+    destroy_events();
     return true;
   };
   // (the device copies may still be read by the kernels of the call before this one on `stream`: the kept block
@@ -205,11 +264,10 @@ bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::ve
   for (size_t i = 0; i < in.size(); ++i)
     if (!sliced[i]) {
       const size_t bytes = row_bytes(in[i]) * (in[i].shape.empty() ? 1 : in[i].shape[0]);
-      if (ihip::Err e = ihip::upload_pipelined(in[i].data, inputs[i].data, bytes, up); !e.empty()) return fail(e);
+      if (ihip::Err e = ihip::upload_pipelined(in[i].data, inputs[i].data, bytes, up); !e.empty()) return finish(e, false);
     }
   for (size_t s = 0; s < slices; ++s) {
-    const size_t r0 = std::min(rows, s * each), r1 = std::min(rows, r0 + each);
-    if (r0 == r1) break;
+    const size_t r0 = s * each, r1 = std::min(rows, r0 + each);
     std::vector<ihipc::DeviceTensor> in_s(in), out_s(out);
     for (size_t i = 0; i < in.size(); ++i) {
       if (!sliced[i]) continue;
@@ -218,27 +276,31 @@ bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::ve
       in_s[i].shape[0] = r1 - r0;
       if (ihip::Err e = ihip::upload_pipelined(in_s[i].data, static_cast<const char*>(static_cast<const void*>(inputs[i].data)) + at, bytes, up);
           !e.empty())
-        return fail(e);
+        return finish(e, false);
     }
     for (size_t o = 0; o < out.size(); ++o) {
       out_s[o].data = static_cast<char*>(out[o].data) + r0 * row_bytes(out[o]);
       out_s[o].shape[0] = r1 - r0;
     }
     if (hipEventRecord(landed[s], up) != hipSuccess || hipStreamWaitEvent(stream, landed[s], 0) != hipSuccess)
-      return fail("hipStreamWaitEvent failed");
+      return finish("hipStreamWaitEvent failed", false);
     std::string e;
     try {
       e = ihipc::execute(p, in_s, out_s, stream);
     } catch (const std::exception& ex) {
       e = ex.what();
     }
-    if (!e.empty()) return fail(e);
+    if (e.empty() && hipEventRecord(done[s], stream) != hipSuccess) e = "hipEventRecord failed";
+    if (!e.empty()) return finish(e, false);
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      enqueued = s + 1;
+    }
+    changed.notify_all();
   }
-  // (the events may be destroyed once recorded and waited for: the waits stay in the stream)
-  for (hipEvent_t e : landed) (void)hipEventDestroy(e);
-  ihipc::append_to_report(p, "host: operands in " + std::to_string((rows + each - 1) / each) + " slices of " + std::to_string(each) +
+  ihipc::append_to_report(p, "host: operands in " + std::to_string(slices) + " slices of " + std::to_string(each) +
                                  " rows, the kernels above are those of the last slice\n");
-  return true;
+  return finish({}, true);
 }
 
 // Host entry: upload f32 operands, run, download, wait.  Mirrors the
@@ -340,7 +402,8 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
   }
   std::string err;
   // large operands: in slices when the program allows it, else one after the other and then the program
-  if (mirror || !run_host_in_slices(p, inputs, in, out, stream, &err)) {
+  const bool in_slices = !mirror && run_host_in_slices(p, inputs, in, out, out_ptrs, stream, &err);  // (outputs included)
+  if (!in_slices) {
     for (size_t i = 0; !mirror && err.empty() && i < input_count; ++i) {
       size_t n = 1;
       for (size_t d : in_shapes[i]) n *= d;
@@ -352,7 +415,7 @@ std::string run_host(ihipc::Program& p, const i_tensor* inputs, size_t input_cou
       err = e.what();
     }
   }
-  for (size_t o = 0; err.empty() && o < out.size(); ++o) {
+  for (size_t o = 0; !in_slices && err.empty() && o < out.size(); ++o) {
     size_t n = 1;
     for (size_t d : out_shapes[o]) n *= d;
     if (n && !out_ptrs[o]) err = "output " + std::to_string(o) + " has no data";

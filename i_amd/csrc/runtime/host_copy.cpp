@@ -80,7 +80,7 @@ class CopyCrew {
   size_t bytes_ = 0, each_ = 0, next_ = 0, slices_ = 0, pending_ = 0, generation_ = 0;
 };
 
-// The ring of page-locked chunks of one device: four chunks of 8 MiB (small enough that the first chunk's fill and
+// A ring of page-locked chunks of one device (one for each direction): four chunks of 8 MiB (small enough that the first chunk's fill and
 // the last chunk's transfer, which nothing overlaps, are a small part of a 64 MiB operand), allocated by the first
 // large host call on that device and kept until the process ends.  One transfer uses the ring at a time; a chunk
 // whose last transfer may still be in flight (in_flight) is awaited before it is touched again, not before: the
@@ -109,12 +109,14 @@ RingTable& ring_table() {
   static RingTable* table = new RingTable();
   return *table;
 }
-Ring* ring_of_current_device() {
+// (a ring for uploads and one for downloads per device, so that a download on one thread can run beside an upload
+// on another: the link carries both directions at once)
+Ring* ring_of_current_device(bool download) {
   RingTable& t = ring_table();
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(t.mu);
-  auto& ring = t.rings[device];
+  auto& ring = t.rings[2 * device + (download ? 1 : 0)];
   if (!ring) ring = std::make_unique<Ring>();
   return ring.get();
 }
@@ -157,7 +159,7 @@ size_t release_copy_chunks() {
 }
 
 Err upload_pipelined(void* dst, const void* src, size_t bytes, hipStream_t stream) {
-  Ring* ring = bytes >= kPipelinedCopyBytes ? ring_of_current_device() : nullptr;
+  Ring* ring = bytes >= kPipelinedCopyBytes ? ring_of_current_device(false) : nullptr;
   std::unique_lock<std::mutex> lock;
   if (ring) lock = std::unique_lock<std::mutex>(ring->busy, std::try_to_lock);
   if (!ring || !lock.owns_lock() || !prepare(ring)) return h2d(dst, src, bytes, stream);
@@ -176,7 +178,7 @@ Err upload_pipelined(void* dst, const void* src, size_t bytes, hipStream_t strea
 }
 
 Err download_pipelined(void* dst, const void* src, size_t bytes, hipStream_t stream) {
-  Ring* ring = bytes >= kPipelinedCopyBytes ? ring_of_current_device() : nullptr;
+  Ring* ring = bytes >= kPipelinedCopyBytes ? ring_of_current_device(true) : nullptr;
   std::unique_lock<std::mutex> lock;
   if (ring) lock = std::unique_lock<std::mutex>(ring->busy, std::try_to_lock);
   if (!ring || !lock.owns_lock() || !prepare(ring)) {
@@ -188,7 +190,7 @@ Err download_pipelined(void* dst, const void* src, size_t bytes, hipStream_t str
   auto request = [&](size_t c) -> Err {
     const size_t at = c * kChunkBytes, len = std::min(kChunkBytes, bytes - at);
     const int slot = (int)((first + c) % kChunks);
-    if (Err e = ring->settle(slot); !e.empty()) return e;  // (an upload that may still be reading the chunk)
+    if (Err e = ring->settle(slot); !e.empty()) return e;
     if (Err e = check(hipMemcpyAsync(ring->chunk[slot], static_cast<const char*>(src) + at, len, hipMemcpyDeviceToHost, stream), "hipMemcpy D2H");
         !e.empty())
       return e;

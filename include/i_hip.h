@@ -173,8 +173,8 @@ int i_hip_shader_clock_probe(void* ticks, unsigned microseconds, void* stream);
  * Memory that the library keeps from call to call, so that a call allocates nothing after the first of its kind: per
  * (device, stream), for the 16 pairs used most recently, a block for temporaries (at most ILANG_HIP_ARENA_MB, default
  * 256 MiB each); per device a block for the device copies of host operands (at most ILANG_HIP_STAGING_MB, default
- * 1 GiB) with an 8 MiB page-locked mirror, four page-locked chunks of 8 MiB for large host operands, up to 1 GiB of
- * freed temporaries in the library's own memory pool, and the fixed workspace of i_exec_into_device_noalloc
+ * 1 GiB) with an 8 MiB page-locked mirror, two rings of four page-locked chunks of 8 MiB for large host operands
+ * (one ring per direction), up to 1 GiB of freed temporaries in the library's own memory pool, and the fixed workspace of i_exec_into_device_noalloc
  * (I_HIP_STATIC_WORKSPACE_BYTES, part of the loaded library).  This call frees all of it except the last, as far as
  * no call is using it at the moment, and returns the bytes released; the next calls allocate again.  No counterpart
  * in the reference, whose generated exec mallocs and frees on every call.

@@ -111,6 +111,7 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKin
 }
 hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 // (no page-locked memory here, so the library never gets as far as the events of its chunked host copies)
+hipError_t hipSetDevice(int) { return hipSuccess; }
 hipError_t hipStreamCreateWithFlags(hipStream_t*, unsigned) { return hipErrorNotSupported; }
 hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) { return hipErrorNotSupported; }
 hipError_t hipEventCreateWithFlags(hipEvent_t*, unsigned) { return hipErrorNotSupported; }
