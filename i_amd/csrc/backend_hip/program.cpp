@@ -664,7 +664,9 @@ size_t generated_parts(const ihip::KernelOptions& knobs, const GridForm& grid, b
     if (total * 2 > target) return 1;
     parts = std::min<size_t>(target / total, reduced / least);
   }
-  parts = std::min<size_t>(std::min<size_t>(parts, 4096), std::max<size_t>(reduced, 1));
+  // (at most 4096 parts; 2048 of wavefronts when left to this rule: the pass over the parts of a sum to one element
+  // is one wavefront's work and grows with their number, 4096^2 to one element 29.7 us in 4096 parts, 23.8 in 2048)
+  parts = std::min<size_t>(std::min<size_t>(parts, wave && knobs.generated_parts <= 1 ? 2048 : 4096), std::max<size_t>(reduced, 1));
   if (parts >= 256) parts = parts / 32 * 32;
   else if (parts >= 16) parts = parts / 8 * 8;
   return parts < 2 ? 1 : parts;
