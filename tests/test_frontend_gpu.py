@@ -258,6 +258,8 @@ def test_large_host_calls_run_in_slices(torch):
     sm.into(y, x)
     assert "host: operands in 4 slices of 4096 rows" in sm.report(), sm.report()
     assert np.array_equal(y, on_device(sm, x))                                   # rows do not know how many there are
+    picked = np.r_[0:64, 4090:4102, 16320:16384]                                 # (rows on both sides of a slice's edge)
+    close(y[picked], oracle.row_softmax(x[picked]), RTOL_F32)
     q, k, v = (g.standard_normal((4, 8, 1024, 128), dtype=np.float32) for _ in range(3))  # 16 MiB each
     attn = flash("i:128,j:32", prefix="bh", scaled=True)
     scale = np.float32(128 ** -0.5)
@@ -265,6 +267,7 @@ def test_large_host_calls_run_in_slices(torch):
     attn.into(o, q, k, scale, v)
     assert "host: operands in 2 slices of 2 rows" in attn.report(), attn.report()
     close(o, on_device(attn, q, k, scale, v), 1e-6)
+    close(o[1:3, 7:8, 1000:1024], oracle.attention_tiled(q[1:3, 7:8, 1000:1024], k[1:3, 7:8], v[1:3, 7:8], scale), RTOL_F32)
     a = g.uniform(-1, 1, (4100, 2048)).astype(np.float32)                        # 32 MiB, in slices
     b = g.uniform(-1, 1, (4096, 2048)).astype(np.float32)                        # 32 MiB, whole
     mm = i("ik*jk~ijk | i:16,j:16 | jii'j'k") >> i("+ijk~ij | i:16,j:16 | jii'j'k0")
@@ -274,6 +277,7 @@ def test_large_host_calls_run_in_slices(torch):
     close(c, on_device(mm, a, b), 1e-5)  # (a slice may take another kernel than the whole: sums in another order)
     rows = np.r_[0:4, 1365:1369, 4096:4100]
     close(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64).T, RTOL_F32)
+    close(c[rows], oracle.mm_t(a[rows], b), RTOL_F32)
     # the first index summed over: whole
     xs = np.abs(x[:, :1024]) + 0.1
     colnorm = (I & i("+ij~j||ij")) >> i("ij/j~ij||1ij")
