@@ -212,7 +212,7 @@ bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::ve
   size_t enqueued = 0;
   bool stop = false;
   std::string down_err;
-  auto bring_down = [&] {
+  auto bring_down_slices = [&] {
     (void)hipSetDevice(device);
     for (size_t s = 0; s < slices; ++s) {
       {
@@ -233,6 +233,13 @@ bool run_host_in_slices(ihipc::Program& p, const i_tensor* inputs, const std::ve
           return;
         }
       }
+    }
+  };
+  auto bring_down = [&] {
+    try {
+      bring_down_slices();
+    } catch (const std::exception& e) {  // (nothing may leave a thread's function)
+      down_err = e.what();
     }
   };
   std::thread helper;
